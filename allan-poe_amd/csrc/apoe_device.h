@@ -1,0 +1,268 @@
+// Device-side building blocks shared by every kernel: the packed corpus record,
+// wave64 reductions and sorts, the LDS term hash that a pivot's sparse terms are
+// scattered into, and the wave-cooperative hybrid inner product.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace apoe {
+
+constexpr int WAVE = 64;
+constexpr uint32_t EMPTY = 0xFFFFFFFFu;
+constexpr uint32_t FLAG = 0x80000000u;     // "explored"/"sampled" bit on a doc id
+constexpr uint32_t BM25_BIT = 0x80000000u; // unified term key: bit31 set = BM25 term
+constexpr float INF_DIS = 1000000.0f;
+constexpr int DIM = 1024;
+constexpr int DENSE_BYTES = DIM * 4;
+constexpr int NV = DIM / (4 * WAVE); // float4 loads per lane for one dense row
+
+// Descriptor of one document: record offset (16-byte units) and the two pair counts.
+constexpr int DESC_OFF_BITS = 36;
+constexpr int DESC_NNZ_BITS = 14;
+constexpr uint32_t DESC_NNZ_MAX = (1u << DESC_NNZ_BITS) - 1;
+constexpr uint64_t DESC_OFF_MASK = (1ull << DESC_OFF_BITS) - 1;
+
+__host__ __device__ inline uint64_t make_desc(uint64_t off16, uint32_t nnz_s, uint32_t nnz_b) {
+    return off16 | ((uint64_t)nnz_s << DESC_OFF_BITS) | ((uint64_t)nnz_b << (DESC_OFF_BITS + DESC_NNZ_BITS));
+}
+__host__ __device__ inline uint64_t desc_off(uint64_t d) { return d & DESC_OFF_MASK; }
+__host__ __device__ inline uint32_t desc_nnz_s(uint64_t d) { return (uint32_t)(d >> DESC_OFF_BITS) & DESC_NNZ_MAX; }
+__host__ __device__ inline uint32_t desc_nnz_b(uint64_t d) { return (uint32_t)(d >> (DESC_OFF_BITS + DESC_NNZ_BITS)) & DESC_NNZ_MAX; }
+
+// Record = [DIM floats][nnz_s x (term, value)][nnz_b x (term | BM25_BIT, value)], 16-byte aligned.
+struct CorpusView {
+    const uint64_t* desc;
+    const char* recs;
+    uint32_t n;
+};
+
+struct SetView { // a set kept in CSR form on the device (queries)
+    const float* dense;
+    const uint32_t* s_off;
+    const uint32_t* s_idx;
+    const float* s_val;
+    const uint32_t* b_off;
+    const uint32_t* b_idx;
+    const float* b_val;
+    uint32_t n;
+};
+
+#ifdef __HIPCC__
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// Total order on floats as unsigned integers (negative distances are common: 1 - IP).
+__device__ __forceinline__ uint32_t float_key(float f) {
+    uint32_t u = __float_as_uint(f);
+    return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+__device__ __forceinline__ uint64_t dist_id_key(float d, uint32_t id) {
+    return ((uint64_t)float_key(d) << 32) | id;
+}
+
+__device__ __forceinline__ uint64_t shfl_xor64(uint64_t v, int m) {
+    uint32_t lo = __shfl_xor((uint32_t)v, m, WAVE), hi = __shfl_xor((uint32_t)(v >> 32), m, WAVE);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// Bitonic sort of one 64-bit key per lane across the wave, ascending by lane.
+__device__ __forceinline__ uint64_t wave_sort64(uint64_t key) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int k = 2; k <= WAVE; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            uint64_t other = shfl_xor64(key, j);
+            bool up = (lane & k) == 0;       // ascending block
+            bool lower = (lane & j) == 0;    // this lane keeps the smaller in an ascending block
+            bool take_min = up == lower;
+            key = take_min ? (key < other ? key : other) : (key < other ? other : key);
+        }
+    }
+    return key;
+}
+// Same with a 32-bit payload that travels with the key.
+__device__ __forceinline__ void wave_sort64_payload(uint64_t& key, uint32_t& pay0, uint32_t& pay1) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int k = 2; k <= WAVE; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            uint64_t other = shfl_xor64(key, j);
+            uint32_t o0 = __shfl_xor(pay0, j, WAVE), o1 = __shfl_xor(pay1, j, WAVE);
+            bool up = (lane & k) == 0;
+            bool lower = (lane & j) == 0;
+            bool take_min = up == lower;
+            bool swap = take_min ? (other < key) : (key < other);
+            if (swap) { key = other; pay0 = o0; pay1 = o1; }
+        }
+    }
+}
+
+// ---- LDS term hash: (key, value-bits) slots, open addressing, linear probing ----
+
+__device__ __forceinline__ uint32_t term_hash(uint32_t key, uint32_t mask) {
+    return ((key * 2654435761u) >> 12) & mask;
+}
+
+__device__ __forceinline__ void term_table_clear(uint2* tab, uint32_t slots, int tid, int nthreads) {
+    for (uint32_t i = tid; i < slots; i += nthreads) tab[i] = make_uint2(EMPTY, 0u);
+}
+
+// Keys inserted into one table are distinct; the table has at least twice as many slots as keys.
+__device__ __forceinline__ void term_table_insert(uint2* tab, uint32_t mask, uint32_t key, float val) {
+    uint32_t h = term_hash(key, mask);
+    while (true) {
+        uint32_t old = atomicCAS(&tab[h].x, EMPTY, key);
+        if (old == EMPTY || old == key) { tab[h].y = __float_as_uint(val); return; }
+        h = (h + 1) & mask;
+    }
+}
+
+// Returns true and adds value*stored on a hit.
+__device__ __forceinline__ bool term_table_probe(const uint2* tab, uint32_t mask, uint32_t key, float val, float& acc) {
+    uint32_t h = term_hash(key, mask);
+    while (true) {
+        uint2 e = tab[h];
+        if (e.x == key) { acc = fmaf(val, __uint_as_float(e.y), acc); return true; }
+        if (e.x == EMPTY) return false;
+        h = (h + 1) & mask;
+    }
+}
+
+// ---- pivot: the vector every candidate is compared with ----
+// Dense part lives in registers (lane l owns float4 number l + 64*i of the row),
+// sparse part lives in the LDS term table.
+struct PivotDense {
+    float4 v[NV];
+};
+
+__device__ __forceinline__ void pivot_dense_load(PivotDense& p, const float* row, float scale) {
+    const float4* r = reinterpret_cast<const float4*>(row);
+    const int lane = lane_id();
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        float4 x = r[lane + WAVE * i];
+        p.v[i] = make_float4(x.x * scale, x.y * scale, x.z * scale, x.w * scale);
+    }
+}
+
+// Insert the sparse part of a packed document record (all pairs, both paths).
+__device__ __forceinline__ void pivot_terms_from_record(uint2* tab, uint32_t mask, const char* rec, uint32_t nnz, int tid, int nthreads) {
+    const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
+    for (uint32_t j = tid; j < nnz; j += nthreads) {
+        uint2 kv = sp[j];
+        term_table_insert(tab, mask, kv.x, __uint_as_float(kv.y));
+    }
+}
+
+// Insert the sparse part of CSR query q, values multiplied by the path weights; a
+// path that is switched off inserts nothing.
+__device__ __forceinline__ void pivot_terms_from_query(uint2* tab, uint32_t mask, const SetView& Q, uint32_t q, float w_s, float w_b,
+                                                        bool use_s, bool use_b, int tid, int nthreads) {
+    if (use_s)
+        for (uint32_t j = Q.s_off[q] + tid; j < Q.s_off[q + 1]; j += nthreads) term_table_insert(tab, mask, Q.s_idx[j], Q.s_val[j] * w_s);
+    if (use_b)
+        for (uint32_t j = Q.b_off[q] + tid; j < Q.b_off[q + 1]; j += nthreads)
+            term_table_insert(tab, mask, Q.b_idx[j] | BM25_BIT, Q.b_val[j] * w_b);
+}
+
+struct EvalOut {
+    float ip;        // dense_mul * <dense> + <sparse pairs that hit the table>
+    uint32_t nnz_s;  // SPLADE pairs read
+    uint32_t nnz_b;  // BM25 pairs read
+};
+
+constexpr uint32_t PATH_DENSE = 1, PATH_SPARSE = 2, PATH_BM25 = 4;
+
+// Read-only probe of a plain id set (keys only).
+__device__ __forceinline__ bool id_set_contains(const uint32_t* set, uint32_t mask, uint32_t key) {
+    uint32_t h = term_hash(key, mask);
+    while (true) {
+        const uint32_t e = set[h];
+        if (e == key) return true;
+        if (e == EMPTY) return false;
+        h = (h + 1) & mask;
+    }
+}
+
+// One pair of the candidate against the pivot's table. With KW, a BM25 term of the
+// candidate that the pivot lacks but the centre node's term set holds raises `kw`
+// (the test of the build-time cal_bm25_dist, index.cu:128-153).
+template <bool KW>
+__device__ __forceinline__ void probe_pair(const uint2* tab, uint32_t mask, uint2 kv, float& acc, const uint32_t* uset, uint32_t umask, bool& kw) {
+    const bool hit = term_table_probe(tab, mask, kv.x, __uint_as_float(kv.y), acc);
+    if (KW) {
+        if (!hit && (kv.x & BM25_BIT) && id_set_contains(uset, umask, kv.x)) kw = true;
+    }
+}
+
+// Wave-cooperative hybrid inner product between the pivot and document `id`
+// (wave-uniform). All 64 lanes must call it; every lane gets the result.
+template <bool KW = false>
+__device__ __forceinline__ EvalOut eval_wave(const CorpusView& C, uint32_t id, const PivotDense& pv, const uint2* tab, uint32_t mask,
+                                             uint32_t paths, float dense_mul, const uint32_t* uset = nullptr, uint32_t umask = 0,
+                                             bool* kw_any = nullptr) {
+    const int lane = lane_id();
+    const uint64_t desc = C.desc[id];
+    const char* rec = C.recs + desc_off(desc) * 16;
+    const uint32_t ns = desc_nnz_s(desc), nb = desc_nnz_b(desc);
+    const uint32_t begin = (paths & PATH_SPARSE) ? 0u : ns;
+    const uint32_t end = (paths & PATH_BM25) ? ns + nb : ns;
+    const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
+    float4 x[NV];
+    if (paths & PATH_DENSE) {
+        const float4* r = reinterpret_cast<const float4*>(rec);
+#pragma unroll
+        for (int i = 0; i < NV; i++) x[i] = r[lane + WAVE * i];
+    }
+    // first three chunks of pairs are requested before anything is consumed
+    uint2 kv0 = make_uint2(0, 0), kv1 = kv0, kv2 = kv0;
+    const uint32_t j0 = begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
+    if (j0 < end) kv0 = sp[j0];
+    if (j1 < end) kv1 = sp[j1];
+    if (j2 < end) kv2 = sp[j2];
+    float acc = 0.f;
+    if (paths & PATH_DENSE) {
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            acc = fmaf(x[i].x, pv.v[i].x, acc);
+            acc = fmaf(x[i].y, pv.v[i].y, acc);
+            acc = fmaf(x[i].z, pv.v[i].z, acc);
+            acc = fmaf(x[i].w, pv.v[i].w, acc);
+        }
+        acc *= dense_mul;
+    }
+    bool kw = false;
+    if (j0 < end) probe_pair<KW>(tab, mask, kv0, acc, uset, umask, kw);
+    if (j1 < end) probe_pair<KW>(tab, mask, kv1, acc, uset, umask, kw);
+    if (j2 < end) probe_pair<KW>(tab, mask, kv2, acc, uset, umask, kw);
+    for (uint32_t j = j2 + WAVE; j < end; j += WAVE) probe_pair<KW>(tab, mask, sp[j], acc, uset, umask, kw);
+    EvalOut o;
+    o.ip = wave_sum(acc);
+    o.nnz_s = (paths & PATH_SPARSE) ? ns : 0u;
+    o.nnz_b = (paths & PATH_BM25) ? nb : 0u;
+    if (KW) *kw_any = __ballot(kw) != 0;
+    return o;
+}
+
+// splitmix64 finaliser (random initial neighbours).
+__host__ __device__ inline uint64_t mix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+#endif // __HIPCC__
+
+} // namespace apoe

@@ -1,0 +1,409 @@
+// NN-Descent on the GPU: random initial lists, the per-node expansion step, and the
+// final merge with the reverse lists. One workgroup (4 waves) per node.
+#include <algorithm>
+#include <memory>
+
+#include "apoe_internal.h"
+
+namespace apoe {
+
+constexpr int NND_THREADS = 256;
+constexpr int NND_PICKS = 4; // neighbours sampled per node and step (index.cu:157,171-181)
+
+__device__ __forceinline__ float key_dist(uint64_t key) {
+    uint32_t u = (uint32_t)(key >> 32);
+    u ^= (u >> 31) ? 0x80000000u : 0xFFFFFFFFu;
+    return __uint_as_float(u);
+}
+
+// ---- id set in LDS (dedupe of gathered candidates) ----
+__device__ __forceinline__ bool id_set_insert(uint32_t* set, uint32_t mask, uint32_t id) {
+    uint32_t h = term_hash(id, mask);
+    while (true) {
+        uint32_t old = atomicCAS(&set[h], EMPTY, id);
+        if (old == EMPTY) return true;
+        if (old == id) return false;
+        h = (h + 1) & mask;
+    }
+}
+
+__global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t n, uint32_t K, uint64_t seed, uint32_t* ids, float* dist, uint32_t* rev,
+                                                       float* rev_dist, uint32_t* rev_cnt) {
+    const uint64_t total = (uint64_t)n * K;
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (uint64_t)gridDim.x * blockDim.x) {
+        ids[t] = (uint32_t)(mix64(seed ^ mix64(t)) % n);
+        dist[t] = INF_DIS;
+        rev[t] = EMPTY;
+        rev_dist[t] = INF_DIS;
+        if (t < n) rev_cnt[t] = 0;
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* p, uint64_t count, uint32_t v) {
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < count; t += (uint64_t)gridDim.x * blockDim.x) p[t] = v;
+}
+
+// Merge of a node's sorted list (o_id with flag bits, o_dist) with survivors given as
+// distinct 64-bit (distance, id) keys. The best min(n_surv, K) survivors are sorted by
+// counting ranks, then old and new elements take their merged ranks: an old element
+// keeps rank pos + #{new <= it}, a new one takes pos + #{old < it} (new first on
+// ties, index.cu:333-351). m_id/m_dist receive the K best. Returns via *n_ins the
+// number of new elements kept. All threads of the block must call it.
+__device__ void block_merge(const uint32_t* o_id, const float* o_dist, uint32_t K, const uint64_t* surv, uint32_t n_surv,
+                            uint64_t* new_sorted, uint32_t* m_id, float* m_dist, uint32_t* n_ins, int tid, int nthreads) {
+    if (tid == 0) *n_ins = 0;
+    for (uint32_t i = tid; i < n_surv; i += nthreads) {
+        const uint64_t k = surv[i];
+        uint32_t r = 0;
+        for (uint32_t j = 0; j < n_surv; j++) r += surv[j] < k;
+        if (r < K) new_sorted[r] = k;
+    }
+    __syncthreads();
+    const uint32_t n_new = min(n_surv, K);
+    for (uint32_t t = tid; t < K + n_new; t += nthreads) {
+        if (t < K) {
+            const float v = o_dist[t];
+            uint32_t lo = 0, len = n_new;
+            while (len > 0) {
+                uint32_t half = len >> 1;
+                if (key_dist(new_sorted[lo + half]) <= v) { lo += half + 1; len -= half + 1; } else len = half;
+            }
+            const uint32_t rank = t + lo;
+            if (rank < K) { m_id[rank] = o_id[t]; m_dist[rank] = v; }
+        } else {
+            const uint32_t i = t - K;
+            const uint64_t k = new_sorted[i];
+            const float v = key_dist(k);
+            uint32_t lo = 0, len = K;
+            while (len > 0) {
+                uint32_t half = len >> 1;
+                if (o_dist[lo + half] < v) { lo += half + 1; len -= half + 1; } else len = half;
+            }
+            const uint32_t rank = i + lo;
+            if (rank < K) { m_id[rank] = (uint32_t)k; m_dist[rank] = v; atomicAdd(n_ins, 1u); }
+        }
+    }
+    __syncthreads();
+}
+
+struct NndLds {
+    uint32_t tab, seen, cand_id, cand_dist, surv, new_sorted, own_id, own_dist, m_id, m_dist, ctl, total;
+    __host__ __device__ NndLds(uint32_t term_slots, uint32_t seen_slots, uint32_t K) {
+        const uint32_t max_cand = NND_PICKS * 2 * K;
+        uint32_t o = 0;
+        tab = o; o += term_slots * 8;
+        surv = o; o += max_cand * 8;
+        new_sorted = o; o += K * 8;
+        seen = o; o += seen_slots * 4;
+        cand_id = o; o += max_cand * 4;
+        cand_dist = o; o += max_cand * 4;
+        own_id = o; o += K * 4;
+        own_dist = o; o += K * 4;
+        m_id = o; o += K * 4;
+        m_dist = o; o += K * 4;
+        ctl = o; o += 16 * 4;
+        total = o;
+    }
+};
+
+// One expansion step for node u = blockIdx.x (index.cu:156-376): sample up to four
+// not-yet-sampled neighbours, gather their forward and reverse lists, drop self,
+// duplicates and ids already in u's list, evaluate the rest against u, merge those
+// closer than u's current worst into the list, and register u with every member of
+// the merged list when the list changed.
+__global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, float dense_mul, uint32_t K, uint32_t* ids, float* dist,
+                                                                  uint32_t* rev, float* rev_dist, uint32_t* rev_cnt, uint32_t term_slots,
+                                                                  uint32_t seen_slots, unsigned long long* inserted) {
+    extern __shared__ __align__(16) char smem[];
+    const NndLds L(term_slots, seen_slots, K);
+    uint2* tab = reinterpret_cast<uint2*>(smem + L.tab);
+    uint64_t* surv = reinterpret_cast<uint64_t*>(smem + L.surv);
+    uint64_t* new_sorted = reinterpret_cast<uint64_t*>(smem + L.new_sorted);
+    uint32_t* seen = reinterpret_cast<uint32_t*>(smem + L.seen);
+    uint32_t* cand_id = reinterpret_cast<uint32_t*>(smem + L.cand_id);
+    float* cand_dist = reinterpret_cast<float*>(smem + L.cand_dist);
+    uint32_t* own_id = reinterpret_cast<uint32_t*>(smem + L.own_id);
+    float* own_dist = reinterpret_cast<float*>(smem + L.own_dist);
+    uint32_t* m_id = reinterpret_cast<uint32_t*>(smem + L.m_id);
+    float* m_dist = reinterpret_cast<float*>(smem + L.m_dist);
+    uint32_t* ctl = reinterpret_cast<uint32_t*>(smem + L.ctl); // [0..3] picks, [4] n_picks, [5] n_cand, [6] n_surv, [7] n_ins
+
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const uint32_t u = blockIdx.x, tmask = term_slots - 1, smask = seen_slots - 1;
+    const size_t base = (size_t)u * K;
+
+    for (uint32_t i = tid; i < K; i += NND_THREADS) { own_id[i] = ids[base + i]; own_dist[i] = dist[base + i]; }
+    term_table_clear(tab, term_slots, tid, NND_THREADS);
+    for (uint32_t i = tid; i < seen_slots; i += NND_THREADS) seen[i] = EMPTY;
+    if (tid < 8) ctl[tid] = 0;
+    __syncthreads();
+
+    // 1. picks: group g takes the first unsampled slot >= g; none left -> slot 0
+    if (wave == 0) {
+        uint64_t m0 = __ballot(!(own_id[lane] & FLAG));
+        uint64_t m1 = K > 64 ? __ballot(!(own_id[64 + lane] & FLAG)) : 0ull;
+        if (lane == 0) {
+            uint32_t np = 0;
+            for (uint32_t g = 0; g < NND_PICKS; g++) {
+                const uint64_t a = m0 & ~((1ull << g) - 1);
+                uint32_t s;
+                if (a) { s = __ffsll((unsigned long long)a) - 1; m0 &= ~(1ull << s); }
+                else if (m1) { s = 64 + __ffsll((unsigned long long)m1) - 1; m1 &= ~(1ull << (s - 64)); }
+                else s = EMPTY;
+                if (s != EMPTY) { own_id[s] |= FLAG; ids[base + s] = own_id[s]; }
+                else s = 0;
+                bool dup = false;
+                for (uint32_t t = 0; t < np; t++) dup |= ctl[t] == s;
+                if (!dup) ctl[np++] = s;
+            }
+            ctl[4] = np;
+        }
+    }
+    // own ids and u itself are never candidates
+    for (uint32_t i = tid; i < K; i += NND_THREADS) id_set_insert(seen, smask, own_id[i] & ~FLAG);
+    if (tid == NND_THREADS - 1) id_set_insert(seen, smask, u);
+    __syncthreads();
+
+    // 2./3. gather forward and reverse lists of the picked neighbours, deduplicated
+    const uint32_t np = ctl[4];
+    for (uint32_t t = tid; t < np * 2 * K; t += NND_THREADS) {
+        const uint32_t p = t / (2 * K), r = t % (2 * K);
+        const uint32_t v = own_id[ctl[p]] & ~FLAG;
+        uint32_t c;
+        if (r < K) c = ids[(size_t)v * K + r] & ~FLAG;
+        else c = rev[(size_t)v * K + (r - K)];
+        if (c < C.n && id_set_insert(seen, smask, c)) cand_id[atomicAdd(&ctl[5], 1u)] = c;
+    }
+    // pivot = u
+    const uint64_t du = C.desc[u];
+    const char* rec = C.recs + desc_off(du) * 16;
+    PivotDense pv;
+    pivot_dense_load(pv, reinterpret_cast<const float*>(rec), 1.0f);
+    pivot_terms_from_record(tab, tmask, rec, desc_nnz_s(du) + desc_nnz_b(du), tid, NND_THREADS);
+    __syncthreads();
+
+    // 4. distances
+    const uint32_t n_cand = ctl[5];
+    for (uint32_t j = wave; j < n_cand; j += NND_THREADS / WAVE) {
+        EvalOut e = eval_wave(C, uniform(cand_id[j]), pv, tab, tmask, PATH_DENSE | PATH_SPARSE | PATH_BM25, dense_mul);
+        if (lane == 0) cand_dist[j] = 1.0f - e.ip;
+    }
+    __syncthreads();
+
+    // 5. survivors: closer than the current worst
+    const float worst = own_dist[K - 1];
+    for (uint32_t j = tid; j < n_cand; j += NND_THREADS)
+        if (cand_dist[j] < worst) surv[atomicAdd(&ctl[6], 1u)] = dist_id_key(cand_dist[j], cand_id[j]);
+    __syncthreads();
+    const uint32_t n_surv = ctl[6];
+    if (n_surv == 0) return;
+    block_merge(own_id, own_dist, K, surv, n_surv, new_sorted, m_id, m_dist, &ctl[7], tid, NND_THREADS);
+
+    // 6. write back and register reverse edges (index.cu:358-372)
+    for (uint32_t j = tid; j < K; j += NND_THREADS) {
+        const uint32_t e = m_id[j];
+        const float dv = m_dist[j];
+        ids[base + j] = e;
+        dist[base + j] = dv;
+        const uint32_t v = e & ~FLAG;
+        const uint32_t slot = atomicAdd(&rev_cnt[v], 1u);
+        const size_t at = (size_t)v * K + (slot % K);
+        if (slot < K || dv < rev_dist[at]) { rev[at] = u; rev_dist[at] = dv; }
+    }
+    if (tid == 0) atomicAdd(inserted, (unsigned long long)ctl[7]);
+}
+
+// Merge with the reverse neighbours registered in the last step (index.cu:386-478).
+__global__ __launch_bounds__(NND_THREADS) void nnd_merge_reverse_kernel(uint32_t n, uint32_t K, uint32_t* ids, float* dist,
+                                                                        const uint32_t* rev, const float* rev_dist,
+                                                                        const uint32_t* rev_cnt) {
+    extern __shared__ __align__(16) char smem[];
+    uint64_t* surv = reinterpret_cast<uint64_t*>(smem);
+    uint64_t* new_sorted = surv + K;
+    uint32_t* own_id = reinterpret_cast<uint32_t*>(new_sorted + K);
+    float* own_dist = reinterpret_cast<float*>(own_id + K);
+    uint32_t* m_id = reinterpret_cast<uint32_t*>(own_dist + K);
+    float* m_dist = reinterpret_cast<float*>(m_id + K);
+    uint32_t* r_id = reinterpret_cast<uint32_t*>(m_dist + K);
+    float* r_dist = reinterpret_cast<float*>(r_id + K);
+    uint32_t* ctl = reinterpret_cast<uint32_t*>(r_dist + K);
+    const int tid = threadIdx.x;
+    const uint32_t u = blockIdx.x;
+    const size_t base = (size_t)u * K;
+    const uint32_t cnt = min(K, rev_cnt[u]);
+    for (uint32_t i = tid; i < K; i += NND_THREADS) {
+        own_id[i] = ids[base + i];
+        own_dist[i] = dist[base + i];
+        r_id[i] = i < cnt ? rev[base + i] : EMPTY;
+        r_dist[i] = i < cnt ? rev_dist[base + i] : INF_DIS;
+    }
+    if (tid < 4) ctl[tid] = 0;
+    __syncthreads();
+    for (uint32_t j = tid; j < cnt; j += NND_THREADS) {
+        const uint32_t r = r_id[j];
+        const float rd = r_dist[j];
+        bool keep = r < n && r != u;
+        for (uint32_t t = 0; keep && t < K; t++) keep = (own_id[t] & ~FLAG) != r;
+        // a repeated reverse id keeps its closest copy (first one on equal distance)
+        for (uint32_t t = 0; keep && t < cnt; t++)
+            if (t != j && r_id[t] == r && (r_dist[t] < rd || (r_dist[t] == rd && t < j))) keep = false;
+        if (keep) surv[atomicAdd(&ctl[0], 1u)] = dist_id_key(rd, r);
+    }
+    __syncthreads();
+    const uint32_t n_surv = ctl[0];
+    if (n_surv == 0) return;
+    block_merge(own_id, own_dist, K, surv, n_surv, new_sorted, m_id, m_dist, &ctl[1], tid, NND_THREADS);
+    for (uint32_t j = tid; j < K; j += NND_THREADS) { ids[base + j] = m_id[j]; dist[base + j] = m_dist[j]; }
+}
+
+static uint32_t doc_term_slots(const apoe_corpus* c) { return next_pow2(std::max(64u, 2 * (c->max_nnz_s + c->max_nnz_b))); }
+
+int launch_nnd_init(apoe_knn* g, uint64_t seed) {
+    apoe_ctx* ctx = g->ctx;
+    const uint64_t total = (uint64_t)g->n * g->K;
+    const uint32_t grid = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
+    nnd_init_kernel<<<grid, 256, 0, ctx->stream>>>(g->n, g->K, seed, g->ids.p, g->dist.p, g->rev.p, g->rev_dist.p, g->rev_cnt.p);
+    APOE_HIP(hipGetLastError());
+    return launch_norms(ctx, g->corpus, g->dense_scale, g->norms.p);
+}
+
+int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted) {
+    apoe_ctx* ctx = g->ctx;
+    const uint32_t term_slots = doc_term_slots(g->corpus);
+    const uint32_t seen_slots = next_pow2(2 * (NND_PICKS * 2 * g->K + g->K + 1));
+    const NndLds L(term_slots, seen_slots, g->K);
+    APOE_REQUIRE(L.total <= 64 * 1024, "NN-Descent needs %u bytes of LDS (rows with up to %u sparse terms)", L.total,
+                 g->corpus->max_nnz_s + g->corpus->max_nnz_b);
+    APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), ctx->stream));
+    APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_iterate_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
+    nnd_iterate_kernel<<<g->n, NND_THREADS, L.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->K, g->ids.p, g->dist.p,
+                                                                    g->rev.p, g->rev_dist.p, g->rev_cnt.p, term_slots, seen_slots, g->counter.p);
+    APOE_HIP(hipGetLastError());
+    if (inserted) {
+        unsigned long long h = 0;
+        APOE_HIP(hipMemcpyAsync(&h, g->counter.p, sizeof(h), hipMemcpyDeviceToHost, ctx->stream));
+        APOE_HIP(hipStreamSynchronize(ctx->stream));
+        *inserted = h;
+    }
+    return APOE_OK;
+}
+
+int launch_nnd_merge_reverse(apoe_knn* g) {
+    apoe_ctx* ctx = g->ctx;
+    const size_t lds = (size_t)g->K * (8 + 8 + 4 * 6) + 16;
+    nnd_merge_reverse_kernel<<<g->n, NND_THREADS, lds, ctx->stream>>>(g->n, g->K, g->ids.p, g->dist.p, g->rev.p, g->rev_dist.p, g->rev_cnt.p);
+    APOE_HIP(hipGetLastError());
+    return APOE_OK;
+}
+
+} // namespace apoe
+
+using namespace apoe;
+
+extern "C" {
+
+int apoe_knn_create(apoe_ctx* ctx, const apoe_corpus* c, uint32_t K, float dense_scale, apoe_knn** out) {
+    APOE_REQUIRE(ctx && c && out, "null argument");
+    *out = nullptr;
+    APOE_REQUIRE(K == 64 || K == 128, "K must be 64 or 128, got %u", K);
+    APOE_REQUIRE(c->n > 1, "at least two documents are needed");
+    APOE_HIP(hipSetDevice(ctx->device));
+    std::unique_ptr<apoe_knn> g(new apoe_knn());
+    g->ctx = ctx;
+    g->corpus = c;
+    g->n = c->n;
+    g->K = K;
+    g->dense_scale = dense_scale;
+    const size_t total = (size_t)c->n * K;
+    APOE_TRY(g->ids.alloc(total));
+    APOE_TRY(g->dist.alloc(total));
+    APOE_TRY(g->rev.alloc(total));
+    APOE_TRY(g->rev_dist.alloc(total));
+    APOE_TRY(g->rev_cnt.alloc(c->n));
+    APOE_TRY(g->norms.alloc(c->n));
+    APOE_TRY(g->counter.alloc(4));
+    *out = g.release();
+    return APOE_OK;
+}
+
+void apoe_knn_destroy(apoe_knn* g) { delete g; }
+
+int apoe_nnd_init(apoe_knn* g, uint64_t seed) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    float ms = 0.f;
+    APOE_TRY(timed(g->ctx, &ms, [&]() { return launch_nnd_init(g, seed); }));
+    g->elapsed_ms = ms;
+    g->pruned = false;
+    return APOE_OK;
+}
+
+int apoe_nnd_iterate(apoe_knn* g, int last, uint64_t* inserted) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    float ms = 0.f;
+    APOE_TRY(timed(g->ctx, &ms, [&]() -> int {
+        APOE_TRY(launch_nnd_iterate(g, nullptr));
+        if (!last) { // reset_reverse_num, index.cu:896
+            fill_u32_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->rev_cnt.p, g->n, 0u);
+            APOE_HIP(hipGetLastError());
+        }
+        return APOE_OK;
+    }));
+    g->elapsed_ms += ms;
+    if (inserted) {
+        unsigned long long h = 0;
+        APOE_HIP(hipMemcpy(&h, g->counter.p, sizeof(h), hipMemcpyDeviceToHost));
+        *inserted = h;
+    }
+    return APOE_OK;
+}
+
+int apoe_nnd_merge_reverse(apoe_knn* g) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    float ms = 0.f;
+    APOE_TRY(timed(g->ctx, &ms, [&]() -> int {
+        APOE_TRY(launch_nnd_merge_reverse(g));
+        fill_u32_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->rev_cnt.p, g->n, 0u); // index.cu:899
+        APOE_HIP(hipGetLastError());
+        return APOE_OK;
+    }));
+    g->elapsed_ms += ms;
+    return APOE_OK;
+}
+
+__global__ __launch_bounds__(256) static void strip_flags_kernel(const uint32_t* in, uint32_t* out, uint64_t count) {
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < count; t += (uint64_t)gridDim.x * blockDim.x) out[t] = in[t] & ~FLAG;
+}
+
+int apoe_knn_download(apoe_knn* g, uint32_t* ids, float* dist) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    const size_t total = (size_t)g->n * g->K;
+    if (ids) {
+        DevBuf<uint32_t> tmp;
+        APOE_TRY(tmp.alloc(total));
+        strip_flags_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->ids.p, tmp.p, total);
+        APOE_HIP(hipGetLastError());
+        APOE_TRY(copy_out(g->ctx, ids, tmp.p, total * sizeof(uint32_t)));
+    }
+    if (dist) APOE_TRY(copy_out(g->ctx, dist, g->dist.p, total * sizeof(float)));
+    return APOE_OK;
+}
+
+int apoe_knn_upload(apoe_knn* g, const uint32_t* ids, const float* dist) {
+    APOE_REQUIRE(g && ids && dist, "null argument");
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    const size_t total = (size_t)g->n * g->K;
+    APOE_TRY(copy_in(g->ctx, g->ids.p, ids, total * sizeof(uint32_t)));
+    APOE_TRY(copy_in(g->ctx, g->dist.p, dist, total * sizeof(float)));
+    APOE_TRY(launch_norms(g->ctx, g->corpus, g->dense_scale, g->norms.p));
+    APOE_HIP(hipStreamSynchronize(g->ctx->stream));
+    g->pruned = false;
+    return APOE_OK;
+}
+
+float apoe_knn_elapsed_ms(const apoe_knn* g) { return g ? g->elapsed_ms : 0.f; }
+
+} // extern "C"

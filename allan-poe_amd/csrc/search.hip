@@ -1,0 +1,367 @@
+// Greedy beam search over the hybrid graph: one workgroup per query, the candidate
+// pool, the query's sparse-term table and the fresh-neighbour list in LDS, the
+// query's dense row in registers, an exact visited bitmap per workgroup in HBM.
+#include "apoe_internal.h"
+
+namespace apoe {
+
+constexpr int MAX_NEW = 64; // fresh candidates per step: one lane each in wave 0
+
+struct SearchArgs {
+    CorpusView C;
+    SetView Q;
+    const uint32_t* graph;
+    uint32_t W, degree;
+    const uint32_t* entry;
+    uint32_t n_entry;
+    float w_d, w_s, w_b;
+    uint32_t paths;
+    uint32_t cands, max_iter, q_begin, q_count;
+    uint32_t* out_ids;
+    float* out_dist;
+    uint32_t* bitmaps;     // one visited bitmap per workgroup
+    uint32_t bitmap_words; // multiple of 4
+    unsigned long long* work; // [0] next query, [1] expansions, [2] evaluations, [3] nnz splade, [4] nnz bm25
+    uint32_t slots;
+    // knowledge graph (KG kernels only)
+    const uint32_t *e2e_off, *e2e_idx, *e2d_off, *e2d_idx, *q2e_off, *q2e_idx;
+    uint32_t n_entities;
+    float kg_weight;
+};
+
+// LDS carve-up shared by host (size) and device (pointers).
+struct SearchLds {
+    uint32_t tab, pool_id, pool_dist, pool_ent, pool_hop, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ctl, total;
+    __host__ __device__ SearchLds(uint32_t slots, uint32_t cands, bool kg) {
+        uint32_t o = 0;
+        tab = o; o += slots * 8;
+        pool_id = o; o += 2 * cands * 4;
+        pool_dist = o; o += 2 * cands * 4;
+        pool_ent = o; o += kg ? 2 * cands * 4 : 0;
+        pool_hop = o; o += kg ? 2 * cands * 4 : 0;
+        new_id = o; o += MAX_NEW * 4;
+        new_dist = o; o += MAX_NEW * 4;
+        new_ent = o; o += kg ? MAX_NEW * 4 : 0;
+        new_hop = o; o += kg ? MAX_NEW * 4 : 0;
+        seed_id = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
+        seed_ent = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
+        seed_dist = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
+        link = o; o += kg ? MAX_NEW * 4 : 0;
+        ctl = o; o += 16 * 4;
+        total = o;
+    }
+};
+
+enum { CTL_QUERY = 0, CTL_PARENT = 1, CTL_NNEW = 2, CTL_CUR = 3, CTL_PENT = 4, CTL_PHOP = 5, CTL_NSEED = 6 };
+
+struct Pool {
+    uint32_t* id;   // [2][cands]
+    float* dist;    // [2][cands]
+    uint32_t* ent;  // KG only
+    uint32_t* hop;  // KG only
+    uint32_t cands;
+};
+
+__device__ __forceinline__ void wave_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// Wave 0 only. Sorts the n (<= 64) new candidates by (distance, id) and rank-merges
+// them into the pool (source half `cur`, destination half `cur ^ 1`): a pool element
+// keeps rank pos + #{new <= it}, a new element takes rank pos + #{pool < it}, so on
+// equal distance the new one goes first; ranks >= cands fall off. Returns cur ^ 1.
+template <bool KG>
+__device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t cur, uint32_t* nid, float* ndist, uint32_t* nent, uint32_t* nhop,
+                                               uint32_t n) {
+    const int lane = lane_id();
+    const uint32_t cands = P.cands;
+    float d = lane < (int)n ? ndist[lane] : INF_DIS;
+    uint32_t id = lane < (int)n ? nid[lane] : EMPTY;
+    uint64_t key = lane < (int)n ? dist_id_key(d, id) : ~0ull;
+    uint32_t ent = EMPTY, hop = 0;
+    if (KG) {
+        if (lane < (int)n) { ent = nent[lane]; hop = nhop[lane]; }
+        // the distance travels inside the key; payloads travel beside it
+        wave_sort64_payload(key, ent, hop);
+    } else {
+        key = wave_sort64(key);
+    }
+    wave_fence();
+    id = (uint32_t)key;
+    {   // recover the float from its order-preserving key
+        uint32_t u = (uint32_t)(key >> 32);
+        u ^= (u >> 31) ? 0x80000000u : 0xFFFFFFFFu;
+        d = __uint_as_float(u);
+    }
+    if (lane >= (int)n) { d = INF_DIS; id = EMPTY; }
+    ndist[lane] = d; // sorted copy for the pool elements' searches
+    wave_fence();
+    const uint32_t* sid = P.id + cur * cands;
+    const float* sdist = P.dist + cur * cands;
+    uint32_t* did = P.id + (cur ^ 1) * cands;
+    float* ddist = P.dist + (cur ^ 1) * cands;
+    // new element: lower_bound over the pool
+    if (lane < (int)n) {
+        uint32_t lo = 0, len = cands;
+        while (len > 0) {
+            uint32_t half = len >> 1;
+            if (sdist[lo + half] < d) { lo += half + 1; len -= half + 1; } else len = half;
+        }
+        uint32_t rank = lo + lane;
+        if (rank < cands) {
+            did[rank] = id;
+            ddist[rank] = d;
+            if (KG) { P.ent[(cur ^ 1) * cands + rank] = ent; P.hop[(cur ^ 1) * cands + rank] = hop; }
+        }
+    }
+    // pool element: upper_bound over the sorted new list
+    for (uint32_t base = 0; base < cands; base += WAVE) {
+        uint32_t p = base + lane;
+        if (p < cands) {
+            float v = sdist[p];
+            uint32_t lo = 0, len = n;
+            while (len > 0) {
+                uint32_t half = len >> 1;
+                if (ndist[lo + half] <= v) { lo += half + 1; len -= half + 1; } else len = half;
+            }
+            uint32_t rank = p + lo;
+            if (rank < cands) {
+                did[rank] = sid[p];
+                ddist[rank] = v;
+                if (KG) { P.ent[(cur ^ 1) * cands + rank] = P.ent[cur * cands + p]; P.hop[(cur ^ 1) * cands + rank] = P.hop[cur * cands + p]; }
+            }
+        }
+    }
+    wave_fence();
+    return cur ^ 1;
+}
+
+template <int NW, bool KG>
+__global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
+    extern __shared__ __align__(16) char smem[];
+    const SearchLds L(a.slots, a.cands, KG);
+    uint2* tab = reinterpret_cast<uint2*>(smem + L.tab);
+    Pool P;
+    P.id = reinterpret_cast<uint32_t*>(smem + L.pool_id);
+    P.dist = reinterpret_cast<float*>(smem + L.pool_dist);
+    P.ent = reinterpret_cast<uint32_t*>(smem + L.pool_ent);
+    P.hop = reinterpret_cast<uint32_t*>(smem + L.pool_hop);
+    P.cands = a.cands;
+    uint32_t* new_id = reinterpret_cast<uint32_t*>(smem + L.new_id);
+    float* new_dist = reinterpret_cast<float*>(smem + L.new_dist);
+    uint32_t* new_ent = reinterpret_cast<uint32_t*>(smem + L.new_ent);
+    uint32_t* new_hop = reinterpret_cast<uint32_t*>(smem + L.new_hop);
+    uint32_t* seed_id = reinterpret_cast<uint32_t*>(smem + L.seed_id);
+    uint32_t* seed_ent = reinterpret_cast<uint32_t*>(smem + L.seed_ent);
+    float* seed_dist = reinterpret_cast<float*>(smem + L.seed_dist);
+    uint32_t* link = reinterpret_cast<uint32_t*>(smem + L.link);
+    volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
+
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const uint32_t mask = a.slots - 1, cands = a.cands;
+    uint32_t* bitmap = a.bitmaps + (size_t)blockIdx.x * a.bitmap_words;
+    const uint64_t lane_lt = (1ull << lane) - 1;
+
+    while (true) {
+        __syncthreads();
+        if (tid == 0) ctl[CTL_QUERY] = (uint32_t)atomicAdd(a.work, 1ull);
+        __syncthreads();
+        const uint32_t qi = ctl[CTL_QUERY];
+        if (qi >= a.q_count) break;
+        const uint32_t q = a.q_begin + qi;
+
+        // ---- reset per-query state ----
+        {
+            uint4* b4 = reinterpret_cast<uint4*>(bitmap);
+            for (uint32_t i = tid; i < a.bitmap_words / 4; i += NW * WAVE) b4[i] = make_uint4(0, 0, 0, 0);
+        }
+        term_table_clear(tab, a.slots, tid, NW * WAVE);
+        for (uint32_t i = tid; i < cands; i += NW * WAVE) {
+            P.id[i] = EMPTY;
+            P.dist[i] = INF_DIS;
+            if (KG) { P.ent[i] = EMPTY; P.hop[i] = 0; }
+        }
+        PivotDense pv;
+        pivot_dense_load(pv, a.Q.dense + (size_t)q * DIM, a.w_d);
+        __threadfence();
+        __syncthreads();
+        pivot_terms_from_query(tab, mask, a.Q, q, a.w_s, a.w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
+
+        uint64_t st_exp = 0, st_eval = 0, st_ns = 0, st_nb = 0; // wave-uniform counters
+        uint32_t cur = 0;                                        // live pool half (wave 0's copy is authoritative)
+
+        // ---- seeds: entry points (query.cu:440-485) ----
+        if (!KG) {
+            if (wave == 0) {
+                uint32_t c = lane < (int)a.n_entry ? a.entry[lane] : EMPTY;
+                bool fresh = false;
+                if (c < a.C.n) {
+                    const uint32_t bit = 1u << (c & 31);
+                    fresh = !(atomicOr(&bitmap[c >> 5], bit) & bit);
+                }
+                const uint64_t b = __ballot(fresh);
+                if (fresh) new_id[__popcll(b & lane_lt)] = c;
+                if (lane == 0) { ctl[CTL_NNEW] = __popcll(b); ctl[CTL_PARENT] = 0; }
+            }
+        }
+        __syncthreads();
+
+        for (uint32_t it = 0; it <= a.max_iter; it++) {
+            // ---- evaluate the fresh candidates: one wave per candidate ----
+            const uint32_t n_new = ctl[CTL_NNEW];
+            if (ctl[CTL_PARENT] == EMPTY) break;
+            for (uint32_t j = wave; j < n_new; j += NW) {
+                const uint32_t id = uniform(new_id[j]);
+                EvalOut e = eval_wave(a.C, id, pv, tab, mask, a.paths, 1.0f);
+                st_eval++;
+                st_ns += e.nnz_s;
+                st_nb += e.nnz_b;
+                if (lane == 0) new_dist[j] = 1.0f - e.ip;
+            }
+            __syncthreads();
+            // ---- wave 0: merge, pick the next parent, fetch its neighbours ----
+            if (wave == 0) {
+                cur = sort_merge<KG>(P, cur, new_id, new_dist, new_ent, new_hop, n_new);
+                uint32_t parent = EMPTY, slot = 0, n_next = 0;
+                if (it < a.max_iter) {
+                    const uint32_t* pid = P.id + cur * cands;
+                    for (uint32_t base = 0; base < cands; base += WAVE) {
+                        const uint32_t id = base + lane < cands ? pid[base + lane] : EMPTY;
+                        const uint64_t b = __ballot((id & FLAG) == 0);
+                        if (b) {
+                            const int l = __ffsll((unsigned long long)b) - 1;
+                            slot = base + l;
+                            parent = __shfl(id, l, WAVE);
+                            break;
+                        }
+                    }
+                }
+                if (parent != EMPTY) {
+                    if (lane == 0) P.id[cur * cands + slot] = parent | FLAG;
+                    st_exp++;
+                    uint32_t c = lane < (int)a.degree ? a.graph[(size_t)parent * a.W + lane] : EMPTY;
+                    bool fresh = false;
+                    if (c < a.C.n) {
+                        const uint32_t bit = 1u << (c & 31);
+                        fresh = !(atomicOr(&bitmap[c >> 5], bit) & bit);
+                    }
+                    const uint64_t b = __ballot(fresh);
+                    if (fresh) new_id[__popcll(b & lane_lt)] = c;
+                    n_next = __popcll(b);
+                }
+                if (lane == 0) { ctl[CTL_PARENT] = parent; ctl[CTL_NNEW] = n_next; ctl[CTL_CUR] = cur; }
+            }
+            __syncthreads();
+        }
+        // ---- results (query.cu:566-569) ----
+        cur = ctl[CTL_CUR];
+        for (uint32_t i = tid; i < cands; i += NW * WAVE) {
+            a.out_ids[(size_t)qi * cands + i] = P.id[cur * cands + i] & ~FLAG;
+            a.out_dist[(size_t)qi * cands + i] = P.dist[cur * cands + i];
+        }
+        if (lane == 0) {
+            if (st_exp) atomicAdd(a.work + 1, st_exp);
+            if (st_eval) atomicAdd(a.work + 2, st_eval);
+            if (st_ns) atomicAdd(a.work + 3, st_ns);
+            if (st_nb) atomicAdd(a.work + 4, st_nb);
+        }
+    }
+}
+
+template <int NW, bool KG>
+static int launch_variant(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, size_t lds) {
+    APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&search_kernel<NW, KG>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    search_kernel<NW, KG><<<grid, NW * WAVE, lds, ctx->stream>>>(a);
+    APOE_HIP(hipGetLastError());
+    return APOE_OK;
+}
+
+int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g, const apoe_kg* kg,
+                  const apoe_search_params* p, uint32_t* out_ids_dev, float* out_dist_dev, apoe_search_stats* stats) {
+    APOE_REQUIRE(p->cands >= 1 && p->cands <= 512, "cands must be in 1..512, got %u", p->cands);
+    APOE_REQUIRE(g->width > APOE_KW_SLOTS && g->width - APOE_KW_SLOTS <= MAX_NEW, "graph degree must be in 1..64, got width %u", g->width);
+    APOE_REQUIRE(g->n == c->n, "graph has %u nodes but the corpus has %u documents", g->n, c->n);
+    APOE_REQUIRE(p->q_begin <= q->n, "q_begin %u beyond %u queries", p->q_begin, q->n);
+    APOE_REQUIRE(kg == nullptr, "knowledge-graph search is not available in this build");
+    const uint32_t q_count = p->q_count ? p->q_count : q->n - p->q_begin;
+    APOE_REQUIRE(p->q_begin + q_count <= q->n, "query range [%u,%u) beyond %u queries", p->q_begin, p->q_begin + q_count, q->n);
+    if (stats) *stats = apoe_search_stats{};
+    if (q_count == 0) return APOE_OK;
+
+    SearchArgs a{};
+    a.C = c->view();
+    a.Q = q->view();
+    a.graph = g->rows.p;
+    a.W = g->width;
+    a.degree = g->width - APOE_KW_SLOTS;
+    a.entry = g->entry.p;
+    a.n_entry = std::min<uint32_t>(g->n_entry, MAX_NEW);
+    a.w_d = p->w_dense;
+    a.w_s = p->w_sparse;
+    a.w_b = p->w_bm25;
+    a.paths = (!(p->w_dense < 1e-5f) ? PATH_DENSE : 0) | (!(p->w_sparse < 1e-5f) ? PATH_SPARSE : 0) | (!(p->w_bm25 < 1e-5f) ? PATH_BM25 : 0);
+    a.cands = p->cands;
+    a.max_iter = p->max_iter ? p->max_iter : 1000;
+    a.q_begin = p->q_begin;
+    a.q_count = q_count;
+    a.out_ids = out_ids_dev;
+    a.out_dist = out_dist_dev;
+    a.slots = next_pow2(std::max(64u, 2 * q->max_nnz));
+    a.kg_weight = p->kg_weight;
+
+    const bool use_kg = false;
+    const SearchLds L(a.slots, a.cands, use_kg);
+    APOE_REQUIRE(L.total <= 64 * 1024, "search needs %u bytes of LDS (query rows with up to %u sparse terms)", L.total, q->max_nnz);
+
+    int nw = 4;
+    if (p->variant == 1) nw = 1;
+    else if (p->variant == 2) nw = 2;
+    else if (p->variant == 3) nw = 8;
+    // resident workgroups: bounded by LDS, by waves per CU, and by the number of queries
+    const uint32_t per_cu_lds = (uint32_t)((160 * 1024) / std::max<uint32_t>(L.total, 1));
+    const uint32_t per_cu_waves = 32u / nw; // up to 8 waves per SIMD; keep half for register headroom
+    const uint32_t per_cu = std::max(1u, std::min(per_cu_lds, per_cu_waves));
+    const uint32_t grid = std::min<uint32_t>(q_count, per_cu * (uint32_t)ctx->num_cus);
+
+    a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;
+    DevBuf<uint32_t> bitmaps;
+    DevBuf<unsigned long long> work;
+    APOE_TRY(bitmaps.alloc((size_t)grid * a.bitmap_words));
+    APOE_TRY(work.alloc(8));
+    APOE_HIP(hipMemsetAsync(work.p, 0, 8 * sizeof(unsigned long long), ctx->stream));
+    a.bitmaps = bitmaps.p;
+    a.work = work.p;
+
+    float ms = 0.f;
+    APOE_TRY(timed(ctx, &ms, [&]() {
+        switch (nw) {
+            case 1: return launch_variant<1, false>(ctx, a, grid, L.total);
+            case 2: return launch_variant<2, false>(ctx, a, grid, L.total);
+            case 8: return launch_variant<8, false>(ctx, a, grid, L.total);
+            default: return launch_variant<4, false>(ctx, a, grid, L.total);
+        }
+    }));
+    APOE_HIP(hipStreamSynchronize(ctx->stream));
+    if (stats) {
+        unsigned long long h[8];
+        APOE_HIP(hipMemcpy(h, work.p, sizeof(h), hipMemcpyDeviceToHost));
+        stats->kernel_ms = ms;
+        stats->expansions = h[1];
+        stats->evaluations = h[2];
+        stats->nnz_sparse = h[3];
+        stats->nnz_bm25 = h[4];
+        // rows + pairs + descriptor (8 B ~ the two CSR offset pairs' 16 B of the reference layout)
+        uint64_t bytes = 0;
+        if (a.paths & PATH_DENSE) bytes += h[2] * (uint64_t)DENSE_BYTES;
+        bytes += 8 * (h[3] + h[4]) + 8 * h[2];
+        bytes += h[1] * 4ull * a.W;
+        uint64_t qbytes = (uint64_t)q_count * DENSE_BYTES + 8 * (q->h_s_off[p->q_begin + q_count] - q->h_s_off[p->q_begin]) +
+                          8 * (q->h_b_off[p->q_begin + q_count] - q->h_b_off[p->q_begin]);
+        bytes += qbytes + (uint64_t)q_count * a.cands * 8;
+        stats->algo_bytes = bytes;
+    }
+    return APOE_OK;
+}
+
+} // namespace apoe

@@ -1,0 +1,164 @@
+/*
+ * apoe.h -- C-ABI of the MI355X (gfx950) implementation of the Allan-Poe hybrid
+ * graph index hot path: fused hybrid distance, NN-Descent, RNG-IP pruning with
+ * keyword recycling, final graph assembly, and greedy beam search with optional
+ * knowledge-graph expansion.
+ *
+ * Conventions
+ *  - Every function returns APOE_OK (0) or a negative status; the message of the
+ *    last failure on the calling thread is apoe_last_error_string(). Nothing here
+ *    throws or exits (the reference calls exit() on any failure, index.cu:19-28).
+ *  - Bulk input/output pointers may point to host memory or to device memory of
+ *    the context's GPU; the library copies with hipMemcpyDefault. The caller owns
+ *    them; the library owns everything it allocates on the device.
+ *  - All work of a context runs on the context's own HIP stream. A context and
+ *    its handles may be used from one thread at a time. There is no global state.
+ *  - Sparse matrices are CSR in the reference's file layout: off[rows+1], idx[nnz]
+ *    ascending inside a row, val[nnz] (utils.cuh:380-398). Term ids must be < 2^31.
+ *  - Document ids must be < 2^30 (bits 30/31 are flags inside pools, query.cu:503).
+ *  - dim must be 1024 (utils.cuh:31 DIM).
+ */
+#ifndef APOE_H
+#define APOE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define APOE_OK 0
+#define APOE_ERR_ARG -1      /* bad argument / unsupported size */
+#define APOE_ERR_HIP -2      /* a HIP runtime call failed */
+#define APOE_ERR_STATE -3    /* call sequence error (e.g. finalize before prune) */
+
+#define APOE_INF_DIS 1000000.0f /* index.cu:8, query.cu:11 */
+#define APOE_KW_SLOTS 8         /* index.cu:15 KEYEDGEFINAL: row width = degree + 8 */
+#define APOE_KW_CAND 32         /* index.cu:14 KEYEDGE */
+
+typedef struct apoe_ctx apoe_ctx;
+typedef struct apoe_corpus apoe_corpus;
+typedef struct apoe_queries apoe_queries;
+typedef struct apoe_kg apoe_kg;
+typedef struct apoe_graph apoe_graph;
+typedef struct apoe_knn apoe_knn;
+
+const char* apoe_last_error_string(void);
+
+/* Replaces the implicit "device 0, default stream" of the reference. */
+int apoe_ctx_create(int device, apoe_ctx** out);
+void apoe_ctx_destroy(apoe_ctx* ctx);
+int apoe_ctx_synchronize(apoe_ctx* ctx);
+
+/*
+ * Corpus upload. Replaces the cudaMalloc/cudaMemcpy block of build_index_impl
+ * (index.cu:842-872) and search_index_impl (query.cu:1909-1934). The rows are
+ * repacked on the device into one record per document (dense row followed by the
+ * SPLADE and BM25 (id, value) pairs) so that one evaluation is one contiguous read.
+ */
+int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* dense,
+                       const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,
+                       const uint32_t* b_off, const uint32_t* b_idx, const float* b_val,
+                       apoe_corpus** out);
+void apoe_corpus_destroy(apoe_corpus* c);
+/* info4 = {n, dim, max splade nnz per row, max bm25 nnz per row} (index.cu:829-835). */
+int apoe_corpus_info(const apoe_corpus* c, uint32_t* info4);
+/* Bytes of the device records: the HBM footprint one full scan reads. */
+uint64_t apoe_corpus_bytes(const apoe_corpus* c);
+
+/* Query upload (query.cu:1936-1961). Weights are NOT folded in here; they are
+ * applied when a search or distance call loads the query (query.cu:1871-1881). */
+int apoe_queries_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* dense,
+                        const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,
+                        const uint32_t* b_off, const uint32_t* b_idx, const float* b_val,
+                        apoe_queries** out);
+void apoe_queries_destroy(apoe_queries* q);
+
+/* KG upload (query.cu:1963-1980). Each CSR has rows+1 offsets. */
+int apoe_kg_create(apoe_ctx* ctx, uint32_t n_entities, const uint32_t* e2e_off,
+                   const uint32_t* e2e_idx, const uint32_t* e2d_off, const uint32_t* e2d_idx,
+                   uint32_t n_queries, const uint32_t* q2e_off, const uint32_t* q2e_idx,
+                   apoe_kg** out);
+void apoe_kg_destroy(apoe_kg* kg);
+
+/*
+ * Fused hybrid distance, query side (the per-candidate block of every search
+ * kernel, query.cu:536-557): out[q*M+m] = 1 - (w3[0]*dense + w3[1]*splade +
+ * w3[2]*bm25) between query q and document ids[q*M+m]; w3 = {dense, splade, bm25};
+ * a path with weight < 1e-5 is skipped (query.cu:2004-2041); ids >= n give INF_DIS.
+ */
+int apoe_hybrid_distance_batch(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q,
+                               const float* w3, const uint32_t* ids, uint32_t M, float* out);
+
+/* Build-metric distance between documents a[i] and b[i] (index.cu:248-267):
+ * 1 - (dense_scale^2*dense + splade + bm25); dense_scale is the x7 of index.cu:836-840. */
+int apoe_hybrid_distance_pairs(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale,
+                               const uint32_t* a, const uint32_t* b, uint32_t n_pairs, float* out);
+
+/* Hybrid squared norms (cal_power, index.cu:483-534). out has n floats. */
+int apoe_norms(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale, float* out);
+
+/* ---- index construction (build_index_impl, index.cu:889-903) ---- */
+
+/* kNN-graph state: ids/dist [n][K], reverse lists, norms. K is 64 or 128 (index.cu:6). */
+int apoe_knn_create(apoe_ctx* ctx, const apoe_corpus* c, uint32_t K, float dense_scale,
+                    apoe_knn** out);
+void apoe_knn_destroy(apoe_knn* g);
+/* initialize_graph + cal_power (index.cu:890-892). */
+int apoe_nnd_init(apoe_knn* g, uint64_t seed);
+/* One nn_descent_gpu + reset_reverse_num step (index.cu:894-897). last != 0 keeps the
+ * reverse counts for the following merge. *inserted (optional) = list entries inserted. */
+int apoe_nnd_iterate(apoe_knn* g, int last, uint64_t* inserted);
+/* merge_reverse_plus (index.cu:898). */
+int apoe_nnd_merge_reverse(apoe_knn* g);
+/* Copy the kNN graph out / in (ids without flag bits, distances), [n][K] each. */
+int apoe_knn_download(apoe_knn* g, uint32_t* ids, float* dist);
+int apoe_knn_upload(apoe_knn* g, const uint32_t* ids, const float* dist);
+/* allan_poe (index.cu:539-714): RNG-IP prune to `degree` + keyword-edge candidates. */
+int apoe_prune(apoe_knn* g, uint32_t degree);
+/* Intermediate result of apoe_prune: fwd/det [n][degree], cnt [n], kw [n][1+APOE_KW_CAND]. */
+int apoe_prune_download(apoe_knn* g, uint32_t* fwd, uint32_t* det, uint32_t* cnt, uint32_t* kw);
+/* allan_poe_final_graph + entry-point selection (index.cu:717-807, 916-925). */
+int apoe_finalize_graph(apoe_knn* g, apoe_graph** out);
+/* Milliseconds of GPU time (HIP events on the context stream) spent in the build
+ * calls on this handle so far: the reference's "Indexing time" region (index.cu:889-908). */
+float apoe_knn_elapsed_ms(const apoe_knn* g);
+
+/* ---- graph handle: the .poe payload (index.cu:927-939, query.cu:35-62) ---- */
+int apoe_graph_create(apoe_ctx* ctx, uint32_t n, uint32_t width, const uint32_t* rows,
+                      const uint32_t* entry, uint32_t n_entry, apoe_graph** out);
+void apoe_graph_destroy(apoe_graph* g);
+/* info3 = {n, width, n_entry}. */
+int apoe_graph_info(const apoe_graph* g, uint32_t* info3);
+int apoe_graph_download(const apoe_graph* g, uint32_t* rows, uint32_t* entry);
+
+/* ---- search (search_with_* kernels, query.cu:277-1268, 1541-1779) ---- */
+typedef struct {
+    float w_dense, w_sparse, w_bm25; /* effective (already calibrated) weights */
+    float kg_weight;                 /* used only when kg != NULL */
+    uint32_t cands;                  /* pool size, 1..512 (query.cu:9 MAX_CAND_POOL) */
+    uint32_t max_iter;               /* 0 -> 1000 (query.cu:7 MAX_ITER) */
+    uint32_t q_begin, q_count;       /* query range; q_count 0 -> all from q_begin */
+    uint32_t variant;                /* 0 = default launch shape; others are tuning shapes */
+} apoe_search_params;
+
+typedef struct {
+    float kernel_ms;      /* HIP-event time of the search kernel on the context stream */
+    uint64_t expansions;  /* parents expanded, summed over the queries */
+    uint64_t evaluations; /* hybrid distance evaluations */
+    uint64_t nnz_sparse;  /* SPLADE pairs read by those evaluations (0 if path off) */
+    uint64_t nnz_bm25;    /* BM25 pairs read by those evaluations (0 if path off) */
+    uint64_t algo_bytes;  /* algorithmic HBM bytes: rows + pairs + descriptors + graph rows
+                             + queries + results */
+} apoe_search_stats;
+
+/* out_ids/out_dist are [q_count][cands], ascending distance; top_k is the row
+ * prefix (query.cu:2070-2075). Empty slots hold id 0x7FFFFFFF, distance INF_DIS. */
+int apoe_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g,
+                const apoe_kg* kg, const apoe_search_params* p, uint32_t* out_ids, float* out_dist,
+                apoe_search_stats* stats);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
