@@ -37,7 +37,7 @@ class SearchStats(C.Structure):
 EXPORTS = [
     "apoe_last_error_string", "apoe_ctx_create", "apoe_ctx_destroy", "apoe_ctx_synchronize", "apoe_corpus_create",
     "apoe_corpus_destroy", "apoe_corpus_info", "apoe_corpus_bytes", "apoe_queries_create", "apoe_queries_destroy",
-    "apoe_kg_create", "apoe_kg_destroy", "apoe_hybrid_distance_batch", "apoe_hybrid_distance_pairs", "apoe_norms",
+    "apoe_kg_create", "apoe_kg_destroy", "apoe_calibrate_weights", "apoe_hybrid_distance_batch", "apoe_hybrid_distance_pairs", "apoe_norms",
     "apoe_knn_create", "apoe_knn_destroy", "apoe_nnd_init", "apoe_nnd_iterate", "apoe_nnd_merge_reverse",
     "apoe_knn_download", "apoe_knn_upload", "apoe_prune", "apoe_prune_download", "apoe_finalize_graph",
     "apoe_knn_elapsed_ms", "apoe_graph_create", "apoe_graph_destroy", "apoe_graph_info", "apoe_graph_download",
@@ -312,6 +312,13 @@ def norms(ctx, corpus, dense_scale):
     out = np.empty(corpus.n, np.float32)
     _check(lib().apoe_norms(ctx.h, corpus.h, C.c_float(dense_scale), C.c_void_p(out.ctypes.data)))
     return out
+
+
+def calibrate_weights(ctx, corpus, queries, w3, n_queries=None):
+    """Effective (dense, sparse, bm25) weights after the reference's calibration step."""
+    w = (C.c_float * 3)(*w3)
+    _check(lib().apoe_calibrate_weights(ctx.h, corpus.h, queries.h, C.c_uint32(queries.n if n_queries is None else n_queries), w))
+    return (float(w[0]), float(w[1]), float(w[2]))
 
 
 def search(ctx, corpus, queries, graph, w3, cands, kg=None, kg_weight=0.0, max_iter=0, q_begin=0, q_count=0, variant=0,

@@ -1,6 +1,7 @@
 // C-ABI entry points (include/apoe.h): handle life cycle, uploads, and thin
 // wrappers that stage caller memory and call the kernel launchers.
 #include <algorithm>
+#include <cmath>
 #include <memory>
 #include <numeric>
 
@@ -307,6 +308,42 @@ int apoe_norms(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale, float* ou
     APOE_TRY(launch_norms(ctx, c, dense_scale, d_out.p));
     APOE_HIP(hipStreamSynchronize(ctx->stream));
     return d_out.finish(ctx);
+}
+
+int apoe_calibrate_weights(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, uint32_t n_queries, float* w3) {
+    APOE_REQUIRE(ctx && c && q && w3, "null argument");
+    APOE_HIP(hipSetDevice(ctx->device));
+    const uint32_t nd = std::min<uint32_t>(c->n, 100), nq = std::min<uint32_t>(std::min(n_queries, q->n), 100);
+    if (nd == 0 || nq == 0) return APOE_OK;
+    // per-path inner products of the first nd documents with the first nq queries
+    std::vector<uint32_t> ids((size_t)q->n * nd);
+    for (uint32_t i = 0; i < q->n; i++)
+        for (uint32_t j = 0; j < nd; j++) ids[(size_t)i * nd + j] = i < nq ? j : 0xFFFFFFFFu;
+    DevBuf<uint32_t> d_ids;
+    DevBuf<float> d_out;
+    APOE_TRY(d_ids.alloc(ids.size()));
+    APOE_TRY(d_out.alloc(ids.size()));
+    APOE_TRY(copy_in(ctx, d_ids.p, ids.data(), ids.size() * sizeof(uint32_t)));
+    std::vector<float> out(ids.size());
+    float mx[3];
+    for (int p = 0; p < 3; p++) {
+        const float w[3] = {p == 0 ? 1.f : 0.f, p == 1 ? 1.f : 0.f, p == 2 ? 1.f : 0.f};
+        APOE_TRY(launch_distance_batch(ctx, c, q, w, d_ids.p, nd, d_out.p));
+        APOE_TRY(copy_out(ctx, out.data(), d_out.p, out.size() * sizeof(float)));
+        float m = -INFINITY;
+        for (uint32_t i = 0; i < nq; i++)
+            for (uint32_t j = 0; j < nd; j++) m = std::max(m, 1.0f - out[(size_t)i * nd + j]);
+        mx[p] = m;
+    }
+    // query.cu:1858-1869: the path with the strictly largest maximum is the yardstick
+    int big = -1;
+    if (mx[1] > mx[2] && mx[1] > mx[0]) big = 1;
+    else if (mx[2] > mx[1] && mx[2] > mx[0]) big = 2;
+    else if (mx[0] > mx[1] && mx[0] > mx[2]) big = 0;
+    if (big < 0) return APOE_OK;
+    for (int p = 0; p < 3; p++)
+        if (p != big && mx[p] > 0.f) w3[p] *= mx[big] / mx[p];
+    return APOE_OK;
 }
 
 int apoe_graph_create(apoe_ctx* ctx, uint32_t n, uint32_t width, const uint32_t* rows, const uint32_t* entry, uint32_t n_entry,

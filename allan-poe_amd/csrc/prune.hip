@@ -1,0 +1,456 @@
+// RNG-IP joint pruning with keyword-aware neighbour recycling, and the final row
+// assembly with reverse edges. One workgroup (4 waves) per node for the prune, one
+// wave per node for the assembly.
+#include <hipcub/hipcub.hpp>
+
+#include <algorithm>
+#include <memory>
+
+#include "apoe_internal.h"
+
+namespace apoe {
+
+constexpr int PR_THREADS = 256;
+constexpr uint32_t ALL_PATHS = PATH_DENSE | PATH_SPARSE | PATH_BM25;
+
+struct PruneLds {
+    uint32_t tab, idmap, uset, nb_id, nb_dist, det, cid, cdet, sel_id, sel_det, sel_live, sel_kw, o_fwd, o_det, o_kw, ctl, total;
+    __host__ __device__ PruneLds(uint32_t term_slots, uint32_t uset_slots, uint32_t map_slots, uint32_t K) {
+        uint32_t o = 0;
+        tab = o; o += term_slots * 8;
+        idmap = o; o += map_slots * 8;
+        uset = o; o += uset_slots * 4;
+        nb_id = o; o += K * 4;
+        nb_dist = o; o += K * 4;
+        det = o; o += K * 4;
+        cid = o; o += K * 4;
+        cdet = o; o += K * 4;
+        sel_id = o; o += K * 4;
+        sel_det = o; o += K * 4;
+        sel_live = o; o += K * 4;
+        sel_kw = o; o += K * 4;
+        o_fwd = o; o += K * 4;
+        o_det = o; o += K * 4;
+        o_kw = o; o += (1 + APOE_KW_CAND) * 4;
+        ctl = o; o += 16 * 4;
+        total = o;
+    }
+};
+
+enum { PC_M = 0, PC_NSEL = 1, PC_REJECT = 2, PC_ALLFLAG = 3, PC_CNT = 4 };
+
+// allan_poe (index.cu:539-714) for node u = blockIdx.x:
+//  (a) detour counts over u's sorted list; (b) order by (detour, rank);
+//  (c) sequential RNG-IP selection: candidate c is the pivot, each live selected s is
+//      evaluated against it by one wave; norm[c] < <c,s> rejects c, norm[s] < <c,s>
+//      tombstones s; (d) c carries the keyword flag when every live s it met has a
+//      BM25 term that u holds and c lacks; (e) first `d` live selected go to the
+//      forward row, flagged live ones beyond become keyword-edge candidates.
+__global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float dense_mul, const float* __restrict__ norms, uint32_t K,
+                                                           const uint32_t* __restrict__ ids, const float* __restrict__ dist, uint32_t d,
+                                                           uint32_t* fwd, uint32_t* det_out, uint32_t* cnt_out, uint32_t* kw_out,
+                                                           uint32_t term_slots, uint32_t uset_slots, uint32_t map_slots) {
+    extern __shared__ __align__(16) char smem[];
+    const PruneLds L(term_slots, uset_slots, map_slots, K);
+    uint2* tab = reinterpret_cast<uint2*>(smem + L.tab);
+    uint2* idmap = reinterpret_cast<uint2*>(smem + L.idmap);
+    uint32_t* uset = reinterpret_cast<uint32_t*>(smem + L.uset);
+    uint32_t* nb_id = reinterpret_cast<uint32_t*>(smem + L.nb_id);
+    float* nb_dist = reinterpret_cast<float*>(smem + L.nb_dist);
+    uint32_t* det = reinterpret_cast<uint32_t*>(smem + L.det);
+    uint32_t* cid = reinterpret_cast<uint32_t*>(smem + L.cid);
+    uint32_t* cdet = reinterpret_cast<uint32_t*>(smem + L.cdet);
+    uint32_t* sel_id = reinterpret_cast<uint32_t*>(smem + L.sel_id);
+    uint32_t* sel_det = reinterpret_cast<uint32_t*>(smem + L.sel_det);
+    volatile uint32_t* sel_live = reinterpret_cast<volatile uint32_t*>(smem + L.sel_live);
+    uint32_t* sel_kw = reinterpret_cast<uint32_t*>(smem + L.sel_kw);
+    uint32_t* o_fwd = reinterpret_cast<uint32_t*>(smem + L.o_fwd);
+    uint32_t* o_det = reinterpret_cast<uint32_t*>(smem + L.o_det);
+    uint32_t* o_kw = reinterpret_cast<uint32_t*>(smem + L.o_kw);
+    volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
+
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const uint32_t u = blockIdx.x, tmask = term_slots - 1, umask = uset_slots - 1, mmask = map_slots - 1;
+    const size_t base = (size_t)u * K;
+    const uint64_t lane_lt = (1ull << lane) - 1;
+
+    for (uint32_t i = tid; i < map_slots; i += PR_THREADS) idmap[i] = make_uint2(EMPTY, 0u);
+    for (uint32_t i = tid; i < uset_slots; i += PR_THREADS) uset[i] = EMPTY;
+    for (uint32_t i = tid; i < K; i += PR_THREADS) det[i] = 0;
+    if (tid < 16) ctl[tid] = 0;
+    __syncthreads();
+
+    // valid list entries, in list order
+    if (wave == 0) {
+        uint32_t m = 0;
+        for (uint32_t b0 = 0; b0 < K; b0 += WAVE) {
+            const uint32_t v = ids[base + b0 + lane] & ~FLAG;
+            const float dv = dist[base + b0 + lane];
+            const bool ok = dv < INF_DIS && v < C.n && v != u;
+            const uint64_t b = __ballot(ok);
+            if (ok) {
+                const uint32_t pos = m + __popcll(b & lane_lt);
+                nb_id[pos] = v;
+                nb_dist[pos] = dv;
+            }
+            m += __popcll(b);
+        }
+        if (lane == 0) ctl[PC_M] = m;
+    }
+    {   // u's BM25 terms
+        const uint64_t du = C.desc[u];
+        const uint2* sp = reinterpret_cast<const uint2*>(C.recs + desc_off(du) * 16 + DENSE_BYTES);
+        const uint32_t ns = desc_nnz_s(du), nb = desc_nnz_b(du);
+        for (uint32_t j = tid; j < nb; j += PR_THREADS) {
+            const uint32_t key = sp[ns + j].x;
+            uint32_t h = term_hash(key, umask);
+            while (true) {
+                const uint32_t old = atomicCAS(&uset[h], EMPTY, key);
+                if (old == EMPTY || old == key) break;
+                h = (h + 1) & umask;
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t m = ctl[PC_M];
+
+    // (a) detour counts
+    for (uint32_t i = tid; i < m; i += PR_THREADS) {
+        const uint32_t key = nb_id[i];
+        uint32_t h = term_hash(key, mmask);
+        while (true) {
+            const uint32_t old = atomicCAS(&idmap[h].x, EMPTY, key);
+            if (old == EMPTY) { idmap[h].y = i; break; }
+            if (old == key) break;
+            h = (h + 1) & mmask;
+        }
+    }
+    __syncthreads();
+    for (uint32_t t = tid; t < m * K; t += PR_THREADS) {
+        const uint32_t r = t / K, j = t % K;
+        const size_t at = (size_t)nb_id[r] * K + j;
+        const uint32_t x = ids[at] & ~FLAG;
+        const float dx = dist[at];
+        uint32_t h = term_hash(x, mmask);
+        while (true) {
+            const uint2 e = idmap[h];
+            if (e.x == x) {
+                if (e.y > r && dx < nb_dist[e.y]) atomicAdd(&det[e.y], 1u);
+                break;
+            }
+            if (e.x == EMPTY) break;
+            h = (h + 1) & mmask;
+        }
+    }
+    __syncthreads();
+    // (b) stable order by detour count
+    for (uint32_t i = tid; i < m; i += PR_THREADS) {
+        const uint32_t key = (det[i] << 16) | i;
+        uint32_t r = 0;
+        for (uint32_t j = 0; j < m; j++) r += ((det[j] << 16) | j) < key;
+        cid[r] = nb_id[i];
+        cdet[r] = det[i];
+    }
+    if (tid == 0 && m > 0) ctl[PC_ALLFLAG] = 1;
+    __syncthreads();
+    if (tid == 0 && m > 0) {
+        sel_id[0] = cid[0];
+        sel_det[0] = cdet[0];
+        sel_live[0] = 1;
+        sel_kw[0] = 0;
+        ctl[PC_NSEL] = 1;
+    }
+    __syncthreads();
+
+    // (c)+(d) sequential selection
+    for (uint32_t t = 1; t < m; t++) {
+        const uint32_t c = cid[t];
+        term_table_clear(tab, term_slots, tid, PR_THREADS);
+        __syncthreads();
+        const uint64_t dc = C.desc[c];
+        const char* rec = C.recs + desc_off(dc) * 16;
+        PivotDense pv;
+        pivot_dense_load(pv, reinterpret_cast<const float*>(rec), 1.0f);
+        pivot_terms_from_record(tab, tmask, rec, desc_nnz_s(dc) + desc_nnz_b(dc), tid, PR_THREADS);
+        __syncthreads();
+        const uint32_t n_sel = ctl[PC_NSEL];
+        const float norm_c = norms[c];
+        for (uint32_t i = wave; i < n_sel; i += PR_THREADS / WAVE) {
+            if (!sel_live[i]) continue;
+            const uint32_t s = uniform(sel_id[i]);
+            bool kwf = false;
+            EvalOut e = eval_wave<true>(C, s, pv, tab, tmask, ALL_PATHS, dense_mul, uset, umask, &kwf);
+            if (lane == 0) {
+                if (norm_c < e.ip) ctl[PC_REJECT] = 1;
+                if (norms[s] < e.ip) sel_live[i] = 0;
+                if (!kwf) ctl[PC_ALLFLAG] = 0;
+            }
+        }
+        __syncthreads();
+        if (tid == 0) {
+            if (!ctl[PC_REJECT]) {
+                sel_id[n_sel] = c;
+                sel_det[n_sel] = cdet[t];
+                sel_live[n_sel] = 1;
+                sel_kw[n_sel] = ctl[PC_ALLFLAG];
+                ctl[PC_NSEL] = n_sel + 1;
+            }
+            ctl[PC_REJECT] = 0;
+            ctl[PC_ALLFLAG] = 1;
+        }
+        __syncthreads();
+    }
+
+    // (e) emit
+    if (tid == 0) {
+        const uint32_t n_sel = ctl[PC_NSEL];
+        uint32_t cnt = 0, nkw = 0;
+        for (uint32_t i = 0; i < n_sel; i++) {
+            if (!sel_live[i]) continue;
+            if (cnt < d) { o_fwd[cnt] = sel_id[i]; o_det[cnt] = sel_det[i]; cnt++; }
+            else if (sel_kw[i] && nkw < APOE_KW_CAND) { o_kw[1 + nkw] = sel_id[i]; nkw++; }
+        }
+        for (uint32_t t = 0; t < m && cnt < d; t++) {
+            const uint32_t c = cid[t];
+            bool present = false;
+            for (uint32_t j = 0; j < cnt; j++) present |= o_fwd[j] == c;
+            if (!present) { o_fwd[cnt] = c; o_det[cnt] = cdet[t]; cnt++; }
+        }
+        ctl[PC_CNT] = cnt;
+        for (; cnt < d; cnt++) { o_fwd[cnt] = u; o_det[cnt] = EMPTY; }
+        o_kw[0] = nkw;
+        for (uint32_t j = nkw; j < APOE_KW_CAND; j++) o_kw[1 + j] = 0;
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < d; i += PR_THREADS) {
+        fwd[(size_t)u * d + i] = o_fwd[i];
+        det_out[(size_t)u * d + i] = o_det[i];
+    }
+    for (uint32_t i = tid; i < 1 + APOE_KW_CAND; i += PR_THREADS) kw_out[(size_t)u * (1 + APOE_KW_CAND) + i] = o_kw[i];
+    if (tid == 0) cnt_out[u] = ctl[PC_CNT];
+}
+
+// ---- final rows (index.cu:717-807) ----
+
+__global__ __launch_bounds__(256) void indegree_kernel(uint32_t n, uint32_t d, const uint32_t* __restrict__ fwd, const uint32_t* __restrict__ cnt,
+                                                       uint32_t* indeg) {
+    const uint64_t total = (uint64_t)n * d;
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t u = (uint32_t)(t / d), j = (uint32_t)(t % d);
+        if (j >= cnt[u]) continue;
+        const uint32_t v = fwd[t];
+        if (v < n && v != u) atomicAdd(&indeg[v], 1u);
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_in_edges_kernel(uint32_t n, uint32_t d, const uint32_t* __restrict__ fwd,
+                                                            const uint32_t* __restrict__ det, const uint32_t* __restrict__ cnt,
+                                                            const uint32_t* __restrict__ in_off, uint32_t* cursor, uint64_t* in_edges) {
+    const uint64_t total = (uint64_t)n * d;
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t u = (uint32_t)(t / d), j = (uint32_t)(t % d);
+        if (j >= cnt[u]) continue;
+        const uint32_t v = fwd[t];
+        if (v < n && v != u) in_edges[in_off[v] + atomicAdd(&cursor[v], 1u)] = ((uint64_t)det[t] << 32) | u;
+    }
+}
+
+__device__ __forceinline__ uint64_t wave_min64(uint64_t v) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) {
+        const uint64_t other = shfl_xor64(v, o);
+        v = other < v ? other : v;
+    }
+    return v;
+}
+
+// One wave per node v. Row = first half of v's forward list, then up to d/2 reverse
+// neighbours in (detour, id) order that are not in the first half, topped up from the
+// second half of the forward list and finally with v itself; then the keyword slots.
+__global__ __launch_bounds__(256) void final_rows_kernel(uint32_t n, uint32_t d, const uint32_t* __restrict__ fwd, const uint32_t* __restrict__ kw,
+                                                         const uint32_t* __restrict__ in_off, const uint64_t* __restrict__ in_edges,
+                                                         uint32_t* rows) {
+    __shared__ uint32_t s_row[4][WAVE + APOE_KW_SLOTS];
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const uint32_t v = blockIdx.x * 4 + wave;
+    if (v >= n) return;
+    uint32_t* row = s_row[wave];
+    const uint32_t W = d + APOE_KW_SLOTS, h = d / 2;
+    const uint32_t* fw = fwd + (size_t)v * d;
+    if ((uint32_t)lane < h) row[lane] = fw[lane];
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    uint32_t fill = h;
+    const uint32_t e0 = in_off[v], e1 = in_off[v + 1];
+    uint64_t last = 0;
+    bool first = true;
+    while (fill < 2 * h) {
+        // smallest key above the last one taken whose node is not in the first half
+        uint64_t best = ~0ull;
+        for (uint32_t e = e0 + lane; e < e1; e += WAVE) {
+            const uint64_t k = in_edges[e];
+            if (!first && k <= last) continue;
+            const uint32_t uu = (uint32_t)k;
+            bool present = false;
+            for (uint32_t j = 0; j < h; j++) present |= row[j] == uu;
+            if (!present && k < best) best = k;
+        }
+        best = wave_min64(best);
+        if (best == ~0ull) break;
+        if (lane == 0) row[fill] = (uint32_t)best;
+        fill++;
+        last = best;
+        first = false;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (uint32_t j = h; j < d && fill < d; j++) {
+        const uint32_t c = fw[j];
+        bool present = false;
+        for (uint32_t t = lane; t < fill; t += WAVE) present |= row[t] == c;
+        if (!__any(present)) {
+            if (lane == 0) row[fill] = c;
+            fill++;
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+    for (uint32_t j = fill + lane; j < d; j += WAVE) row[j] = v;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    // keyword edges
+    const uint32_t* kv = kw + (size_t)v * (1 + APOE_KW_CAND);
+    const uint32_t nk = min(kv[0], (uint32_t)APOE_KW_CAND);
+    if (lane < APOE_KW_SLOTS) row[d + lane] = 0;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    uint32_t c = 0;
+    for (uint32_t j = 0; j < nk && c < APOE_KW_SLOTS - 1; j++) {
+        const uint32_t x = kv[1 + j];
+        bool present = false;
+        for (uint32_t t = h + lane; t < d; t += WAVE) present |= row[t] == x;
+        if (!__any(present)) {
+            if (lane == 0) row[d + 1 + c] = x;
+            c++;
+        }
+    }
+    if (lane == 0) row[d] = c;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (uint32_t j = lane; j < W; j += WAVE) rows[(size_t)v * W + j] = row[j];
+}
+
+static uint32_t doc_term_slots(const apoe_corpus* c) { return next_pow2(std::max(64u, 2 * (c->max_nnz_s + c->max_nnz_b))); }
+
+int launch_prune(apoe_knn* g, uint32_t degree) {
+    apoe_ctx* ctx = g->ctx;
+    const uint32_t term_slots = doc_term_slots(g->corpus);
+    const uint32_t uset_slots = next_pow2(std::max(64u, 2 * g->corpus->max_nnz_b));
+    const uint32_t map_slots = next_pow2(4 * g->K);
+    const PruneLds L(term_slots, uset_slots, map_slots, g->K);
+    APOE_REQUIRE(L.total <= 64 * 1024, "prune needs %u bytes of LDS (rows with up to %u sparse terms)", L.total,
+                 g->corpus->max_nnz_s + g->corpus->max_nnz_b);
+    APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&prune_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
+    prune_kernel<<<g->n, PR_THREADS, L.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->norms.p, g->K, g->ids.p,
+                                                             g->dist.p, degree, g->fwd.p, g->det.p, g->cnt.p, g->kw.p, term_slots, uset_slots,
+                                                             map_slots);
+    APOE_HIP(hipGetLastError());
+    return APOE_OK;
+}
+
+int launch_final_graph(apoe_knn* g, uint32_t* rows_dev) {
+    apoe_ctx* ctx = g->ctx;
+    const uint32_t n = g->n, d = g->degree;
+    DevBuf<uint32_t> indeg, in_off, cursor;
+    DevBuf<uint64_t> in_edges;
+    DevBuf<char> temp;
+    APOE_TRY(indeg.alloc((size_t)n + 1));
+    APOE_TRY(in_off.alloc((size_t)n + 1));
+    APOE_TRY(cursor.alloc(n));
+    APOE_TRY(in_edges.alloc((size_t)n * d));
+    APOE_HIP(hipMemsetAsync(indeg.p, 0, ((size_t)n + 1) * sizeof(uint32_t), ctx->stream));
+    APOE_HIP(hipMemsetAsync(cursor.p, 0, (size_t)n * sizeof(uint32_t), ctx->stream));
+    const uint32_t grid = (uint32_t)std::min<uint64_t>(((uint64_t)n * d + 255) / 256, 1u << 20);
+    indegree_kernel<<<grid, 256, 0, ctx->stream>>>(n, d, g->fwd.p, g->cnt.p, indeg.p);
+    APOE_HIP(hipGetLastError());
+    size_t temp_bytes = 0;
+    APOE_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, temp_bytes, indeg.p, in_off.p, (int)(n + 1), ctx->stream));
+    APOE_TRY(temp.alloc(temp_bytes));
+    APOE_HIP(hipcub::DeviceScan::ExclusiveSum(temp.p, temp_bytes, indeg.p, in_off.p, (int)(n + 1), ctx->stream));
+    fill_in_edges_kernel<<<grid, 256, 0, ctx->stream>>>(n, d, g->fwd.p, g->det.p, g->cnt.p, in_off.p, cursor.p, in_edges.p);
+    APOE_HIP(hipGetLastError());
+    final_rows_kernel<<<(n + 3) / 4, 256, 0, ctx->stream>>>(n, d, g->fwd.p, g->kw.p, in_off.p, in_edges.p, rows_dev);
+    APOE_HIP(hipGetLastError());
+    APOE_HIP(hipStreamSynchronize(ctx->stream)); // temporaries are released on return
+    return APOE_OK;
+}
+
+} // namespace apoe
+
+using namespace apoe;
+
+extern "C" {
+
+int apoe_prune(apoe_knn* g, uint32_t degree) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_REQUIRE(degree >= 2 && degree <= 64 && degree % 2 == 0 && degree <= g->K, "degree must be even, in [2, 64] and <= K, got %u", degree);
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    g->degree = degree;
+    APOE_TRY(g->fwd.alloc((size_t)g->n * degree));
+    APOE_TRY(g->det.alloc((size_t)g->n * degree));
+    APOE_TRY(g->cnt.alloc(g->n));
+    APOE_TRY(g->kw.alloc((size_t)g->n * (1 + APOE_KW_CAND)));
+    float ms = 0.f;
+    APOE_TRY(timed(g->ctx, &ms, [&]() { return launch_prune(g, degree); }));
+    g->elapsed_ms += ms;
+    g->pruned = true;
+    return APOE_OK;
+}
+
+int apoe_prune_download(apoe_knn* g, uint32_t* fwd, uint32_t* det, uint32_t* cnt, uint32_t* kw) {
+    APOE_REQUIRE(g, "null argument");
+    if (!g->pruned) {
+        set_error("apoe_prune has not run on this handle");
+        return APOE_ERR_STATE;
+    }
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    if (fwd) APOE_TRY(copy_out(g->ctx, fwd, g->fwd.p, g->fwd.bytes()));
+    if (det) APOE_TRY(copy_out(g->ctx, det, g->det.p, g->det.bytes()));
+    if (cnt) APOE_TRY(copy_out(g->ctx, cnt, g->cnt.p, (size_t)g->n * sizeof(uint32_t)));
+    if (kw) APOE_TRY(copy_out(g->ctx, kw, g->kw.p, g->kw.bytes()));
+    return APOE_OK;
+}
+
+int apoe_finalize_graph(apoe_knn* g, apoe_graph** out) {
+    APOE_REQUIRE(g && out, "null argument");
+    *out = nullptr;
+    if (!g->pruned) {
+        set_error("apoe_prune has not run on this handle");
+        return APOE_ERR_STATE;
+    }
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    std::unique_ptr<apoe_graph> gr(new apoe_graph());
+    gr->ctx = g->ctx;
+    gr->n = g->n;
+    gr->width = g->degree + APOE_KW_SLOTS;
+    gr->n_entry = g->degree;
+    APOE_TRY(gr->rows.alloc((size_t)gr->n * gr->width));
+    APOE_TRY(gr->entry.alloc(gr->n_entry));
+    float ms = 0.f;
+    APOE_TRY(timed(g->ctx, &ms, [&]() { return launch_final_graph(g, gr->rows.p); }));
+    g->elapsed_ms += ms;
+    // entry points: the `degree` documents of smallest hybrid norm, ties by id (index.cu:916-925)
+    std::vector<float> nrm(g->n);
+    APOE_TRY(copy_out(g->ctx, nrm.data(), g->norms.p, (size_t)g->n * sizeof(float)));
+    std::vector<std::pair<float, uint32_t>> dp(g->n);
+    for (uint32_t i = 0; i < g->n; i++) dp[i] = {nrm[i], i};
+    const uint32_t k = std::min(gr->n_entry, g->n);
+    std::partial_sort(dp.begin(), dp.begin() + k, dp.end());
+    std::vector<uint32_t> ep(gr->n_entry);
+    for (uint32_t i = 0; i < gr->n_entry; i++) ep[i] = dp[i % k].second;
+    APOE_TRY(copy_in(g->ctx, gr->entry.p, ep.data(), ep.size() * sizeof(uint32_t)));
+    *out = gr.release();
+    return APOE_OK;
+}
+
+} // extern "C"

@@ -98,6 +98,17 @@ int apoe_hybrid_distance_pairs(apoe_ctx* ctx, const apoe_corpus* c, float dense_
 /* Hybrid squared norms (cal_power, index.cu:483-534). out has n floats. */
 int apoe_norms(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale, float* out);
 
+/*
+ * Query-time weight calibration (query.cu:1847-1869): the largest per-path inner
+ * product over the first min(n,100) documents x first min(n_queries,100) queries is
+ * taken for each path; the two paths with the smaller maxima have their weights
+ * multiplied by max_largest / max_path. w3 = {dense, splade, bm25}, updated in place.
+ * Nothing changes on a tie for the largest; a path whose maximum is not positive
+ * keeps its weight (the reference divides by it).
+ */
+int apoe_calibrate_weights(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q,
+                           uint32_t n_queries, float* w3);
+
 /* ---- index construction (build_index_impl, index.cu:889-903) ---- */
 
 /* kNN-graph state: ids/dist [n][K], reverse lists, norms. K is 64 or 128 (index.cu:6). */

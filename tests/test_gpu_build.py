@@ -99,3 +99,110 @@ def test_nnd_recall_close_to_oracle(small_world, gpu_knn, exact_knn):
 def test_merge_reverse_only_improves(gpu_knn):
     (b_ids, b_dist), (a_ids, a_dist) = gpu_knn["before"], gpu_knn["after"]
     assert np.all(a_dist <= b_dist + 0.0)
+
+
+# ---------------------------------------------------------------- prune + final rows
+
+
+@pytest.fixture(scope="module")
+def pruned(gpu_world):
+    """GPU prune and CPU prune of the SAME kNN graph (the oracle's)."""
+    import apoe
+    import oracle as O
+    w = gpu_world
+    knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+    knn.upload(w["knn_ids"], w["knn_dist"])
+    knn.prune(32)
+    gpu = knn.prune_download()
+    graph = knn.finalize()
+    rows, entry = graph.download()
+    nrm = O.norms(w["C"], 7.0)
+    cpu = O.prune(w["C"], 7.0, nrm, w["knn_ids"], w["knn_dist"], 32)
+    yield dict(gpu=gpu, cpu=cpu, rows=rows, entry=entry, norms=nrm, graph=graph)
+    graph.close()
+    knn.close()
+
+
+def test_prune_matches_oracle(pruned):
+    """Integer outputs are identical except where a float comparison norm < <c,s> sits
+    within rounding of equality; allow a handful of such rows."""
+    (g_fwd, g_det, g_cnt, g_kw), (c_fwd, c_det, c_cnt, c_kw) = pruned["gpu"], pruned["cpu"]
+    same_rows = np.all(g_fwd == c_fwd, axis=1)
+    print(f"identical forward rows: {same_rows.mean():.5f}")
+    assert same_rows.mean() >= 0.995
+    ok = same_rows
+    assert np.array_equal(g_det[ok], c_det[ok])
+    assert np.array_equal(g_cnt[ok], c_cnt[ok])
+    same_kw = np.all(g_kw == c_kw, axis=1)
+    assert same_kw[ok].mean() >= 0.995
+
+
+def test_prune_invariants(gpu_world, pruned):
+    import oracle as O
+    w = gpu_world
+    fwd, det, cnt, kw = pruned["gpu"]
+    n, d = fwd.shape
+    assert np.all(cnt <= d) and np.all(kw[:, 0] <= 32)
+    assert fwd.max() < n
+    for u in range(0, n, 37):
+        real = fwd[u, :cnt[u]]
+        assert u not in real.tolist() and len(set(real.tolist())) == len(real)
+        assert set(real.tolist()) <= set(w["knn_ids"][u].tolist())
+        k = kw[u, 0]
+        assert set(kw[u, 1:1 + k].tolist()) <= set(w["knn_ids"][u].tolist())
+        assert not (set(kw[u, 1:1 + k].tolist()) & set(real.tolist()))
+    # detour counts against the O(K^2) definition on a few nodes
+    ids, dist = w["knn_ids"], w["knn_dist"]
+    for u in (0, 5, 1234, n - 1):
+        want = {}
+        for s in range(64):
+            c = 0
+            for r in range(s):
+                lr = ids[ids[u, r]].tolist()
+                if ids[u, s] in lr and dist[ids[u, r], lr.index(ids[u, s])] < dist[u, s]:
+                    c += 1
+            want[int(ids[u, s])] = c
+        for j in range(cnt[u]):
+            assert det[u, j] == want[int(fwd[u, j])]
+
+
+def test_final_rows_match_oracle(pruned):
+    import oracle as O
+    fwd, det, cnt, kw = pruned["gpu"]
+    want = O.final_graph(fwd, det, cnt, kw)  # same prune output in, rows must be identical
+    assert np.array_equal(pruned["rows"], want)
+    n, d = fwd.shape
+    rows = pruned["rows"]
+    assert rows.shape == (n, d + 8)
+    assert np.all(rows[:, d] <= 7)
+    assert np.array_equal(rows[:, :d // 2], fwd[:, :d // 2])
+    for v in range(0, n, 41):
+        c = rows[v, d]
+        assert np.all(rows[v, d + 1 + c:] == 0)
+        assert not (set(rows[v, d + 1:d + 1 + c].tolist()) & set(rows[v, d // 2:d].tolist()))
+        body = [x for x in rows[v, :d].tolist() if x != v]
+        assert len(set(body)) == len(body)
+
+
+def test_entry_points_match_oracle(pruned):
+    import oracle as O
+    assert np.array_equal(pruned["entry"], O.entry_points(pruned["norms"], 32))
+
+
+def test_gpu_built_index_recall(gpu_world):
+    """Whole GPU build; recall@10 of search on it within 0.5 points of the oracle-built index."""
+    import apoe
+    import oracle as O
+    from parity import recall_at_k
+    w = gpu_world
+    graph, ms = apoe.build_graph(w["ctx"], w["gc"], K=64, iters=8, degree=32, dense_scale=7.0, seed=5)
+    w3 = (1.0, 1.0, 1.0)
+    truth, _ = O.bruteforce_topk(w["C"], w["Q"], w3, 10)
+    ids_g, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], graph, w3, 128)
+    ids_c, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], w3, 128)
+    r_g, r_c = recall_at_k(ids_g, truth, 10), recall_at_k(ids_c, truth, 10)
+    print(f"recall@10 cands=128: gpu-built {r_g:.4f}, oracle-built {r_c:.4f}, gpu build {ms:.1f} ms")
+    assert r_g >= r_c - 0.005
+    rows, entry = graph.download()
+    assert rows.shape == (w["C"].n, 40) and len(entry) == 32
+    graph.close()
