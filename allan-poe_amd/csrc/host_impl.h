@@ -1,0 +1,59 @@
+// Host drivers of the hybrid_search module (see host_impl.cpp).
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace hs {
+
+struct Csr {
+    std::vector<unsigned> off, idx;
+    std::vector<float> val;
+};
+
+// Knobs that the reference hard-wires; the defaults are the reference's constants.
+struct BuildOptions {
+    unsigned degree = 32;           // index.cu:888
+    unsigned nnd_k = 64;            // index.cu:6
+    unsigned nnd_iters = 25;        // index.cu:884
+    float dense_build_scale = 7.0f; // index.cu:836-840
+    uint64_t seed = 20251125;       // the reference seeds from clock(), index.cu:102
+    int device = 0;
+};
+
+struct SearchOptions {
+    unsigned max_queries = 100; // query.cu:1825
+    bool calibrate = true;      // query.cu:1847-1869
+    int device = 0;
+};
+
+struct SearchResult {
+    unsigned query_num = 0, cands = 0;
+    std::vector<unsigned> ids; // [query_num][cands]
+    std::vector<float> dist;   // [query_num][cands]
+    float weights[3] = {0, 0, 0}; // effective dense, sparse, bm25
+    float kernel_ms = 0;
+    double ndcg = 0, recall = 0;
+    uint64_t evaluations = 0, expansions = 0, algo_bytes = 0;
+};
+
+void load_fvecs(const std::string& path, std::vector<float>& data, unsigned& num, unsigned& dim);
+void load_sparse(const std::string& path, unsigned rows, Csr& out);
+void load_kg(const std::string& path, std::vector<unsigned>& off, std::vector<unsigned>& idx, unsigned& num);
+void load_txt(const std::string& path, std::vector<std::vector<unsigned>>& results, unsigned query_num);
+void write_graph(const std::string& path, const std::vector<unsigned>& rows, unsigned n, unsigned width, const std::vector<unsigned>& entry);
+void load_graph(const std::string& path, std::vector<unsigned>& rows, std::vector<unsigned>& entry, unsigned& width, unsigned& num);
+double ndcg_at_k(const std::vector<std::vector<unsigned>>& res, std::vector<std::vector<unsigned>> gt, double* recall);
+
+void build_index_impl(const std::string& dense_data_path, const std::string& sparse_data_path, const std::string& bm25_data_path,
+                      const std::string& output_graph_path, const BuildOptions& opt);
+
+SearchResult search_index_impl(const std::string& dense_data_path, const std::string& dense_query_path, const std::string& sparse_data_path,
+                               const std::string& sparse_query_path, const std::string& bm25_data_path, const std::string& bm25_query_path,
+                               const std::string& keyword_id_path, const std::string& knowledge_path, const std::string& entity2doc_path,
+                               const std::string& query_entity_path, const std::string& graph_path, const std::string& ground_truth_path,
+                               int top_k, int cands, float sparse_weight, float bm25_weight, float dense_weight, float kg_weight,
+                               const SearchOptions& opt);
+
+} // namespace hs

@@ -191,8 +191,9 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
         uint64_t st_exp = 0, st_eval = 0, st_ns = 0, st_nb = 0; // wave-uniform counters
         uint32_t cur = 0;                                        // live pool half (wave 0's copy is authoritative)
 
-        // ---- seeds: entry points (query.cu:440-485) ----
+        // ---- seeds ----
         if (!KG) {
+            // entry points (query.cu:440-485)
             if (wave == 0) {
                 uint32_t c = lane < (int)a.n_entry ? a.entry[lane] : EMPTY;
                 bool fresh = false;
@@ -204,8 +205,72 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
                 if (fresh) new_id[__popcll(b & lane_lt)] = c;
                 if (lane == 0) { ctl[CTL_NNEW] = __popcll(b); ctl[CTL_PARENT] = 0; }
             }
+            __syncthreads();
+        } else {
+            // documents of the query's entities first, entry points only if those do not
+            // fill the pool (query.cu:1577-1604); at most cands + degree seeds
+            if (wave == 0) {
+                const uint32_t seed_cap = cands + a.degree;
+                uint32_t n_seed = 0;
+                const uint32_t qe0 = uniform(a.q2e_off[q]), qe1 = uniform(a.q2e_off[q + 1]);
+                for (uint32_t i = qe0; i < qe1; i++) {
+                    const uint32_t e = uniform(a.q2e_idx[i]);
+                    if (e >= a.n_entities) continue;
+                    const uint32_t d0 = uniform(a.e2d_off[e]), d1 = uniform(a.e2d_off[e + 1]);
+                    for (uint32_t b0 = d0; b0 < d1; b0 += WAVE) {
+                        const uint32_t doc = b0 + lane < d1 ? a.e2d_idx[b0 + lane] : EMPTY;
+                        bool fresh = false;
+                        if (doc < a.C.n) {
+                            const uint32_t bit = 1u << (doc & 31);
+                            fresh = !(atomicOr(&bitmap[doc >> 5], bit) & bit);
+                        }
+                        const uint64_t b = __ballot(fresh);
+                        const uint32_t pos = n_seed + __popcll(b & lane_lt);
+                        if (fresh && pos < seed_cap) { seed_id[pos] = doc; seed_ent[pos] = e; }
+                        n_seed = min(seed_cap, n_seed + (uint32_t)__popcll(b));
+                    }
+                }
+                if (n_seed < cands) {
+                    const uint32_t c = lane < (int)a.n_entry ? a.entry[lane] : EMPTY;
+                    bool fresh = false;
+                    if (c < a.C.n) {
+                        const uint32_t bit = 1u << (c & 31);
+                        fresh = !(atomicOr(&bitmap[c >> 5], bit) & bit);
+                    }
+                    const uint64_t b = __ballot(fresh);
+                    const uint32_t pos = n_seed + __popcll(b & lane_lt);
+                    if (fresh && pos < seed_cap) { seed_id[pos] = c; seed_ent[pos] = EMPTY; }
+                    n_seed = min(seed_cap, n_seed + (uint32_t)__popcll(b));
+                }
+                if (lane == 0) ctl[CTL_NSEED] = n_seed;
+            }
+            __syncthreads();
+            const uint32_t n_seed = ctl[CTL_NSEED];
+            for (uint32_t j = wave; j < n_seed; j += NW) {
+                const uint32_t id = uniform(seed_id[j]);
+                EvalOut e = eval_wave(a.C, id, pv, tab, mask, a.paths, 1.0f);
+                st_eval++;
+                st_ns += e.nnz_s;
+                st_nb += e.nnz_b;
+                if (lane == 0) seed_dist[j] = 1.0f - e.ip - (seed_ent[j] != EMPTY ? a.kg_weight : 0.0f); // query.cu:1637-1638
+            }
+            __syncthreads();
+            if (wave == 0) {
+                for (uint32_t b0 = 0; b0 < n_seed; b0 += WAVE) {
+                    const uint32_t nb = min((uint32_t)WAVE, n_seed - b0);
+                    if (lane < (int)nb) {
+                        new_id[lane] = seed_id[b0 + lane];
+                        new_dist[lane] = seed_dist[b0 + lane];
+                        new_ent[lane] = seed_ent[b0 + lane];
+                        new_hop[lane] = 0;
+                    }
+                    wave_fence();
+                    cur = sort_merge<KG>(P, cur, new_id, new_dist, new_ent, new_hop, nb);
+                }
+                if (lane == 0) { ctl[CTL_NNEW] = 0; ctl[CTL_PARENT] = 0; ctl[CTL_CUR] = cur; }
+            }
+            __syncthreads();
         }
-        __syncthreads();
 
         for (uint32_t it = 0; it <= a.max_iter; it++) {
             // ---- evaluate the fresh candidates: one wave per candidate ----
@@ -217,7 +282,11 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
                 st_eval++;
                 st_ns += e.nnz_s;
                 st_nb += e.nnz_b;
-                if (lane == 0) new_dist[j] = 1.0f - e.ip;
+                float dist = 1.0f - e.ip;
+                if (KG) {
+                    if (new_ent[j] != EMPTY) dist -= a.kg_weight / (float)new_hop[j]; // query.cu:1759-1760
+                }
+                if (lane == 0) new_dist[j] = dist;
             }
             __syncthreads();
             // ---- wave 0: merge, pick the next parent, fetch its neighbours ----
@@ -238,6 +307,8 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
                     }
                 }
                 if (parent != EMPTY) {
+                    uint32_t p_ent = EMPTY, p_hop = 0;
+                    if (KG) { p_ent = P.ent[cur * cands + slot]; p_hop = P.hop[cur * cands + slot]; }
                     if (lane == 0) P.id[cur * cands + slot] = parent | FLAG;
                     st_exp++;
                     uint32_t c = lane < (int)a.degree ? a.graph[(size_t)parent * a.W + lane] : EMPTY;
@@ -246,8 +317,87 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
                         const uint32_t bit = 1u << (c & 31);
                         fresh = !(atomicOr(&bitmap[c >> 5], bit) & bit);
                     }
-                    const uint64_t b = __ballot(fresh);
-                    if (fresh) new_id[__popcll(b & lane_lt)] = c;
+                    bool alive = fresh;
+                    uint32_t ent = EMPTY;
+                    if (KG) {
+                        // logical edges: parent's entity -> neighbour entity -> document
+                        if (p_hop < 3 && p_ent < a.n_entities) {
+                            uint32_t* slot_id = seed_id; // scratch, free after seeding
+                            uint32_t* prop = seed_ent;
+                            const uint32_t e0 = uniform(a.e2e_off[p_ent]), e1 = uniform(a.e2e_off[p_ent + 1]);
+                            slot_id[lane] = fresh ? c : EMPTY;
+                            link[lane] = EMPTY;
+                            wave_fence();
+                            // (i) a fresh graph neighbour that is also a logical neighbour is
+                            //     tagged with the first linking entity (query.cu:1699-1715)
+                            for (uint32_t jb = e0; jb < e1; jb += WAVE) {
+                                const uint32_t j = jb + lane;
+                                if (j < e1) {
+                                    const uint32_t e2 = a.e2e_idx[j];
+                                    if (e2 < a.n_entities) {
+                                        for (uint32_t k = a.e2d_off[e2]; k < a.e2d_off[e2 + 1]; k++) {
+                                            const uint32_t doc = a.e2d_idx[k];
+                                            for (uint32_t t = 0; t < a.degree; t++)
+                                                if (slot_id[t] == doc) atomicMin(&link[t], j - e0);
+                                        }
+                                    }
+                                }
+                            }
+                            wave_fence();
+                            if (fresh && link[lane] != EMPTY) ent = a.e2e_idx[e0 + link[lane]];
+                            // (ii) slots whose graph neighbour was already visited (or invalid) are
+                            //      recycled: the t-th such slot takes the first unvisited document
+                            //      of the t-th neighbour entity (query.cu:1718-1735). A document
+                            //      claimed by several slots in one round goes to the lowest slot;
+                            //      the others move on to their next document.
+                            const bool recyc = lane < (int)a.degree && !fresh;
+                            const uint64_t rb = __ballot(recyc);
+                            const uint32_t t = __popcll(rb & lane_lt);
+                            bool unresolved = recyc && t < e1 - e0;
+                            uint32_t e2 = EMPTY, k = 0, k1 = 0;
+                            if (unresolved) {
+                                e2 = a.e2e_idx[e0 + t];
+                                if (e2 < a.n_entities) { k = a.e2d_off[e2]; k1 = a.e2d_off[e2 + 1]; }
+                                else unresolved = false;
+                            }
+                            while (__any(unresolved)) {
+                                uint32_t doc = EMPTY;
+                                if (unresolved) {
+                                    while (k < k1) {
+                                        const uint32_t x = a.e2d_idx[k];
+                                        if (x != parent && x < a.C.n) {
+                                            const uint32_t word = __hip_atomic_load(&bitmap[x >> 5], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                            if (!(word & (1u << (x & 31)))) { doc = x; break; }
+                                        }
+                                        k++;
+                                    }
+                                    if (doc == EMPTY) unresolved = false;
+                                }
+                                prop[lane] = doc;
+                                wave_fence();
+                                if (unresolved) {
+                                    bool lose = false;
+                                    for (int l = 0; l < lane; l++) lose |= prop[l] == doc;
+                                    if (lose) k++;
+                                    else {
+                                        atomicOr(&bitmap[doc >> 5], 1u << (doc & 31));
+                                        c = doc;
+                                        ent = e2;
+                                        alive = true;
+                                        unresolved = false;
+                                    }
+                                }
+                                wave_fence();
+                                __threadfence();
+                            }
+                        }
+                    }
+                    const uint64_t b = __ballot(alive);
+                    if (alive) {
+                        const uint32_t pos = __popcll(b & lane_lt);
+                        new_id[pos] = c;
+                        if (KG) { new_ent[pos] = ent; new_hop[pos] = p_hop + 1; }
+                    }
                     n_next = __popcll(b);
                 }
                 if (lane == 0) { ctl[CTL_PARENT] = parent; ctl[CTL_NNEW] = n_next; ctl[CTL_CUR] = cur; }
@@ -279,11 +429,10 @@ static int launch_variant(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, siz
 
 int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g, const apoe_kg* kg,
                   const apoe_search_params* p, uint32_t* out_ids_dev, float* out_dist_dev, apoe_search_stats* stats) {
-    APOE_REQUIRE(p->cands >= 1 && p->cands <= 512, "cands must be in 1..512, got %u", p->cands);
+    APOE_REQUIRE(p->cands >= 1 && p->cands <= APOE_MAX_CANDS, "cands must be in 1..%d, got %u", APOE_MAX_CANDS, p->cands);
     APOE_REQUIRE(g->width > APOE_KW_SLOTS && g->width - APOE_KW_SLOTS <= MAX_NEW, "graph degree must be in 1..64, got width %u", g->width);
     APOE_REQUIRE(g->n == c->n, "graph has %u nodes but the corpus has %u documents", g->n, c->n);
     APOE_REQUIRE(p->q_begin <= q->n, "q_begin %u beyond %u queries", p->q_begin, q->n);
-    APOE_REQUIRE(kg == nullptr, "knowledge-graph search is not available in this build");
     const uint32_t q_count = p->q_count ? p->q_count : q->n - p->q_begin;
     APOE_REQUIRE(p->q_begin + q_count <= q->n, "query range [%u,%u) beyond %u queries", p->q_begin, p->q_begin + q_count, q->n);
     if (stats) *stats = apoe_search_stats{};
@@ -310,19 +459,36 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     a.slots = next_pow2(std::max(64u, 2 * q->max_nnz));
     a.kg_weight = p->kg_weight;
 
-    const bool use_kg = false;
+    const bool use_kg = kg != nullptr;
+    if (use_kg) {
+        APOE_REQUIRE(kg->n_queries >= p->q_begin + q_count, "knowledge graph holds entities for %u queries, %u needed", kg->n_queries, p->q_begin + q_count);
+        a.e2e_off = kg->e2e_off.p;
+        a.e2e_idx = kg->e2e_idx.p;
+        a.e2d_off = kg->e2d_off.p;
+        a.e2d_idx = kg->e2d_idx.p;
+        a.q2e_off = kg->q2e_off.p;
+        a.q2e_idx = kg->q2e_idx.p;
+        a.n_entities = kg->n_entities;
+    }
     const SearchLds L(a.slots, a.cands, use_kg);
     APOE_REQUIRE(L.total <= 64 * 1024, "search needs %u bytes of LDS (query rows with up to %u sparse terms)", L.total, q->max_nnz);
 
-    int nw = 4;
+    // variant 0: two waves per query (the measured best); 1, 2, 3: one, four, eight waves
+    int nw = 2;
     if (p->variant == 1) nw = 1;
-    else if (p->variant == 2) nw = 2;
+    else if (p->variant == 2) nw = 4;
     else if (p->variant == 3) nw = 8;
-    // resident workgroups: bounded by LDS, by waves per CU, and by the number of queries
-    const uint32_t per_cu_lds = (uint32_t)((160 * 1024) / std::max<uint32_t>(L.total, 1));
-    const uint32_t per_cu_waves = 32u / nw; // up to 8 waves per SIMD; keep half for register headroom
-    const uint32_t per_cu = std::max(1u, std::min(per_cu_lds, per_cu_waves));
-    const uint32_t grid = std::min<uint32_t>(q_count, per_cu * (uint32_t)ctx->num_cus);
+    // persistent grid: as many workgroups as can be resident, never more than queries
+    int per_cu = 1;
+    {
+        const void* fn = nullptr;
+        if (use_kg) fn = nw == 1 ? (const void*)&search_kernel<1, true> : nw == 2 ? (const void*)&search_kernel<2, true> : nw == 8 ? (const void*)&search_kernel<8, true> : (const void*)&search_kernel<4, true>;
+        else fn = nw == 1 ? (const void*)&search_kernel<1, false> : nw == 2 ? (const void*)&search_kernel<2, false> : nw == 8 ? (const void*)&search_kernel<8, false> : (const void*)&search_kernel<4, false>;
+        APOE_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
+        APOE_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, nw * WAVE, L.total));
+        if (per_cu < 1) per_cu = 1;
+    }
+    const uint32_t grid = std::min<uint32_t>(q_count, (uint32_t)per_cu * (uint32_t)ctx->num_cus);
 
     a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;
     DevBuf<uint32_t> bitmaps;
@@ -335,11 +501,19 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
 
     float ms = 0.f;
     APOE_TRY(timed(ctx, &ms, [&]() {
+        if (use_kg) {
+            switch (nw) {
+                case 1: return launch_variant<1, true>(ctx, a, grid, L.total);
+                case 8: return launch_variant<8, true>(ctx, a, grid, L.total);
+                case 4: return launch_variant<4, true>(ctx, a, grid, L.total);
+                default: return launch_variant<2, true>(ctx, a, grid, L.total);
+            }
+        }
         switch (nw) {
             case 1: return launch_variant<1, false>(ctx, a, grid, L.total);
-            case 2: return launch_variant<2, false>(ctx, a, grid, L.total);
             case 8: return launch_variant<8, false>(ctx, a, grid, L.total);
-            default: return launch_variant<4, false>(ctx, a, grid, L.total);
+            case 4: return launch_variant<4, false>(ctx, a, grid, L.total);
+            default: return launch_variant<2, false>(ctx, a, grid, L.total);
         }
     }));
     APOE_HIP(hipStreamSynchronize(ctx->stream));

@@ -35,6 +35,7 @@ extern "C" {
 #define APOE_INF_DIS 1000000.0f /* index.cu:8, query.cu:11 */
 #define APOE_KW_SLOTS 8         /* index.cu:15 KEYEDGEFINAL: row width = degree + 8 */
 #define APOE_KW_CAND 32         /* index.cu:14 KEYEDGE */
+#define APOE_MAX_CANDS 2048     /* pool size limit (the reference stops at 512, query.cu:9) */
 
 typedef struct apoe_ctx apoe_ctx;
 typedef struct apoe_corpus apoe_corpus;
@@ -147,7 +148,7 @@ int apoe_graph_download(const apoe_graph* g, uint32_t* rows, uint32_t* entry);
 typedef struct {
     float w_dense, w_sparse, w_bm25; /* effective (already calibrated) weights */
     float kg_weight;                 /* used only when kg != NULL */
-    uint32_t cands;                  /* pool size, 1..512 (query.cu:9 MAX_CAND_POOL) */
+    uint32_t cands;                  /* pool size, 1..APOE_MAX_CANDS */
     uint32_t max_iter;               /* 0 -> 1000 (query.cu:7 MAX_ITER) */
     uint32_t q_begin, q_count;       /* query range; q_count 0 -> all from q_begin */
     uint32_t variant;                /* 0 = default launch shape; others are tuning shapes */

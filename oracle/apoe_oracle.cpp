@@ -351,16 +351,16 @@ void orc_search_kg(const orc_set* corpus, const orc_set* queries, const orc_kg* 
                 if (e >= kg->n_entities) continue;
                 for (uint32_t j = kg->e2d_off[e]; j < kg->e2d_off[e + 1]; j++) {
                     uint32_t doc = kg->e2d_idx[j];
-                    if (doc >= corpus->n || fresh.size() >= seed_cap) continue;
-                    if (visited.test_and_set(doc)) continue;
+                    if (doc >= corpus->n || visited.test_and_set(doc)) continue;
+                    if (fresh.size() >= seed_cap) continue; /* still marked visited, query.cu:1581 */
                     fresh.push_back({0.f, doc, e, 0});
                 }
             }
             if (fresh.size() < cands) {
                 for (uint32_t i = 0; i < n_entry; i++) {
                     uint32_t e = entry[i];
-                    if (e >= corpus->n || fresh.size() >= seed_cap) continue;
-                    if (visited.test_and_set(e)) continue;
+                    if (e >= corpus->n || visited.test_and_set(e)) continue;
+                    if (fresh.size() >= seed_cap) continue;
                     fresh.push_back({0.f, e, ORC_EMPTY, 0});
                 }
             }
@@ -396,21 +396,44 @@ void orc_search_kg(const orc_set* corpus, const orc_set* queries, const orc_kg* 
                                 if (s.state == 0 && s.id == doc) { s.state = 1; s.ent = e2; }
                         }
                     }
-                    /* (ii) logical edges into recycled slots, query.cu:1718-1735 */
+                    /* (ii) logical edges into recycled slots, query.cu:1718-1735. The t-th
+                     * recycled slot walks the documents of the t-th neighbour entity. Rounds:
+                     * every open slot proposes its first unvisited document (not the parent);
+                     * a document proposed by several slots goes to the lowest slot, the others
+                     * step past it and propose again in the next round. */
+                    struct Rec { size_t slot; uint32_t e2, k, k1; };
+                    std::vector<Rec> open;
                     uint32_t taken = 0;
-                    for (Slot& s : slots) {
-                        if (s.state != 2) continue;
+                    for (size_t si = 0; si < slots.size(); si++) {
+                        if (slots[si].state != 2) continue;
                         uint32_t t = taken++;
                         if (t >= e1 - e0) continue;
                         uint32_t e2 = kg->e2e_idx[e0 + t];
                         if (e2 >= kg->n_entities) continue;
-                        for (uint32_t k = kg->e2d_off[e2]; k < kg->e2d_off[e2 + 1]; k++) {
-                            uint32_t doc = kg->e2d_idx[k];
-                            if (doc == parent || doc >= corpus->n) continue;
-                            if (visited.test_and_set(doc)) continue;
-                            s.id = doc; s.ent = e2; s.hop = p_hop + 1; s.state = 1;
-                            break;
+                        open.push_back({si, e2, kg->e2d_off[e2], kg->e2d_off[e2 + 1]});
+                    }
+                    while (!open.empty()) {
+                        std::vector<Rec> next;
+                        std::vector<uint32_t> prop;
+                        std::vector<Rec> live;
+                        for (Rec r : open) {
+                            while (r.k < r.k1) {
+                                uint32_t doc = kg->e2d_idx[r.k];
+                                if (doc != parent && doc < corpus->n && !(visited.w[doc >> 6] >> (doc & 63) & 1)) break;
+                                r.k++;
+                            }
+                            if (r.k < r.k1) { live.push_back(r); prop.push_back(kg->e2d_idx[r.k]); }
                         }
+                        for (size_t i = 0; i < live.size(); i++) {
+                            bool lose = false;
+                            for (size_t j = 0; j < i; j++) lose |= prop[j] == prop[i];
+                            if (lose) { Rec r = live[i]; r.k++; next.push_back(r); continue; }
+                            Slot& sl = slots[live[i].slot];
+                            sl.id = prop[i]; sl.ent = live[i].e2; sl.hop = p_hop + 1; sl.state = 1;
+                        }
+                        for (size_t i = 0; i < live.size(); i++)
+                            if (slots[live[i].slot].state == 1 && slots[live[i].slot].id == prop[i]) visited.test_and_set(prop[i]);
+                        open.swap(next);
                     }
                 }
                 fresh.clear();

@@ -1,0 +1,96 @@
+"""The hybrid_search Python module end to end on the GPU: files in, .poe out, search."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def files(tmp_path_factory, small_world):
+    import apoe_synth as S
+    import oracle as O
+    d = tmp_path_factory.mktemp("poe")
+    n = 1500
+    C = small_world["C"].head(n)
+    Q = small_world["Q"]
+    p = {k: str(d / k) for k in ("dense.fvecs", "sparse.bin", "bm25.bin", "qdense.fvecs", "qsparse.bin", "qbm25.bin", "index.poe",
+                                 "qrels.txt", "kg.bin", "e2d.bin", "qe.bin")}
+    O.write_fvecs(p["dense.fvecs"], C.dense)
+    O.write_csr(p["sparse.bin"], C.s_off, C.s_idx, C.s_val)
+    O.write_csr(p["bm25.bin"], C.b_off, C.b_idx, C.b_val)
+    O.write_fvecs(p["qdense.fvecs"], Q.dense)
+    O.write_csr(p["qsparse.bin"], Q.s_off, Q.s_idx, Q.s_val)
+    O.write_csr(p["qbm25.bin"], Q.b_off, Q.b_idx, Q.b_val)
+    kg = S.to_numpy(S.knowledge_graph(500, n, Q.n, seed=31, device="cpu", mean_out=5.0))
+    O.write_kg(p["kg.bin"], kg[0], kg[1])
+    O.write_kg(p["e2d.bin"], kg[2], kg[3])
+    O.write_kg(p["qe.bin"], kg[4], kg[5])
+    return dict(paths=p, C=C, Q=Q, kg=kg, n=n)
+
+
+def test_build_and_search_roundtrip(files, capfd):
+    import hybrid_search
+    import oracle as O
+    p, C, Q = files["paths"], files["C"], files["Q"]
+    hybrid_search.build_index(dense_data_path=p["dense.fvecs"], sparse_data_path=p["sparse.bin"], bm25_data_path=p["bm25.bin"],
+                              output_graph_path=p["index.poe"], nnd_iters=8)
+    out = capfd.readouterr().out
+    for line in ("Loading dense data from", "Non zero num:", f"Points: {files['n']}, Dim: 1024", "Max sparse dim:", "Indexing time:"):
+        assert line in out, out
+    rows, entry = O.read_poe(p["index.poe"])
+    assert rows.shape == (files["n"], 40) and len(entry) == 32
+    assert os.path.getsize(p["index.poe"]) == 8 + 4 * 32 + files["n"] * 41 * 4
+    assert np.array_equal(entry, O.entry_points(O.norms(C, 7.0), 32))
+
+    w_user = (1.0, 1.0, 1.0)
+    w_eff = O.calibrate(C, Q, 100, w_user)
+    truth, _ = O.bruteforce_topk(C, Q.head(100), w_eff, 10)
+    with open(p["qrels.txt"], "w") as f:
+        for row in truth:
+            f.write(" ".join(str(x) for x in row[:3]) + "\n")
+    common = dict(dense_data_path=p["dense.fvecs"], dense_query_path=p["qdense.fvecs"], sparse_data_path=p["sparse.bin"],
+                  sparse_query_path=p["qsparse.bin"], bm25_data_path=p["bm25.bin"], bm25_query_path=p["qbm25.bin"], keyword_id_path="",
+                  graph_path=p["index.poe"], ground_truth_path=p["qrels.txt"], top_k=10, cands=128, sparse_weight=1.0, bm25_weight=1.0,
+                  dense_weight=1.0)
+    r = hybrid_search.search(knowledge_path="", entity2doc_path="", query_entity_path="", kg_weight=0.0, **common)
+    out = capfd.readouterr().out
+    for line in ("query num: 100", "Dense weight: 1, Sparse weight: 1, BM25 weight: 1, KG weight: 0", "Degree: 40,num: 1500", "Begin search",
+                 "Search with dense + sparse + bm25", "Query time:", "nDCG@10:"):
+        assert line in out, out
+    assert r["ids"].shape == (100, 128)
+    assert np.allclose(r["weights"], w_eff, rtol=1e-4)
+    oid, odist, _ = O.search(C, Q.head(100), rows, entry, r["weights"], 128)
+    assert (r["ids"][:, :10] == oid[:, :10]).mean() > 0.97
+    want_ndcg, want_recall = O.ndcg(r["ids"][:, :10], [t[:3].tolist() for t in truth])
+    assert abs(r["ndcg"] - want_ndcg) < 1e-5 and abs(r["recall"] - want_recall) < 1e-5
+    assert r["ndcg"] > 0.5
+
+    # dense-only dispatch and the print-only entry point
+    hybrid_search.search_index(knowledge_path="", entity2doc_path="", query_entity_path="", kg_weight=0.0,
+                               **{**common, "sparse_weight": 0.0, "bm25_weight": 0.0})
+    out = capfd.readouterr().out
+    assert "Search with dense\n" in out
+
+    # knowledge-graph path (example.py:14-30 calls it with kg_weight=40)
+    rk = hybrid_search.search(knowledge_path=p["kg.bin"], entity2doc_path=p["e2d.bin"], query_entity_path=p["qe.bin"], kg_weight=40.0, **common)
+    out = capfd.readouterr().out
+    assert "Entity num: 501" in out and "KG Copy end" in out and "Search with dense + sparse + bm25 + kg" in out
+    kg = files["kg"]
+    okg = O.Kg(kg[0], kg[1], kg[2], kg[3], kg[4][:101], kg[5][:kg[4][100]])
+    kid, kdist, _ = O.search(C, Q.head(100), rows, entry, rk["weights"], 128, kg=okg, kg_weight=40.0)
+    assert (rk["ids"][:, :10] == kid[:, :10]).mean() > 0.97
+
+
+def test_errors_raise(files):
+    import hybrid_search
+    p = files["paths"]
+    with pytest.raises(RuntimeError, match="open file error"):
+        hybrid_search.build_index("/nonexistent.fvecs", p["sparse.bin"], p["bm25.bin"], "/tmp/x.poe")
+    with pytest.raises(RuntimeError):
+        hybrid_search.build_index(p["dense.fvecs"], p["sparse.bin"], p["bm25.bin"], "/tmp/x.poe", degree=33)
+    with pytest.raises(RuntimeError, match="knowledge_path"):
+        hybrid_search.search_index(p["dense.fvecs"], p["qdense.fvecs"], p["sparse.bin"], p["qsparse.bin"], p["bm25.bin"], p["qbm25.bin"], "",
+                                   "", "", "", p["index.poe"], p["qrels.txt"], 10, 64, 1.0, 1.0, 1.0, 40.0)
