@@ -20,6 +20,11 @@ sys.path.insert(0, os.path.join(ROOT, "allan-poe_amd"))
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per search launch from FETCH_SIZE + WRITE_SIZE counter runs (rocprofv3 --pmc,
+# scaled by what the counters read for a 1 GiB copy), keyed by the workload they were taken on:
+# (docs, degree, queries, cands, variant). Other workloads report null.
+MEASURED_TRAFFIC = {(1_000_000, 48, 10_000, 512, 0): 9.495e11}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -221,7 +226,8 @@ def main():
             "kernel_ms": avg_kernel_ms,
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": None, "kernel": "search_kernel", "algo_bytes_per_launch": algo_bytes},
+                     "traffic": MEASURED_TRAFFIC.get((args.docs, args.degree, args.queries, cands, args.variant)) if not args.calibrate else None,
+                     "kernel": "search_kernel", "algo_bytes_per_launch": algo_bytes},
         "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)
