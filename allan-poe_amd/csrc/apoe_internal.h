@@ -116,6 +116,7 @@ struct apoe_knn {
     float dense_scale = 1.f;
     float elapsed_ms = 0.f;
     bool pruned = false;
+    bool force_sequential_prune = false; // K = 64 handles use the gather-once prune unless this is set
     apoe::DevBuf<uint32_t> ids, rev, rev_cnt;
     apoe::DevBuf<float> dist, rev_dist, norms;
     apoe::DevBuf<unsigned long long> counter;

@@ -6,12 +6,18 @@
 #include <algorithm>
 #include <memory>
 
+#include "apoe_gram.h"
 #include "apoe_internal.h"
 
 namespace apoe {
 
 constexpr int PR_THREADS = 256;
 constexpr uint32_t ALL_PATHS = PATH_DENSE | PATH_SPARSE | PATH_BM25;
+
+__device__ __forceinline__ void wave_fence_lds() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
 
 struct PruneLds {
     uint32_t tab, idmap, uset, nb_id, nb_dist, det, cid, cdet, sel_id, sel_det, sel_live, sel_kw, o_fwd, o_det, o_kw, ctl, total;
@@ -37,7 +43,7 @@ struct PruneLds {
     }
 };
 
-enum { PC_M = 0, PC_NSEL = 1, PC_REJECT = 2, PC_ALLFLAG = 3, PC_CNT = 4 };
+enum { PC_M = 0, PC_NSEL = 1, PC_REJECT = 2, PC_ALLFLAG = 3, PC_CNT = 4, PC_FAIL = 5 };
 
 // allan_poe (index.cu:539-714) for node u = blockIdx.x:
 //  (a) detour counts over u's sorted list; (b) order by (detour, rank);
@@ -230,6 +236,242 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
     if (tid == 0) cnt_out[u] = ctl[PC_CNT];
 }
 
+// ---- gather-once form of the prune (K = 64) ----
+
+constexpr int GRAM_THREADS = 512; // 8 waves share one node's tables: more lookups in flight per byte of LDS
+constexpr int GRAM_T = 8; // upper bound on the pivot rows whose term tables are live at once
+
+struct GramPruneLds {
+    uint32_t G, tabs, ovf_cnt, rowptr, rownnz, umap, R, idmap, nb_id, nb_dist, nrm, det, order, sel_gi, sel_live, sel_kw, o_fwd, o_det, o_kw, ctl, total;
+    __host__ __device__ GramPruneLds(uint32_t term_slots, uint32_t tgroup, uint32_t umap_slots, uint32_t map_slots, uint32_t words) {
+        uint32_t o = 0;
+        G = o; o += GRAM_ROWS * GRAM_STRIDE * 4;
+        o = (o + 15) & ~15u;
+        tabs = o; o += tgroup * (term_slots + GRAM_OVF) * 8;
+        ovf_cnt = o; o += 8 * 4;
+        rowptr = o; o += GRAM_ROWS * 8;
+        rownnz = o; o += GRAM_ROWS * 4;
+        umap = o; o += umap_slots * 8;
+        idmap = o; o += map_slots * 8;
+        R = o; o += GRAM_ROWS * words * 4;
+        nb_id = o; o += GRAM_ROWS * 4;
+        nb_dist = o; o += GRAM_ROWS * 4;
+        nrm = o; o += GRAM_ROWS * 4;
+        det = o; o += GRAM_ROWS * 4;
+        order = o; o += GRAM_ROWS * 4;
+        sel_gi = o; o += GRAM_ROWS * 4;
+        sel_live = o; o += GRAM_ROWS * 4;
+        sel_kw = o; o += GRAM_ROWS * 4;
+        o_fwd = o; o += GRAM_ROWS * 4;
+        o_det = o; o += GRAM_ROWS * 4;
+        o_kw = o; o += (1 + APOE_KW_CAND) * 4;
+        ctl = o; o += 16 * 4;
+        total = o;
+    }
+};
+
+// Same result as prune_kernel, different traffic: the node's <= 64 neighbour rows are read
+// once, their hybrid Gram matrix is built in LDS (dense part on the matrix cores), every
+// row's overlap with the centre node's BM25 terms becomes a bit mask, and the sequential
+// RNG-IP selection with its keyword flags then runs on LDS only:
+//   <c,s> = G[c][s];   flag(c,s) = (R[s] & ~R[c]) != 0   with R[x] = bm25(x) ∩ bm25(u).
+template <int NT>
+__global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dense_mul, const float* __restrict__ norms,
+                                                                const uint32_t* __restrict__ ids, const float* __restrict__ dist,
+                                                                uint32_t d, uint32_t* fwd, uint32_t* det_out, uint32_t* cnt_out,
+                                                                uint32_t* kw_out, uint32_t term_slots, uint32_t tgroup,
+                                                                uint32_t umap_slots, uint32_t map_slots, uint32_t words,
+                                                                unsigned long long* gfail) {
+    constexpr uint32_t K = GRAM_ROWS;
+    extern __shared__ __align__(16) char smem[];
+    const GramPruneLds L(term_slots, tgroup, umap_slots, map_slots, words);
+    float* G = reinterpret_cast<float*>(smem + L.G);
+    uint2* tabs = reinterpret_cast<uint2*>(smem + L.tabs);
+    uint32_t* ovf_cnt = reinterpret_cast<uint32_t*>(smem + L.ovf_cnt);
+    unsigned long long* rowptr = reinterpret_cast<unsigned long long*>(smem + L.rowptr);
+    uint32_t* rownnz = reinterpret_cast<uint32_t*>(smem + L.rownnz);
+    uint2* umap = reinterpret_cast<uint2*>(smem + L.umap);
+    uint2* idmap = reinterpret_cast<uint2*>(smem + L.idmap);
+    uint32_t* R = reinterpret_cast<uint32_t*>(smem + L.R);
+    uint32_t* nb_id = reinterpret_cast<uint32_t*>(smem + L.nb_id);
+    float* nb_dist = reinterpret_cast<float*>(smem + L.nb_dist);
+    float* nrm = reinterpret_cast<float*>(smem + L.nrm);
+    uint32_t* det = reinterpret_cast<uint32_t*>(smem + L.det);
+    uint32_t* order = reinterpret_cast<uint32_t*>(smem + L.order);
+    uint32_t* sel_gi = reinterpret_cast<uint32_t*>(smem + L.sel_gi);
+    uint32_t* sel_live = reinterpret_cast<uint32_t*>(smem + L.sel_live);
+    uint32_t* sel_kw = reinterpret_cast<uint32_t*>(smem + L.sel_kw);
+    uint32_t* o_fwd = reinterpret_cast<uint32_t*>(smem + L.o_fwd);
+    uint32_t* o_det = reinterpret_cast<uint32_t*>(smem + L.o_det);
+    uint32_t* o_kw = reinterpret_cast<uint32_t*>(smem + L.o_kw);
+    volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
+
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const uint32_t u = blockIdx.x, umask = umap_slots - 1, mmask = map_slots - 1;
+    const size_t base = (size_t)u * K;
+    const uint64_t lane_lt = (1ull << lane) - 1;
+
+    for (uint32_t i = tid; i < map_slots; i += NT) idmap[i] = make_uint2(EMPTY, 0u);
+    for (uint32_t i = tid; i < umap_slots; i += NT) umap[i] = make_uint2(EMPTY, 0u);
+    for (uint32_t i = tid; i < K * words; i += NT) R[i] = 0;
+    for (uint32_t i = tid; i < K; i += NT) det[i] = 0;
+    if (tid < 16) ctl[tid] = 0;
+    __syncthreads();
+
+    if (wave == 0) {
+        const uint32_t v = ids[base + lane] & ~FLAG;
+        const float dv = dist[base + lane];
+        const bool ok = dv < INF_DIS && v < C.n && v != u;
+        const uint64_t b = __ballot(ok);
+        if (ok) {
+            const uint32_t pos = __popcll(b & lane_lt);
+            nb_id[pos] = v;
+            nb_dist[pos] = dv;
+            nrm[pos] = norms[v];
+        }
+        if (lane == 0) ctl[PC_M] = __popcll(b);
+    }
+    {   // u's BM25 terms -> index
+        const uint64_t du = C.desc[u];
+        const uint2* sp = reinterpret_cast<const uint2*>(C.recs + desc_off(du) * 16 + DENSE_BYTES);
+        const uint32_t ns = desc_nnz_s(du), nb = desc_nnz_b(du);
+        for (uint32_t j = tid; j < nb; j += NT) {
+            const uint32_t key = sp[ns + j].x;
+            uint32_t h = term_hash(key, umask);
+            while (true) {
+                const uint32_t old = atomicCAS(&umap[h].x, EMPTY, key);
+                if (old == EMPTY) { umap[h].y = j; break; }
+                if (old == key) break;
+                h = (h + 1) & umask;
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t m = ctl[PC_M];
+
+    // (a) detour counts (as prune_kernel)
+    for (uint32_t i = tid; i < m; i += NT) {
+        const uint32_t key = nb_id[i];
+        uint32_t h = term_hash(key, mmask);
+        while (true) {
+            const uint32_t old = atomicCAS(&idmap[h].x, EMPTY, key);
+            if (old == EMPTY) { idmap[h].y = i; break; }
+            if (old == key) break;
+            h = (h + 1) & mmask;
+        }
+    }
+    // R[r] = bits of u's BM25 terms that row r holds too: one wave per row, lanes over its BM25 pairs
+    for (uint32_t r = wave; r < m; r += NT / WAVE) {
+        const uint64_t dr = C.desc[nb_id[r]];
+        const uint2* sp = reinterpret_cast<const uint2*>(C.recs + desc_off(dr) * 16 + DENSE_BYTES);
+        const uint32_t ns = desc_nnz_s(dr), nb = desc_nnz_b(dr);
+        for (uint32_t j = lane; j < nb; j += WAVE) {
+            const uint32_t key = sp[ns + j].x;
+            uint32_t h = term_hash(key, umask);
+            while (true) {
+                const uint2 e = umap[h];
+                if (e.x == key) { atomicOr(&R[r * words + (e.y >> 5)], 1u << (e.y & 31)); break; }
+                if (e.x == EMPTY) break;
+                h = (h + 1) & umask;
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t t = tid; t < m * K; t += NT) {
+        const uint32_t r = t / K, j = t % K;
+        const size_t at = (size_t)nb_id[r] * K + j;
+        const uint32_t x = ids[at] & ~FLAG;
+        const float dx = dist[at];
+        uint32_t h = term_hash(x, mmask);
+        while (true) {
+            const uint2 e = idmap[h];
+            if (e.x == x) {
+                if (e.y > r && dx < nb_dist[e.y]) atomicAdd(&det[e.y], 1u);
+                break;
+            }
+            if (e.x == EMPTY) break;
+            h = (h + 1) & mmask;
+        }
+    }
+    // hybrid Gram matrix of the m rows
+    if (m > 0 && wave < 4) gram_dense_64(C, nb_id, m, dense_mul, G, wave, lane);
+    __syncthreads();
+    if (tgroup == 8) gram_sparse_64<8>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
+    else gram_sparse_64<4>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
+    // (b) stable order by detour count
+    for (uint32_t i = tid; i < m; i += NT) {
+        const uint32_t key = (det[i] << 16) | i;
+        uint32_t r = 0;
+        for (uint32_t j = 0; j < m; j++) r += ((det[j] << 16) | j) < key;
+        order[r] = i;
+    }
+    __syncthreads();
+
+    // (c)+(d) sequential selection on the Gram matrix: wave 0, one lane per selected member
+    if (wave == 0 && m > 0) {
+        uint32_t n_sel = 1;
+        if (lane == 0) { sel_gi[0] = order[0]; sel_live[0] = 1; sel_kw[0] = 0; }
+        wave_fence_lds();
+        for (uint32_t t = 1; t < m; t++) {
+            const uint32_t c = order[t];
+            const float norm_c = nrm[c];
+            bool rej = false, noflag = false, tomb = false;
+            if ((uint32_t)lane < n_sel && sel_live[lane]) {
+                const uint32_t sgi = sel_gi[lane];
+                const float p = G[c * GRAM_STRIDE + sgi];
+                rej = norm_c < p;
+                tomb = nrm[sgi] < p;
+                bool flag = false;
+                for (uint32_t w = 0; w < words; w++) flag |= (R[sgi * words + w] & ~R[c * words + w]) != 0;
+                noflag = !flag;
+            }
+            const bool reject = __ballot(rej) != 0;
+            const bool allflag = __ballot(noflag) == 0;
+            if (tomb) sel_live[lane] = 0;
+            if (!reject) {
+                if (lane == 0) { sel_gi[n_sel] = c; sel_live[n_sel] = 1; sel_kw[n_sel] = allflag ? 1u : 0u; }
+                n_sel++;
+            }
+            wave_fence_lds();
+        }
+        // (e) emit
+        if (lane == 0) {
+            uint32_t cnt = 0, nkw = 0;
+            for (uint32_t i = 0; i < n_sel; i++) {
+                if (!sel_live[i]) continue;
+                const uint32_t gi = sel_gi[i];
+                if (cnt < d) { o_fwd[cnt] = nb_id[gi]; o_det[cnt] = det[gi]; cnt++; }
+                else if (sel_kw[i] && nkw < APOE_KW_CAND) { o_kw[1 + nkw] = nb_id[gi]; nkw++; }
+            }
+            for (uint32_t t = 0; t < m && cnt < d; t++) {
+                const uint32_t cidv = nb_id[order[t]];
+                bool present = false;
+                for (uint32_t j = 0; j < cnt; j++) present |= o_fwd[j] == cidv;
+                if (!present) { o_fwd[cnt] = cidv; o_det[cnt] = det[order[t]]; cnt++; }
+            }
+            ctl[PC_CNT] = cnt;
+            for (; cnt < d; cnt++) { o_fwd[cnt] = u; o_det[cnt] = EMPTY; }
+            o_kw[0] = nkw;
+            for (uint32_t j = nkw; j < APOE_KW_CAND; j++) o_kw[1 + j] = 0;
+        }
+    }
+    if (m == 0 && tid == 0) {
+        for (uint32_t j = 0; j < d; j++) { o_fwd[j] = u; o_det[j] = EMPTY; }
+        for (uint32_t j = 0; j <= APOE_KW_CAND; j++) o_kw[j] = 0;
+        ctl[PC_CNT] = 0;
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < d; i += NT) {
+        fwd[(size_t)u * d + i] = o_fwd[i];
+        det_out[(size_t)u * d + i] = o_det[i];
+    }
+    for (uint32_t i = tid; i < 1 + APOE_KW_CAND; i += NT) kw_out[(size_t)u * (1 + APOE_KW_CAND) + i] = o_kw[i];
+    if (tid == 0) {
+        cnt_out[u] = ctl[PC_CNT];
+        if (ctl[PC_FAIL]) atomicOr(gfail, 1ull); // an overflow list was too short: the host redoes the prune with prune_kernel
+    }
+}
+
 // ---- final rows (index.cu:717-807) ----
 
 __global__ __launch_bounds__(256) void indegree_kernel(uint32_t n, uint32_t d, const uint32_t* __restrict__ fwd, const uint32_t* __restrict__ cnt,
@@ -347,6 +589,26 @@ int launch_prune(apoe_knn* g, uint32_t degree) {
     const uint32_t term_slots = doc_term_slots(g->corpus);
     const uint32_t uset_slots = next_pow2(std::max(64u, 2 * g->corpus->max_nnz_b));
     const uint32_t map_slots = next_pow2(4 * g->K);
+    // gather-once form: K = 64 and the BM25 overlap masks fit in LDS
+    const uint32_t words = (g->corpus->max_nnz_b + 31) / 32 + (g->corpus->max_nnz_b == 0);
+    const uint32_t gram_slots = next_pow2(std::max(64u, 2 * (g->corpus->max_nnz_s + g->corpus->max_nnz_b)));
+    // 8 live pivot tables if two workgroups then still share a CU's LDS, else 4
+    const uint32_t lds_budget = (uint32_t)std::min<size_t>(ctx->lds_per_block, 80 * 1024);
+    uint32_t tgroup = GramPruneLds(gram_slots, 8, uset_slots, map_slots, words).total <= lds_budget ? 8 : 4;
+    const GramPruneLds GL(gram_slots, tgroup, uset_slots, map_slots, words);
+    if (g->K == GRAM_ROWS && GL.total <= lds_budget && !g->force_sequential_prune) {
+        APOE_HIP(hipMemsetAsync(g->counter.p + 1, 0, sizeof(unsigned long long), ctx->stream));
+        APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&prune_gram_kernel<GRAM_THREADS>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GL.total));
+        prune_gram_kernel<GRAM_THREADS><<<g->n, GRAM_THREADS, GL.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->norms.p, g->ids.p,
+                                                                      g->dist.p, degree, g->fwd.p, g->det.p, g->cnt.p, g->kw.p, gram_slots,
+                                                                      tgroup, uset_slots, map_slots, words, g->counter.p + 1);
+        APOE_HIP(hipGetLastError());
+        unsigned long long failed = 0;
+        APOE_HIP(hipMemcpyAsync(&failed, g->counter.p + 1, sizeof(failed), hipMemcpyDeviceToHost, ctx->stream));
+        APOE_HIP(hipStreamSynchronize(ctx->stream));
+        if (!failed) return APOE_OK;
+        // a row's terms clustered on the same table slots: redo with the table-probing kernel below
+    }
     const PruneLds L(term_slots, uset_slots, map_slots, g->K);
     APOE_REQUIRE(L.total <= 64 * 1024, "prune needs %u bytes of LDS (rows with up to %u sparse terms)", L.total,
                  g->corpus->max_nnz_s + g->corpus->max_nnz_b);

@@ -206,3 +206,31 @@ def test_gpu_built_index_recall(gpu_world):
     rows, entry = graph.download()
     assert rows.shape == (w["C"].n, 40) and len(entry) == 32
     graph.close()
+
+
+def test_prune_k128_sequential_kernel_matches_oracle(gpu_world):
+    """K = 128 lists go through the table-probing prune kernel (the gather-once form is K = 64 only)."""
+    import apoe
+    import oracle as O
+    w = gpu_world
+    C = w["C"]
+    st = O.nnd_init(C.n, 128, 3)
+    for it in range(4):
+        O.nnd_iterate(C, 7.0, st)
+        if it < 3:
+            st.rev_cnt[:] = 0
+    ids, dist = st.ids & 0x7FFFFFFF, st.dist.copy()
+    knn = apoe.Knn(w["ctx"], w["gc"], 128, 7.0)
+    knn.upload(ids, dist)
+    knn.prune(64)
+    g_fwd, g_det, g_cnt, g_kw = knn.prune_download()
+    c_fwd, c_det, c_cnt, c_kw = O.prune(C, 7.0, O.norms(C, 7.0), ids, dist, 64)
+    same = np.all(g_fwd == c_fwd, axis=1)
+    assert same.mean() >= 0.995
+    assert np.array_equal(g_det[same], c_det[same]) and np.array_equal(g_cnt[same], c_cnt[same])
+    graph = knn.finalize()
+    rows, entry = graph.download()
+    assert np.array_equal(rows, O.final_graph(g_fwd, g_det, g_cnt, g_kw))
+    assert rows.shape == (C.n, 72)
+    graph.close()
+    knn.close()
