@@ -31,7 +31,7 @@ class SearchParams(C.Structure):
 
 class SearchStats(C.Structure):
     _fields_ = [("kernel_ms", C.c_float), ("expansions", C.c_uint64), ("evaluations", C.c_uint64),
-                ("nnz_sparse", C.c_uint64), ("nnz_bm25", C.c_uint64), ("algo_bytes", C.c_uint64)]
+                ("nnz_sparse", C.c_uint64), ("nnz_bm25", C.c_uint64), ("dense_rows", C.c_uint64), ("algo_bytes", C.c_uint64)]
 
 
 EXPORTS = [
@@ -40,7 +40,7 @@ EXPORTS = [
     "apoe_kg_create", "apoe_kg_destroy", "apoe_calibrate_weights", "apoe_hybrid_distance_batch", "apoe_hybrid_distance_pairs", "apoe_norms",
     "apoe_knn_create", "apoe_knn_destroy", "apoe_nnd_init", "apoe_nnd_iterate", "apoe_nnd_merge_reverse",
     "apoe_knn_download", "apoe_knn_upload", "apoe_prune", "apoe_prune_download", "apoe_finalize_graph",
-    "apoe_knn_elapsed_ms", "apoe_graph_create", "apoe_graph_destroy", "apoe_graph_info", "apoe_graph_download",
+    "apoe_knn_elapsed_ms", "apoe_knn_counters", "apoe_graph_create", "apoe_graph_destroy", "apoe_graph_info", "apoe_graph_download",
     "apoe_search",
 ]
 
@@ -262,6 +262,12 @@ class Knn:
 
     def elapsed_ms(self):
         return float(lib().apoe_knn_elapsed_ms(self.h))
+
+    def counters(self):
+        """(evaluations, dense rows read) of the NN-Descent steps since init."""
+        out = (C.c_uint64 * 2)()
+        _check(lib().apoe_knn_counters(self.h, out))
+        return int(out[0]), int(out[1])
 
     def close(self):
         if self.h:

@@ -34,6 +34,7 @@ __host__ __device__ inline uint32_t desc_nnz_b(uint64_t d) { return (uint32_t)(d
 struct CorpusView {
     const uint64_t* desc;
     const char* recs;
+    const float* dnorm; // Euclidean norm of each dense row (bounds the dense inner product)
     uint32_t n;
 };
 
@@ -59,6 +60,18 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// Sum over the wave with DPP adds inside each 16-lane row and four lane reads across rows;
+// every lane gets the total.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));  // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));  // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)); // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)); // row_mirror
+    const int iv = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+}
 
 // Total order on floats as unsigned integers (negative distances are common: 1 - IP).
 __device__ __forceinline__ uint32_t float_key(float f) {
@@ -252,6 +265,166 @@ __device__ __forceinline__ EvalOut eval_wave(const CorpusView& C, uint32_t id, c
     o.nnz_s = (paths & PATH_SPARSE) ? ns : 0u;
     o.nnz_b = (paths & PATH_BM25) ? nb : 0u;
     if (KW) *kw_any = __ballot(kw) != 0;
+    return o;
+}
+
+// Euclidean norm of the pivot's dense part as held in registers (weights included).
+__device__ __forceinline__ float pivot_dense_norm(const PivotDense& p) {
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) a += p.v[i].x * p.v[i].x + p.v[i].y * p.v[i].y + p.v[i].z * p.v[i].z + p.v[i].w * p.v[i].w;
+    return sqrtf(wave_sum_dpp(a));
+}
+
+struct BoundedOut {
+    float dist;      // 1 - ip - bonus, or INF_DIS when the dense part was skipped
+    uint32_t nnz_s;  // SPLADE pairs read
+    uint32_t nnz_b;  // BM25 pairs read
+    bool dense_read; // the 4 KB dense row was read
+};
+
+// Two-stage hybrid distance between the pivot and document `id` (wave-uniform).
+// Stage 1 reads the descriptor, the dense norm and the pairs and forms the sparse sum.
+// |<pivot_d, doc_d>| <= |pivot_d| * |doc_d|, so 1 - (sparse + dense_mul*|p|*|d|) - bonus is a
+// lower bound of the distance: if even that is above `thr` (the value the caller would reject
+// anyway: the worst entry of a full pool / list), the dense row is not read and INF_DIS is
+// returned. Otherwise stage 2 reads the row. Pass thr = +inf to always get the exact distance.
+__device__ __forceinline__ BoundedOut eval_wave_bounded(const CorpusView& C, uint32_t id, const PivotDense& pv, float pv_norm, const uint2* tab,
+                                                        uint32_t mask, uint32_t paths, float dense_mul, float bonus, float thr) {
+    const int lane = lane_id();
+    const uint64_t desc = C.desc[id];
+    const char* rec = C.recs + desc_off(desc) * 16;
+    const uint32_t ns = desc_nnz_s(desc), nb = desc_nnz_b(desc);
+    const uint32_t begin = (paths & PATH_SPARSE) ? 0u : ns;
+    const uint32_t end = (paths & PATH_BM25) ? ns + nb : ns;
+    BoundedOut o;
+    o.nnz_s = (paths & PATH_SPARSE) ? ns : 0u;
+    o.nnz_b = (paths & PATH_BM25) ? nb : 0u;
+    o.dense_read = false;
+    float ssum = 0.f;
+    const bool has_sparse = (paths & (PATH_SPARSE | PATH_BM25)) != 0;
+    if (has_sparse) {
+        const float dub = (paths & PATH_DENSE) ? dense_mul * pv_norm * C.dnorm[id] : 0.f;
+        const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
+        uint2 kv0 = make_uint2(0, 0), kv1 = kv0, kv2 = kv0;
+        const uint32_t j0 = begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
+        if (j0 < end) kv0 = sp[j0];
+        if (j1 < end) kv1 = sp[j1];
+        if (j2 < end) kv2 = sp[j2];
+        float acc = 0.f;
+        if (j0 < end) term_table_probe(tab, mask, kv0.x, __uint_as_float(kv0.y), acc);
+        if (j1 < end) term_table_probe(tab, mask, kv1.x, __uint_as_float(kv1.y), acc);
+        if (j2 < end) term_table_probe(tab, mask, kv2.x, __uint_as_float(kv2.y), acc);
+        for (uint32_t j = j2 + WAVE; j < end; j += WAVE) {
+            const uint2 kv = sp[j];
+            term_table_probe(tab, mask, kv.x, __uint_as_float(kv.y), acc);
+        }
+        ssum = wave_sum_dpp(acc);
+        if (!(paths & PATH_DENSE)) {
+            o.dist = 1.0f - ssum - bonus;
+            return o;
+        }
+        const float lb = 1.0f - (ssum + dub) - bonus;
+        if (lb > thr + 1e-5f * (fabsf(ssum) + dub + fabsf(bonus) + 1.0f)) {
+            o.dist = INF_DIS;
+            return o;
+        }
+    }
+    float dsum = 0.f;
+    if (paths & PATH_DENSE) {
+        const float4* r = reinterpret_cast<const float4*>(rec);
+        float4 x[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) x[i] = r[lane + WAVE * i];
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            acc = fmaf(x[i].x, pv.v[i].x, acc);
+            acc = fmaf(x[i].y, pv.v[i].y, acc);
+            acc = fmaf(x[i].z, pv.v[i].z, acc);
+            acc = fmaf(x[i].w, pv.v[i].w, acc);
+        }
+        dsum = dense_mul * wave_sum_dpp(acc);
+        o.dense_read = true;
+    }
+    o.dist = 1.0f - (dsum + ssum) - bonus;
+    return o;
+}
+
+// The same two-stage evaluation split in two calls, so that a wave can have the sparse
+// parts of several candidates in flight before it consumes the first one.
+struct PendingEval {
+    const char* rec;
+    uint2 kv0, kv1, kv2;
+    uint32_t ns, nb, begin, end;
+    float dub;
+};
+
+__device__ __forceinline__ void eval_issue(PendingEval& p, const CorpusView& C, uint32_t id, float pv_norm, uint32_t paths, float dense_mul) {
+    const int lane = lane_id();
+    const uint64_t desc = C.desc[id];
+    p.rec = C.recs + desc_off(desc) * 16;
+    p.ns = desc_nnz_s(desc);
+    p.nb = desc_nnz_b(desc);
+    p.begin = (paths & PATH_SPARSE) ? 0u : p.ns;
+    p.end = (paths & PATH_BM25) ? p.ns + p.nb : p.ns;
+    p.dub = (paths & PATH_DENSE) ? dense_mul * pv_norm * C.dnorm[id] : 0.f;
+    const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
+    const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
+    p.kv0 = p.kv1 = p.kv2 = make_uint2(0, 0);
+    if (j0 < p.end) p.kv0 = sp[j0];
+    if (j1 < p.end) p.kv1 = sp[j1];
+    if (j2 < p.end) p.kv2 = sp[j2];
+}
+
+__device__ __forceinline__ BoundedOut eval_finish(const PendingEval& p, const PivotDense& pv, const uint2* tab, uint32_t mask, uint32_t paths,
+                                                  float dense_mul, float bonus, float thr) {
+    const int lane = lane_id();
+    BoundedOut o;
+    o.nnz_s = (paths & PATH_SPARSE) ? p.ns : 0u;
+    o.nnz_b = (paths & PATH_BM25) ? p.nb : 0u;
+    o.dense_read = false;
+    float ssum = 0.f;
+    if (paths & (PATH_SPARSE | PATH_BM25)) {
+        const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
+        const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
+        float acc = 0.f;
+        if (j0 < p.end) term_table_probe(tab, mask, p.kv0.x, __uint_as_float(p.kv0.y), acc);
+        if (j1 < p.end) term_table_probe(tab, mask, p.kv1.x, __uint_as_float(p.kv1.y), acc);
+        if (j2 < p.end) term_table_probe(tab, mask, p.kv2.x, __uint_as_float(p.kv2.y), acc);
+        for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) {
+            const uint2 kv = sp[j];
+            term_table_probe(tab, mask, kv.x, __uint_as_float(kv.y), acc);
+        }
+        ssum = wave_sum_dpp(acc);
+        if (!(paths & PATH_DENSE)) {
+            o.dist = 1.0f - ssum - bonus;
+            return o;
+        }
+        const float lb = 1.0f - (ssum + p.dub) - bonus;
+        if (lb > thr + 1e-5f * (fabsf(ssum) + p.dub + fabsf(bonus) + 1.0f)) {
+            o.dist = INF_DIS;
+            return o;
+        }
+    }
+    float dsum = 0.f;
+    if (paths & PATH_DENSE) {
+        const float4* r = reinterpret_cast<const float4*>(p.rec);
+        float4 x[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) x[i] = r[lane + WAVE * i];
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            acc = fmaf(x[i].x, pv.v[i].x, acc);
+            acc = fmaf(x[i].y, pv.v[i].y, acc);
+            acc = fmaf(x[i].z, pv.v[i].z, acc);
+            acc = fmaf(x[i].w, pv.v[i].w, acc);
+        }
+        dsum = dense_mul * wave_sum_dpp(acc);
+        o.dense_read = true;
+    }
+    o.dist = 1.0f - (dsum + ssum) - bonus;
     return o;
 }
 

@@ -101,17 +101,6 @@ __device__ __forceinline__ Slots3 gram_slots3(uint32_t key, uint32_t mask) {
     return s;
 }
 
-// Sum over the wave with DPP adds inside each 16-lane row and four lane reads across rows.
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));  // quad_perm [1,0,3,2]
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));  // quad_perm [2,3,0,1]
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)); // row_half_mirror
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)); // row_mirror
-    const int iv = __builtin_bit_cast(int, v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16)) +
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
-}
-
 // tabs: T tables of `slots` entries, then T overflow lists of GRAM_OVF entries; ovf_cnt[T];
 // rowptr/rownnz: LDS scratch for 64 rows; *fail is set when an overflow list is too short
 // (the caller must then discard G). All threads of the block call it; G must already hold

@@ -84,7 +84,8 @@ struct apoe_corpus {
     uint64_t rec_bytes = 0;
     apoe::DevBuf<uint64_t> desc;
     apoe::DevBuf<char> recs;
-    apoe::CorpusView view() const { return apoe::CorpusView{desc.p, recs.p, n}; }
+    apoe::DevBuf<float> dnorm;
+    apoe::CorpusView view() const { return apoe::CorpusView{desc.p, recs.p, dnorm.p, n}; }
 };
 
 struct apoe_queries {
@@ -117,8 +118,9 @@ struct apoe_knn {
     float elapsed_ms = 0.f;
     bool pruned = false;
     bool force_sequential_prune = false; // K = 64 handles use the gather-once prune unless this is set
-    apoe::DevBuf<uint32_t> ids, rev, rev_cnt;
-    apoe::DevBuf<float> dist, rev_dist, norms;
+    apoe::DevBuf<uint32_t> ids, rev_cnt;
+    apoe::DevBuf<unsigned long long> rev; // [n][K] reverse lists: (distance key << 32 | id) per slot
+    apoe::DevBuf<float> dist, norms;
     apoe::DevBuf<unsigned long long> counter;
     // prune outputs
     apoe::DevBuf<uint32_t> fwd, det, cnt, kw;
@@ -132,7 +134,7 @@ int copy_out(apoe_ctx* ctx, void* dst_any, const void* src_dev, size_t bytes);
 
 // Kernel launchers (one per .hip file).
 int launch_pack(apoe_ctx* ctx, uint32_t n, const float* dense, const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,
-                const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs);
+                const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs, float* dnorm);
 int launch_distance_batch(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const float* w3, const uint32_t* ids_dev,
                           uint32_t M, float* out_dev);
 int launch_distance_pairs(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale, const uint32_t* a_dev, const uint32_t* b_dev,

@@ -166,6 +166,7 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
     c->rec_bytes = off16 * 16;
     APOE_TRY(c->desc.alloc(n));
     APOE_TRY(c->recs.alloc(c->rec_bytes));
+    APOE_TRY(c->dnorm.alloc(n));
     APOE_TRY(copy_in(ctx, c->desc.p, desc.data(), n * sizeof(uint64_t)));
     {
         DevInput<float> d_dense, d_sval, d_bval;
@@ -177,7 +178,7 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
         APOE_TRY(d_boff.init(ctx, b_off, n + 1));
         APOE_TRY(d_bidx.init(ctx, b_idx, hb[n]));
         APOE_TRY(d_bval.init(ctx, b_val, hb[n]));
-        APOE_TRY(launch_pack(ctx, n, d_dense.p, d_soff.p, d_sidx.p, d_sval.p, d_boff.p, d_bidx.p, d_bval.p, c->desc.p, c->recs.p));
+        APOE_TRY(launch_pack(ctx, n, d_dense.p, d_soff.p, d_sidx.p, d_sval.p, d_boff.p, d_bidx.p, d_bval.p, c->desc.p, c->recs.p, c->dnorm.p));
         APOE_HIP(hipStreamSynchronize(ctx->stream));
     }
     *out = c.release();
@@ -195,7 +196,7 @@ int apoe_corpus_info(const apoe_corpus* c, uint32_t* info4) {
     return APOE_OK;
 }
 
-uint64_t apoe_corpus_bytes(const apoe_corpus* c) { return c ? c->rec_bytes + (uint64_t)c->n * 8 : 0; }
+uint64_t apoe_corpus_bytes(const apoe_corpus* c) { return c ? c->rec_bytes + (uint64_t)c->n * 12 : 0; }
 
 int apoe_queries_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* dense, const uint32_t* s_off, const uint32_t* s_idx,
                         const float* s_val, const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, apoe_queries** out) {

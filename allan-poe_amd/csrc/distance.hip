@@ -8,13 +8,24 @@ namespace apoe {
 __global__ __launch_bounds__(256) void pack_kernel(uint32_t n, const float* __restrict__ dense, const uint32_t* __restrict__ s_off,
                                                    const uint32_t* __restrict__ s_idx, const float* __restrict__ s_val,
                                                    const uint32_t* __restrict__ b_off, const uint32_t* __restrict__ b_idx,
-                                                   const float* __restrict__ b_val, const uint64_t* __restrict__ desc, char* recs) {
+                                                   const float* __restrict__ b_val, const uint64_t* __restrict__ desc, char* recs, float* dnorm) {
+    __shared__ float part[4];
     for (uint32_t doc = blockIdx.x; doc < n; doc += gridDim.x) {
         const uint64_t d = desc[doc];
         char* rec = recs + desc_off(d) * 16;
         const float4* src = reinterpret_cast<const float4*>(dense + (size_t)doc * DIM);
         float4* dst = reinterpret_cast<float4*>(rec);
-        for (int i = threadIdx.x; i < DIM / 4; i += blockDim.x) dst[i] = src[i];
+        float sq = 0.f;
+        for (int i = threadIdx.x; i < DIM / 4; i += blockDim.x) {
+            const float4 x = src[i];
+            dst[i] = x;
+            sq += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+        }
+        sq = wave_sum_dpp(sq);
+        __syncthreads();
+        if (lane_id() == 0) part[threadIdx.x / WAVE] = sq;
+        __syncthreads();
+        if (threadIdx.x == 0) dnorm[doc] = sqrtf(part[0] + part[1] + part[2] + part[3]);
         uint2* sp = reinterpret_cast<uint2*>(rec + DENSE_BYTES);
         const uint32_t s0 = s_off[doc], ns = desc_nnz_s(d), b0 = b_off[doc], nb = desc_nnz_b(d);
         for (uint32_t j = threadIdx.x; j < ns; j += blockDim.x) sp[j] = make_uint2(s_idx[s0 + j], __float_as_uint(s_val[s0 + j]));
@@ -26,10 +37,10 @@ __global__ __launch_bounds__(256) void pack_kernel(uint32_t n, const float* __re
 }
 
 int launch_pack(apoe_ctx* ctx, uint32_t n, const float* dense, const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,
-                const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs) {
+                const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs, float* dnorm) {
     uint32_t grid = n < 65536u * 16u ? n : 65536u * 16u;
     if (grid == 0) return APOE_OK;
-    pack_kernel<<<grid, 256, 0, ctx->stream>>>(n, dense, s_off, s_idx, s_val, b_off, b_idx, b_val, desc, recs);
+    pack_kernel<<<grid, 256, 0, ctx->stream>>>(n, dense, s_off, s_idx, s_val, b_off, b_idx, b_val, desc, recs, dnorm);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
 }

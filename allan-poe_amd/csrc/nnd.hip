@@ -9,6 +9,7 @@ namespace apoe {
 
 constexpr int NND_THREADS = 256;
 constexpr int NND_PICKS = 4; // neighbours sampled per node and step (index.cu:157,171-181)
+constexpr uint32_t ALLP = PATH_DENSE | PATH_SPARSE | PATH_BM25;
 
 __device__ __forceinline__ float key_dist(uint64_t key) {
     uint32_t u = (uint32_t)(key >> 32);
@@ -27,14 +28,13 @@ __device__ __forceinline__ bool id_set_insert(uint32_t* set, uint32_t mask, uint
     }
 }
 
-__global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t n, uint32_t K, uint64_t seed, uint32_t* ids, float* dist, uint32_t* rev,
-                                                       float* rev_dist, uint32_t* rev_cnt) {
+__global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t n, uint32_t K, uint64_t seed, uint32_t* ids, float* dist,
+                                                       unsigned long long* rev, uint32_t* rev_cnt) {
     const uint64_t total = (uint64_t)n * K;
     for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (uint64_t)gridDim.x * blockDim.x) {
         ids[t] = (uint32_t)(mix64(seed ^ mix64(t)) % n);
         dist[t] = INF_DIS;
-        rev[t] = EMPTY;
-        rev_dist[t] = INF_DIS;
+        rev[t] = ~0ull; // (distance key, id) in one word: id part reads as EMPTY
         if (t < n) rev_cnt[t] = 0;
     }
 }
@@ -112,7 +112,7 @@ struct NndLds {
 // closer than u's current worst into the list, and register u with every member of
 // the merged list when the list changed.
 __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, float dense_mul, uint32_t K, uint32_t* ids, float* dist,
-                                                                  uint32_t* rev, float* rev_dist, uint32_t* rev_cnt, uint32_t term_slots,
+                                                                  unsigned long long* rev, uint32_t* rev_cnt, uint32_t term_slots,
                                                                   uint32_t seen_slots, unsigned long long* inserted) {
     extern __shared__ __align__(16) char smem[];
     const NndLds L(term_slots, seen_slots, K);
@@ -171,7 +171,7 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
         const uint32_t v = own_id[ctl[p]] & ~FLAG;
         uint32_t c;
         if (r < K) c = ids[(size_t)v * K + r] & ~FLAG;
-        else c = rev[(size_t)v * K + (r - K)];
+        else c = (uint32_t)rev[(size_t)v * K + (r - K)];
         if (c < C.n && id_set_insert(seen, smask, c)) cand_id[atomicAdd(&ctl[5], 1u)] = c;
     }
     // pivot = u
@@ -182,16 +182,32 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
     pivot_terms_from_record(tab, tmask, rec, desc_nnz_s(du) + desc_nnz_b(du), tid, NND_THREADS);
     __syncthreads();
 
-    // 4. distances
+    // 4. distances; only those below the current worst matter (step 5), so a candidate whose
+    //    sparse part plus the bound of its dense part cannot get there is not read in full
     const uint32_t n_cand = ctl[5];
-    for (uint32_t j = wave; j < n_cand; j += NND_THREADS / WAVE) {
-        EvalOut e = eval_wave(C, uniform(cand_id[j]), pv, tab, tmask, PATH_DENSE | PATH_SPARSE | PATH_BM25, dense_mul);
-        if (lane == 0) cand_dist[j] = 1.0f - e.ip;
+    const float worst = own_dist[K - 1];
+    const float thr = worst < INF_DIS ? worst : __builtin_inff();
+    const float pv_norm = pivot_dense_norm(pv);
+    unsigned long long n_dense = 0;
+    for (uint32_t j = wave; j < n_cand; j += (NND_THREADS / WAVE) * 2) {
+        const uint32_t j2 = j + NND_THREADS / WAVE;
+        PendingEval p0, p1;
+        eval_issue(p0, C, uniform(cand_id[j]), pv_norm, ALLP, dense_mul);
+        if (j2 < n_cand) eval_issue(p1, C, uniform(cand_id[j2]), pv_norm, ALLP, dense_mul);
+        BoundedOut e0 = eval_finish(p0, pv, tab, tmask, ALLP, dense_mul, 0.f, thr);
+        n_dense += e0.dense_read;
+        if (lane == 0) cand_dist[j] = e0.dist;
+        if (j2 < n_cand) {
+            BoundedOut e1 = eval_finish(p1, pv, tab, tmask, ALLP, dense_mul, 0.f, thr);
+            n_dense += e1.dense_read;
+            if (lane == 0) cand_dist[j2] = e1.dist;
+        }
     }
+    if (lane == 0 && n_dense) atomicAdd(inserted + 3, n_dense);
+    if (tid == 0) atomicAdd(inserted + 2, (unsigned long long)n_cand);
     __syncthreads();
 
     // 5. survivors: closer than the current worst
-    const float worst = own_dist[K - 1];
     for (uint32_t j = tid; j < n_cand; j += NND_THREADS)
         if (cand_dist[j] < worst) surv[atomicAdd(&ctl[6], 1u)] = dist_id_key(cand_dist[j], cand_id[j]);
     __syncthreads();
@@ -206,17 +222,20 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
         ids[base + j] = e;
         dist[base + j] = dv;
         const uint32_t v = e & ~FLAG;
+        // (distance, u) travels as one 64-bit word, so a slot never holds the id of one writer with
+        // the distance of another; beyond K registrations slot (count % K) keeps the closer one
         const uint32_t slot = atomicAdd(&rev_cnt[v], 1u);
-        const size_t at = (size_t)v * K + (slot % K);
-        if (slot < K || dv < rev_dist[at]) { rev[at] = u; rev_dist[at] = dv; }
+        const unsigned long long key = dist_id_key(dv, u);
+        unsigned long long* at = rev + (size_t)v * K + (slot % K);
+        if (slot < K) *at = key;
+        else atomicMin(at, key);
     }
     if (tid == 0) atomicAdd(inserted, (unsigned long long)ctl[7]);
 }
 
 // Merge with the reverse neighbours registered in the last step (index.cu:386-478).
 __global__ __launch_bounds__(NND_THREADS) void nnd_merge_reverse_kernel(uint32_t n, uint32_t K, uint32_t* ids, float* dist,
-                                                                        const uint32_t* rev, const float* rev_dist,
-                                                                        const uint32_t* rev_cnt) {
+                                                                        const unsigned long long* rev, const uint32_t* rev_cnt) {
     extern __shared__ __align__(16) char smem[];
     uint64_t* surv = reinterpret_cast<uint64_t*>(smem);
     uint64_t* new_sorted = surv + K;
@@ -234,8 +253,9 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_merge_reverse_kernel(uint32_t
     for (uint32_t i = tid; i < K; i += NND_THREADS) {
         own_id[i] = ids[base + i];
         own_dist[i] = dist[base + i];
-        r_id[i] = i < cnt ? rev[base + i] : EMPTY;
-        r_dist[i] = i < cnt ? rev_dist[base + i] : INF_DIS;
+        const unsigned long long rk = i < cnt ? rev[base + i] : ~0ull;
+        r_id[i] = (uint32_t)rk;
+        r_dist[i] = r_id[i] != EMPTY ? key_dist(rk) : INF_DIS;
     }
     if (tid < 4) ctl[tid] = 0;
     __syncthreads();
@@ -260,9 +280,10 @@ static uint32_t doc_term_slots(const apoe_corpus* c) { return next_pow2(std::max
 
 int launch_nnd_init(apoe_knn* g, uint64_t seed) {
     apoe_ctx* ctx = g->ctx;
+    APOE_HIP(hipMemsetAsync(g->counter.p, 0, 4 * sizeof(unsigned long long), ctx->stream));
     const uint64_t total = (uint64_t)g->n * g->K;
     const uint32_t grid = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
-    nnd_init_kernel<<<grid, 256, 0, ctx->stream>>>(g->n, g->K, seed, g->ids.p, g->dist.p, g->rev.p, g->rev_dist.p, g->rev_cnt.p);
+    nnd_init_kernel<<<grid, 256, 0, ctx->stream>>>(g->n, g->K, seed, g->ids.p, g->dist.p, g->rev.p, g->rev_cnt.p);
     APOE_HIP(hipGetLastError());
     return launch_norms(ctx, g->corpus, g->dense_scale, g->norms.p);
 }
@@ -274,10 +295,10 @@ int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted) {
     const NndLds L(term_slots, seen_slots, g->K);
     APOE_REQUIRE(L.total <= 64 * 1024, "NN-Descent needs %u bytes of LDS (rows with up to %u sparse terms)", L.total,
                  g->corpus->max_nnz_s + g->corpus->max_nnz_b);
-    APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), ctx->stream));
+    APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), ctx->stream)); // [0] inserted; [2], [3] accumulate over the build
     APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_iterate_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
     nnd_iterate_kernel<<<g->n, NND_THREADS, L.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->K, g->ids.p, g->dist.p,
-                                                                    g->rev.p, g->rev_dist.p, g->rev_cnt.p, term_slots, seen_slots, g->counter.p);
+                                                                    g->rev.p, g->rev_cnt.p, term_slots, seen_slots, g->counter.p);
     APOE_HIP(hipGetLastError());
     if (inserted) {
         unsigned long long h = 0;
@@ -291,7 +312,7 @@ int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted) {
 int launch_nnd_merge_reverse(apoe_knn* g) {
     apoe_ctx* ctx = g->ctx;
     const size_t lds = (size_t)g->K * (8 + 8 + 4 * 6) + 16;
-    nnd_merge_reverse_kernel<<<g->n, NND_THREADS, lds, ctx->stream>>>(g->n, g->K, g->ids.p, g->dist.p, g->rev.p, g->rev_dist.p, g->rev_cnt.p);
+    nnd_merge_reverse_kernel<<<g->n, NND_THREADS, lds, ctx->stream>>>(g->n, g->K, g->ids.p, g->dist.p, g->rev.p, g->rev_cnt.p);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
 }
@@ -318,7 +339,6 @@ int apoe_knn_create(apoe_ctx* ctx, const apoe_corpus* c, uint32_t K, float dense
     APOE_TRY(g->ids.alloc(total));
     APOE_TRY(g->dist.alloc(total));
     APOE_TRY(g->rev.alloc(total));
-    APOE_TRY(g->rev_dist.alloc(total));
     APOE_TRY(g->rev_cnt.alloc(c->n));
     APOE_TRY(g->norms.alloc(c->n));
     APOE_TRY(g->counter.alloc(4));
@@ -405,5 +425,16 @@ int apoe_knn_upload(apoe_knn* g, const uint32_t* ids, const float* dist) {
 }
 
 float apoe_knn_elapsed_ms(const apoe_knn* g) { return g ? g->elapsed_ms : 0.f; }
+
+int apoe_knn_counters(apoe_knn* g, uint64_t* out2) {
+    APOE_REQUIRE(g && out2, "null argument");
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    unsigned long long h[4] = {0, 0, 0, 0};
+    APOE_HIP(hipStreamSynchronize(g->ctx->stream));
+    APOE_HIP(hipMemcpy(h, g->counter.p, sizeof(h), hipMemcpyDeviceToHost));
+    out2[0] = h[2];
+    out2[1] = h[3];
+    return APOE_OK;
+}
 
 } // extern "C"

@@ -5,7 +5,8 @@
 
 namespace apoe {
 
-constexpr int MAX_NEW = 64; // fresh candidates per step: one lane each in wave 0
+constexpr int MAX_NEW = 64;   // fresh candidates per step: one lane each in wave 0
+constexpr int EVAL_BATCH = 2; // candidates whose sparse parts a wave keeps in flight together
 
 struct SearchArgs {
     CorpusView C;
@@ -21,7 +22,8 @@ struct SearchArgs {
     float* out_dist;
     uint32_t* bitmaps;     // one visited bitmap per workgroup
     uint32_t bitmap_words; // multiple of 4
-    unsigned long long* work; // [0] next query, [1] expansions, [2] evaluations, [3] nnz splade, [4] nnz bm25
+    unsigned long long* work; // [0] next query, [1] expansions, [2] evaluations, [3] nnz splade, [4] nnz bm25, [5] dense rows read
+    uint32_t full_eval;       // 1: read the dense row of every candidate (no bound test)
     uint32_t slots;
     // knowledge graph (KG kernels only)
     const uint32_t *e2e_off, *e2e_idx, *e2d_off, *e2d_idx, *q2e_off, *q2e_idx;
@@ -138,7 +140,7 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t cur, uint
 }
 
 template <int NW, bool KG>
-__global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
+__global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))) void search_kernel(SearchArgs a) {
     extern __shared__ __align__(16) char smem[];
     const SearchLds L(a.slots, a.cands, KG);
     uint2* tab = reinterpret_cast<uint2*>(smem + L.tab);
@@ -188,7 +190,8 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
         __syncthreads();
         pivot_terms_from_query(tab, mask, a.Q, q, a.w_s, a.w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
 
-        uint64_t st_exp = 0, st_eval = 0, st_ns = 0, st_nb = 0; // wave-uniform counters
+        const float pv_norm = pivot_dense_norm(pv);
+        uint64_t st_exp = 0, st_eval = 0, st_ns = 0, st_nb = 0, st_dense = 0; // wave-uniform counters
         uint32_t cur = 0;                                        // live pool half (wave 0's copy is authoritative)
 
         // ---- seeds ----
@@ -203,7 +206,7 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
                 }
                 const uint64_t b = __ballot(fresh);
                 if (fresh) new_id[__popcll(b & lane_lt)] = c;
-                if (lane == 0) { ctl[CTL_NNEW] = __popcll(b); ctl[CTL_PARENT] = 0; }
+                if (lane == 0) { ctl[CTL_NNEW] = __popcll(b); ctl[CTL_PARENT] = 0; ctl[CTL_CUR] = 0; }
             }
             __syncthreads();
         } else {
@@ -248,11 +251,13 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
             const uint32_t n_seed = ctl[CTL_NSEED];
             for (uint32_t j = wave; j < n_seed; j += NW) {
                 const uint32_t id = uniform(seed_id[j]);
-                EvalOut e = eval_wave(a.C, id, pv, tab, mask, a.paths, 1.0f);
+                const float bonus = seed_ent[j] != EMPTY ? a.kg_weight : 0.0f; // query.cu:1637-1638
+                BoundedOut e = eval_wave_bounded(a.C, id, pv, pv_norm, tab, mask, a.paths, 1.0f, bonus, __builtin_inff());
                 st_eval++;
                 st_ns += e.nnz_s;
                 st_nb += e.nnz_b;
-                if (lane == 0) seed_dist[j] = 1.0f - e.ip - (seed_ent[j] != EMPTY ? a.kg_weight : 0.0f); // query.cu:1637-1638
+                st_dense += e.dense_read;
+                if (lane == 0) seed_dist[j] = e.dist;
             }
             __syncthreads();
             if (wave == 0) {
@@ -276,17 +281,33 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
             // ---- evaluate the fresh candidates: one wave per candidate ----
             const uint32_t n_new = ctl[CTL_NNEW];
             if (ctl[CTL_PARENT] == EMPTY) break;
-            for (uint32_t j = wave; j < n_new; j += NW) {
-                const uint32_t id = uniform(new_id[j]);
-                EvalOut e = eval_wave(a.C, id, pv, tab, mask, a.paths, 1.0f);
-                st_eval++;
-                st_ns += e.nnz_s;
-                st_nb += e.nnz_b;
-                float dist = 1.0f - e.ip;
-                if (KG) {
-                    if (new_ent[j] != EMPTY) dist -= a.kg_weight / (float)new_hop[j]; // query.cu:1759-1760
+            // a candidate that provably cannot enter the (full) pool is dropped after its sparse part:
+            // it is reported as INF_DIS and falls off the end of the merge like any other loser
+            const float thr = a.full_eval ? __builtin_inff() : P.dist[ctl[CTL_CUR] * cands + cands - 1];
+            const float thr_eff = thr < INF_DIS ? thr : __builtin_inff();
+            for (uint32_t j = wave; j < n_new; j += NW * EVAL_BATCH) {
+                PendingEval pe[EVAL_BATCH];
+#pragma unroll
+                for (int b = 0; b < EVAL_BATCH; b++) {
+                    const uint32_t jj = j + b * NW;
+                    if (jj < n_new) eval_issue(pe[b], a.C, uniform(new_id[jj]), pv_norm, a.paths, 1.0f);
                 }
-                if (lane == 0) new_dist[j] = dist;
+#pragma unroll
+                for (int b = 0; b < EVAL_BATCH; b++) {
+                    const uint32_t jj = j + b * NW;
+                    if (jj < n_new) {
+                        float bonus = 0.f;
+                        if (KG) {
+                            if (new_ent[jj] != EMPTY) bonus = a.kg_weight / (float)new_hop[jj]; // query.cu:1759-1760
+                        }
+                        BoundedOut e = eval_finish(pe[b], pv, tab, mask, a.paths, 1.0f, bonus, thr_eff);
+                        st_eval++;
+                        st_ns += e.nnz_s;
+                        st_nb += e.nnz_b;
+                        st_dense += e.dense_read;
+                        if (lane == 0) new_dist[jj] = e.dist;
+                    }
+                }
             }
             __syncthreads();
             // ---- wave 0: merge, pick the next parent, fetch its neighbours ----
@@ -415,6 +436,7 @@ __global__ __launch_bounds__(NW* WAVE) void search_kernel(SearchArgs a) {
             if (st_eval) atomicAdd(a.work + 2, st_eval);
             if (st_ns) atomicAdd(a.work + 3, st_ns);
             if (st_nb) atomicAdd(a.work + 4, st_nb);
+            if (st_dense) atomicAdd(a.work + 5, st_dense);
         }
     }
 }
@@ -458,6 +480,7 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     a.out_dist = out_dist_dev;
     a.slots = next_pow2(std::max(64u, 2 * q->max_nnz));
     a.kg_weight = p->kg_weight;
+    a.full_eval = (p->variant & 0x100u) ? 1u : 0u;
 
     const bool use_kg = kg != nullptr;
     if (use_kg) {
@@ -475,9 +498,10 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
 
     // variant 0: two waves per query (the measured best); 1, 2, 3: one, four, eight waves
     int nw = 2;
-    if (p->variant == 1) nw = 1;
-    else if (p->variant == 2) nw = 4;
-    else if (p->variant == 3) nw = 8;
+    const uint32_t shape = p->variant & 0xFFu;
+    if (shape == 1) nw = 1;
+    else if (shape == 2) nw = 4;
+    else if (shape == 3) nw = 8;
     // persistent grid: as many workgroups as can be resident, never more than queries
     int per_cu = 1;
     {
@@ -525,10 +549,10 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
         stats->evaluations = h[2];
         stats->nnz_sparse = h[3];
         stats->nnz_bm25 = h[4];
-        // rows + pairs + descriptor (8 B ~ the two CSR offset pairs' 16 B of the reference layout)
-        uint64_t bytes = 0;
-        if (a.paths & PATH_DENSE) bytes += h[2] * (uint64_t)DENSE_BYTES;
-        bytes += 8 * (h[3] + h[4]) + 8 * h[2];
+        stats->dense_rows = h[5];
+        // dense rows actually needed + pairs + descriptor and dense norm (12 B per evaluation)
+        uint64_t bytes = h[5] * (uint64_t)DENSE_BYTES;
+        bytes += 8 * (h[3] + h[4]) + 12 * h[2];
         bytes += h[1] * 4ull * a.W;
         uint64_t qbytes = (uint64_t)q_count * DENSE_BYTES + 8 * (q->h_s_off[p->q_begin + q_count] - q->h_s_off[p->q_begin]) +
                           8 * (q->h_b_off[p->q_begin + q_count] - q->h_b_off[p->q_begin]);

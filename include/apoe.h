@@ -135,6 +135,10 @@ int apoe_finalize_graph(apoe_knn* g, apoe_graph** out);
 /* Milliseconds of GPU time (HIP events on the context stream) spent in the build
  * calls on this handle so far: the reference's "Indexing time" region (index.cu:889-908). */
 float apoe_knn_elapsed_ms(const apoe_knn* g);
+/* out2 = {hybrid distance evaluations, dense rows read} of the NN-Descent steps since apoe_nnd_init
+ * (a candidate whose sparse part plus the bound of its dense part cannot enter the list is not
+ * read in full). No counterpart in the reference; used to price the build against the HBM roofline. */
+int apoe_knn_counters(apoe_knn* g, uint64_t* out2);
 
 /* ---- graph handle: the .poe payload (index.cu:927-939, query.cu:35-62) ---- */
 int apoe_graph_create(apoe_ctx* ctx, uint32_t n, uint32_t width, const uint32_t* rows,
@@ -151,7 +155,11 @@ typedef struct {
     uint32_t cands;                  /* pool size, 1..APOE_MAX_CANDS */
     uint32_t max_iter;               /* 0 -> 1000 (query.cu:7 MAX_ITER) */
     uint32_t q_begin, q_count;       /* query range; q_count 0 -> all from q_begin */
-    uint32_t variant;                /* 0 = default launch shape; others are tuning shapes */
+    uint32_t variant;                /* low byte: launch shape, 0 = default (2 waves per query), 1/2/3 =
+                                        1/4/8 waves. 0x100: read the dense row of every candidate; by
+                                        default a candidate whose sparse part plus the Cauchy-Schwarz
+                                        bound of its dense part cannot beat the worst entry of the full
+                                        pool is dropped without reading its dense row (same results) */
 } apoe_search_params;
 
 typedef struct {
@@ -160,8 +168,9 @@ typedef struct {
     uint64_t evaluations; /* hybrid distance evaluations */
     uint64_t nnz_sparse;  /* SPLADE pairs read by those evaluations (0 if path off) */
     uint64_t nnz_bm25;    /* BM25 pairs read by those evaluations (0 if path off) */
-    uint64_t algo_bytes;  /* algorithmic HBM bytes: rows + pairs + descriptors + graph rows
-                             + queries + results */
+    uint64_t dense_rows;  /* evaluations that had to read the 4 KB dense row (see variant) */
+    uint64_t algo_bytes;  /* algorithmic HBM bytes: dense rows read + pairs + descriptors + graph
+                             rows + queries + results */
 } apoe_search_stats;
 
 /* out_ids/out_dist are [q_count][cands], ascending distance; top_k is the row
