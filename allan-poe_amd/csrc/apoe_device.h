@@ -360,21 +360,35 @@ struct PendingEval {
     float dub;
 };
 
-__device__ __forceinline__ void eval_issue(PendingEval& p, const CorpusView& C, uint32_t id, float pv_norm, uint32_t paths, float dense_mul) {
+// desc / dnorm are the candidate's descriptor and dense norm (wave-uniform).
+__device__ __forceinline__ void eval_issue_desc(PendingEval& p, const CorpusView& C, uint64_t desc, float dnorm, float pv_norm, uint32_t paths,
+                                                float dense_mul) {
     const int lane = lane_id();
-    const uint64_t desc = C.desc[id];
     p.rec = C.recs + desc_off(desc) * 16;
     p.ns = desc_nnz_s(desc);
     p.nb = desc_nnz_b(desc);
     p.begin = (paths & PATH_SPARSE) ? 0u : p.ns;
     p.end = (paths & PATH_BM25) ? p.ns + p.nb : p.ns;
-    p.dub = (paths & PATH_DENSE) ? dense_mul * pv_norm * C.dnorm[id] : 0.f;
+    p.dub = (paths & PATH_DENSE) ? dense_mul * pv_norm * dnorm : 0.f;
     const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
     const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
     p.kv0 = p.kv1 = p.kv2 = make_uint2(0, 0);
     if (j0 < p.end) p.kv0 = sp[j0];
     if (j1 < p.end) p.kv1 = sp[j1];
     if (j2 < p.end) p.kv2 = sp[j2];
+}
+
+__device__ __forceinline__ void eval_issue(PendingEval& p, const CorpusView& C, uint32_t id, float pv_norm, uint32_t paths, float dense_mul) {
+    eval_issue_desc(p, C, C.desc[id], C.dnorm[id], pv_norm, paths, dense_mul);
+}
+
+// Lane `src` of a 64-bit / float register as a wave-uniform value (src is wave-uniform).
+__device__ __forceinline__ uint64_t readlane64(uint64_t v, uint32_t src) {
+    const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)v, src), hi = __builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), src);
+    return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ float readlane_f32(float v, uint32_t src) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
 }
 
 __device__ __forceinline__ BoundedOut eval_finish(const PendingEval& p, const PivotDense& pv, const uint2* tab, uint32_t mask, uint32_t paths,

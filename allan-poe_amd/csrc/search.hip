@@ -285,12 +285,20 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             // it is reported as INF_DIS and falls off the end of the merge like any other loser
             const float thr = a.full_eval ? __builtin_inff() : P.dist[ctl[CTL_CUR] * cands + cands - 1];
             const float thr_eff = thr < INF_DIS ? thr : __builtin_inff();
+            // descriptors and dense norms of all fresh candidates in one gather: lane l holds candidate l's
+            uint64_t my_desc = 0;
+            float my_dn = 0.f;
+            if ((uint32_t)lane < n_new) {
+                const uint32_t cid = new_id[lane];
+                my_desc = a.C.desc[cid];
+                my_dn = a.C.dnorm[cid];
+            }
             for (uint32_t j = wave; j < n_new; j += NW * EVAL_BATCH) {
                 PendingEval pe[EVAL_BATCH];
 #pragma unroll
                 for (int b = 0; b < EVAL_BATCH; b++) {
                     const uint32_t jj = j + b * NW;
-                    if (jj < n_new) eval_issue(pe[b], a.C, uniform(new_id[jj]), pv_norm, a.paths, 1.0f);
+                    if (jj < n_new) eval_issue_desc(pe[b], a.C, readlane64(my_desc, jj), readlane_f32(my_dn, jj), pv_norm, a.paths, 1.0f);
                 }
 #pragma unroll
                 for (int b = 0; b < EVAL_BATCH; b++) {
