@@ -33,14 +33,15 @@ struct SearchArgs {
 
 // LDS carve-up shared by host (size) and device (pointers).
 struct SearchLds {
-    uint32_t tab, pool_id, pool_dist, pool_ent, pool_hop, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ctl, total;
+    uint32_t tab, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ctl, total;
     __host__ __device__ SearchLds(uint32_t slots, uint32_t cands, bool kg) {
         uint32_t o = 0;
         tab = o; o += slots * 8;
-        pool_id = o; o += 2 * cands * 4;
-        pool_dist = o; o += 2 * cands * 4;
-        pool_ent = o; o += kg ? 2 * cands * 4 : 0;
-        pool_hop = o; o += kg ? 2 * cands * 4 : 0;
+        pool_id = o; o += cands * 4;
+        pool_dist = o; o += cands * 4;
+        pool_ent = o; o += kg ? cands * 4 : 0;
+        pool_hop = o; o += kg ? cands * 4 : 0;
+        new_lb = o; o += MAX_NEW * 4;
         new_id = o; o += MAX_NEW * 4;
         new_dist = o; o += MAX_NEW * 4;
         new_ent = o; o += kg ? MAX_NEW * 4 : 0;
@@ -54,13 +55,14 @@ struct SearchLds {
     }
 };
 
-enum { CTL_QUERY = 0, CTL_PARENT = 1, CTL_NNEW = 2, CTL_CUR = 3, CTL_PENT = 4, CTL_PHOP = 5, CTL_NSEED = 6 };
+enum { CTL_QUERY = 0, CTL_PARENT = 1, CTL_NNEW = 2, CTL_NSEED = 3 };
 
 struct Pool {
-    uint32_t* id;   // [2][cands]
-    float* dist;    // [2][cands]
+    uint32_t* id;   // [cands], ascending distance
+    float* dist;    // [cands]
     uint32_t* ent;  // KG only
     uint32_t* hop;  // KG only
+    uint32_t* lb;   // [MAX_NEW] scratch of the merge
     uint32_t cands;
 };
 
@@ -69,74 +71,86 @@ __device__ __forceinline__ void wave_fence() {
     __builtin_amdgcn_wave_barrier();
 }
 
-// Wave 0 only. Sorts the n (<= 64) new candidates by (distance, id) and rank-merges
-// them into the pool (source half `cur`, destination half `cur ^ 1`): a pool element
-// keeps rank pos + #{new <= it}, a new element takes rank pos + #{pool < it}, so on
-// equal distance the new one goes first; ranks >= cands fall off. Returns cur ^ 1.
+// Wave 0 only. Orders the n (<= 64) new candidates by (distance, id) and merges them into the
+// sorted pool in place: a pool element keeps rank pos + #{new <= it}, a new element takes rank
+// pos + #{pool < it}, so on equal distance the new one goes first (query.cu:181-224); ranks >=
+// cands fall off. With lb_i = #{pool < new_i}: new_i <= pool[p]  <=>  lb_i <= p, so a pool element
+// moves up by the number of new elements whose lb is <= its position, and nothing below lb_0
+// moves at all -- only the 64-element rounds from the top down to lb_0 are touched (each round
+// is read into registers before anything at or above it is written). Returns the lowest rank a
+// new element took (cands if none entered).
 template <bool KG>
-__device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t cur, uint32_t* nid, float* ndist, uint32_t* nent, uint32_t* nhop,
-                                               uint32_t n) {
+__device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, float* ndist, uint32_t* nent, uint32_t* nhop, uint32_t n) {
     const int lane = lane_id();
     const uint32_t cands = P.cands;
-    float d = lane < (int)n ? ndist[lane] : INF_DIS;
-    uint32_t id = lane < (int)n ? nid[lane] : EMPTY;
-    uint64_t key = lane < (int)n ? dist_id_key(d, id) : ~0ull;
-    uint32_t ent = EMPTY, hop = 0;
-    if (KG) {
-        if (lane < (int)n) { ent = nent[lane]; hop = nhop[lane]; }
-        // the distance travels inside the key; payloads travel beside it
-        wave_sort64_payload(key, ent, hop);
-    } else {
-        key = wave_sort64(key);
-    }
-    wave_fence();
-    id = (uint32_t)key;
-    {   // recover the float from its order-preserving key
-        uint32_t u = (uint32_t)(key >> 32);
-        u ^= (u >> 31) ? 0x80000000u : 0xFFFFFFFFu;
-        d = __uint_as_float(u);
-    }
-    if (lane >= (int)n) { d = INF_DIS; id = EMPTY; }
-    ndist[lane] = d; // sorted copy for the pool elements' searches
-    wave_fence();
-    const uint32_t* sid = P.id + cur * cands;
-    const float* sdist = P.dist + cur * cands;
-    uint32_t* did = P.id + (cur ^ 1) * cands;
-    float* ddist = P.dist + (cur ^ 1) * cands;
-    // new element: lower_bound over the pool
+    if (n == 0) return cands;
+    // order by counting: rank = #{(d, id) pairs below mine}; ids are distinct
+    float d = INF_DIS;
+    uint32_t id = EMPTY, ent = EMPTY, hop = 0, rank = 0;
     if (lane < (int)n) {
-        uint32_t lo = 0, len = cands;
-        while (len > 0) {
-            uint32_t half = len >> 1;
-            if (sdist[lo + half] < d) { lo += half + 1; len -= half + 1; } else len = half;
-        }
-        uint32_t rank = lo + lane;
-        if (rank < cands) {
-            did[rank] = id;
-            ddist[rank] = d;
-            if (KG) { P.ent[(cur ^ 1) * cands + rank] = ent; P.hop[(cur ^ 1) * cands + rank] = hop; }
-        }
-    }
-    // pool element: upper_bound over the sorted new list
-    for (uint32_t base = 0; base < cands; base += WAVE) {
-        uint32_t p = base + lane;
-        if (p < cands) {
-            float v = sdist[p];
-            uint32_t lo = 0, len = n;
-            while (len > 0) {
-                uint32_t half = len >> 1;
-                if (ndist[lo + half] <= v) { lo += half + 1; len -= half + 1; } else len = half;
-            }
-            uint32_t rank = p + lo;
-            if (rank < cands) {
-                did[rank] = sid[p];
-                ddist[rank] = v;
-                if (KG) { P.ent[(cur ^ 1) * cands + rank] = P.ent[cur * cands + p]; P.hop[(cur ^ 1) * cands + rank] = P.hop[cur * cands + p]; }
-            }
+        d = ndist[lane];
+        id = nid[lane];
+        if (KG) { ent = nent[lane]; hop = nhop[lane]; }
+        for (uint32_t i = 0; i < n; i++) {
+            const float di = ndist[i];
+            const uint32_t ii = nid[i];
+            rank += (di < d) || (di == d && ii < id);
         }
     }
     wave_fence();
-    return cur ^ 1;
+    if (lane < (int)n) {
+        ndist[rank] = d;
+        nid[rank] = id;
+        if (KG) { nent[rank] = ent; nhop[rank] = hop; }
+    }
+    wave_fence();
+    // lane i now takes the i-th smallest
+    uint32_t lb = cands;
+    if (lane < (int)n) {
+        d = ndist[lane];
+        id = nid[lane];
+        if (KG) { ent = nent[lane]; hop = nhop[lane]; }
+        if (d <= P.dist[cands - 1]) {
+            uint32_t lo = 0, len = cands;
+            while (len > 0) {
+                const uint32_t half = len >> 1;
+                if (P.dist[lo + half] < d) { lo += half + 1; len -= half + 1; } else len = half;
+            }
+            lb = lo;
+        }
+        P.lb[lane] = lb;
+    }
+    const bool enters = lane < (int)n && lb + lane < cands;
+    const uint32_t n_in = __popcll(__ballot(enters)); // ranks grow with the lane: the first n_in enter
+    if (n_in == 0) return cands;
+    wave_fence();
+    const uint32_t lo0 = P.lb[0];
+    for (int base = (int)((cands - 1) & ~(uint32_t)(WAVE - 1)); base >= 0 && (uint32_t)base + WAVE > lo0; base -= WAVE) {
+        const uint32_t p = base + lane;
+        const bool act = p >= lo0 && p < cands;
+        float v = 0.f;
+        uint32_t pid = 0, pent = 0, phop = 0, shift = 0;
+        if (act) {
+            v = P.dist[p];
+            pid = P.id[p];
+            if (KG) { pent = P.ent[p]; phop = P.hop[p]; }
+            for (uint32_t i = 0; i < n_in; i++) shift += P.lb[i] <= p;
+        }
+        wave_fence();
+        if (act && p + shift < cands) {
+            P.dist[p + shift] = v;
+            P.id[p + shift] = pid;
+            if (KG) { P.ent[p + shift] = pent; P.hop[p + shift] = phop; }
+        }
+        wave_fence();
+    }
+    if (enters) {
+        P.dist[lb + lane] = d;
+        P.id[lb + lane] = id;
+        if (KG) { P.ent[lb + lane] = ent; P.hop[lb + lane] = hop; }
+    }
+    wave_fence();
+    return lo0;
 }
 
 template <int NW, bool KG>
@@ -149,6 +163,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
     P.dist = reinterpret_cast<float*>(smem + L.pool_dist);
     P.ent = reinterpret_cast<uint32_t*>(smem + L.pool_ent);
     P.hop = reinterpret_cast<uint32_t*>(smem + L.pool_hop);
+    P.lb = reinterpret_cast<uint32_t*>(smem + L.new_lb);
     P.cands = a.cands;
     uint32_t* new_id = reinterpret_cast<uint32_t*>(smem + L.new_id);
     float* new_dist = reinterpret_cast<float*>(smem + L.new_dist);
@@ -192,7 +207,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
 
         const float pv_norm = pivot_dense_norm(pv);
         uint64_t st_exp = 0, st_eval = 0, st_ns = 0, st_nb = 0, st_dense = 0; // wave-uniform counters
-        uint32_t cur = 0;                                        // live pool half (wave 0's copy is authoritative)
+        uint32_t hint = 0;                                       // wave 0: every pool slot below hint is explored
 
         // ---- seeds ----
         if (!KG) {
@@ -206,7 +221,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                 }
                 const uint64_t b = __ballot(fresh);
                 if (fresh) new_id[__popcll(b & lane_lt)] = c;
-                if (lane == 0) { ctl[CTL_NNEW] = __popcll(b); ctl[CTL_PARENT] = 0; ctl[CTL_CUR] = 0; }
+                if (lane == 0) { ctl[CTL_NNEW] = __popcll(b); ctl[CTL_PARENT] = 0; }
             }
             __syncthreads();
         } else {
@@ -270,9 +285,9 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                         new_hop[lane] = 0;
                     }
                     wave_fence();
-                    cur = sort_merge<KG>(P, cur, new_id, new_dist, new_ent, new_hop, nb);
+                    sort_merge<KG>(P, new_id, new_dist, new_ent, new_hop, nb);
                 }
-                if (lane == 0) { ctl[CTL_NNEW] = 0; ctl[CTL_PARENT] = 0; ctl[CTL_CUR] = cur; }
+                if (lane == 0) { ctl[CTL_NNEW] = 0; ctl[CTL_PARENT] = 0; }
             }
             __syncthreads();
         }
@@ -283,7 +298,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             if (ctl[CTL_PARENT] == EMPTY) break;
             // a candidate that provably cannot enter the (full) pool is dropped after its sparse part:
             // it is reported as INF_DIS and falls off the end of the merge like any other loser
-            const float thr = a.full_eval ? __builtin_inff() : P.dist[ctl[CTL_CUR] * cands + cands - 1];
+            const float thr = a.full_eval ? __builtin_inff() : P.dist[cands - 1];
             const float thr_eff = thr < INF_DIS ? thr : __builtin_inff();
             // descriptors and dense norms of all fresh candidates in one gather: lane l holds candidate l's
             uint64_t my_desc = 0;
@@ -320,12 +335,11 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             __syncthreads();
             // ---- wave 0: merge, pick the next parent, fetch its neighbours ----
             if (wave == 0) {
-                cur = sort_merge<KG>(P, cur, new_id, new_dist, new_ent, new_hop, n_new);
+                hint = min(hint, sort_merge<KG>(P, new_id, new_dist, new_ent, new_hop, n_new));
                 uint32_t parent = EMPTY, slot = 0, n_next = 0;
                 if (it < a.max_iter) {
-                    const uint32_t* pid = P.id + cur * cands;
-                    for (uint32_t base = 0; base < cands; base += WAVE) {
-                        const uint32_t id = base + lane < cands ? pid[base + lane] : EMPTY;
+                    for (uint32_t base = hint & ~(uint32_t)(WAVE - 1); base < cands; base += WAVE) {
+                        const uint32_t id = base + lane < cands ? P.id[base + lane] : EMPTY;
                         const uint64_t b = __ballot((id & FLAG) == 0);
                         if (b) {
                             const int l = __ffsll((unsigned long long)b) - 1;
@@ -334,11 +348,12 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                             break;
                         }
                     }
+                    hint = parent != EMPTY ? slot + 1 : cands;
                 }
                 if (parent != EMPTY) {
                     uint32_t p_ent = EMPTY, p_hop = 0;
-                    if (KG) { p_ent = P.ent[cur * cands + slot]; p_hop = P.hop[cur * cands + slot]; }
-                    if (lane == 0) P.id[cur * cands + slot] = parent | FLAG;
+                    if (KG) { p_ent = P.ent[slot]; p_hop = P.hop[slot]; }
+                    if (lane == 0) P.id[slot] = parent | FLAG;
                     st_exp++;
                     uint32_t c = lane < (int)a.degree ? a.graph[(size_t)parent * a.W + lane] : EMPTY;
                     bool fresh = false;
@@ -429,15 +444,14 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                     }
                     n_next = __popcll(b);
                 }
-                if (lane == 0) { ctl[CTL_PARENT] = parent; ctl[CTL_NNEW] = n_next; ctl[CTL_CUR] = cur; }
+                if (lane == 0) { ctl[CTL_PARENT] = parent; ctl[CTL_NNEW] = n_next; }
             }
             __syncthreads();
         }
         // ---- results (query.cu:566-569) ----
-        cur = ctl[CTL_CUR];
         for (uint32_t i = tid; i < cands; i += NW * WAVE) {
-            a.out_ids[(size_t)qi * cands + i] = P.id[cur * cands + i] & ~FLAG;
-            a.out_dist[(size_t)qi * cands + i] = P.dist[cur * cands + i];
+            a.out_ids[(size_t)qi * cands + i] = P.id[i] & ~FLAG;
+            a.out_dist[(size_t)qi * cands + i] = P.dist[i];
         }
         if (lane == 0) {
             if (st_exp) atomicAdd(a.work + 1, st_exp);
