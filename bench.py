@@ -23,7 +23,13 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per search launch from FETCH_SIZE + WRITE_SIZE counter runs (rocprofv3 --pmc,
 # scaled by what the counters read for a 1 GiB copy), keyed by the workload they were taken on:
 # (docs, degree, queries, cands, variant). Other workloads report null.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    (1000000, 48, 10000, 512, 0): 391340624251,
+}
+# The same for the launches that read every dense row (variant | 0x100).
+MEASURED_TRAFFIC_FULL = {
+    (1000000, 48, 10000, 512, 0): 978286162104,
+}
 
 
 def log(*a):
@@ -192,7 +198,9 @@ def main():
             full_bytes = stf.algo_bytes
     full_avg = sum(full_ms) / len(full_ms)
     full_eval = {"kernel_ms": full_avg, "qps": args.queries / (full_avg / 1e3), "achieved": full_bytes / (full_avg / 1e3) / 1e9,
-                 "frac": full_bytes / (full_avg / 1e3) / 1e9 / HBM_PEAK_GBS, "algo_bytes_per_launch": full_bytes}
+                 "frac": full_bytes / (full_avg / 1e3) / 1e9 / HBM_PEAK_GBS, "algo_bytes_per_launch": full_bytes,
+                 "traffic": MEASURED_TRAFFIC_FULL.get((args.docs, args.degree, args.queries, cands, args.variant))
+                 if not args.calibrate else None}
     log(f"[bench] timed: {avg_kernel_ms:.2f} ms/launch, {achieved:.0f} GB/s algorithmic; every dense row read: {full_avg:.2f} ms, "
         f"{full_eval['achieved']:.0f} GB/s")
 
