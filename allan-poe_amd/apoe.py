@@ -26,7 +26,7 @@ class ApoeError(RuntimeError):
 class SearchParams(C.Structure):
     _fields_ = [("w_dense", C.c_float), ("w_sparse", C.c_float), ("w_bm25", C.c_float), ("kg_weight", C.c_float),
                 ("cands", C.c_uint32), ("max_iter", C.c_uint32), ("q_begin", C.c_uint32), ("q_count", C.c_uint32),
-                ("variant", C.c_uint32)]
+                ("variant", C.c_uint32), ("keyword_filter", C.c_uint32)]
 
 
 class SearchStats(C.Structure):
@@ -328,14 +328,16 @@ def calibrate_weights(ctx, corpus, queries, w3, n_queries=None):
 
 
 def search(ctx, corpus, queries, graph, w3, cands, kg=None, kg_weight=0.0, max_iter=0, q_begin=0, q_count=0, variant=0,
-           out_ids=None, out_dist=None):
-    """Returns (ids [q, cands] u32, dist [q, cands] f32, SearchStats). w3 = (dense, sparse, bm25)."""
+           out_ids=None, out_dist=None, keyword_filter=False):
+    """Returns (ids [q, cands] u32, dist [q, cands] f32, SearchStats). w3 = (dense, sparse, bm25).
+    keyword_filter: rows hold only documents with a BM25 term that the query flags (bit 31 of the
+    query's BM25 term id) as a required keyword."""
     nq = q_count if q_count else queries.n - q_begin
     if out_ids is None:
         out_ids = np.empty((nq, cands), np.uint32)
         out_dist = np.empty((nq, cands), np.float32)
     ki, kd = _ptr(out_ids, np.uint32), _ptr(out_dist, np.float32)
-    p = SearchParams(w3[0], w3[1], w3[2], kg_weight, cands, max_iter, q_begin, q_count, variant)
+    p = SearchParams(w3[0], w3[1], w3[2], kg_weight, cands, max_iter, q_begin, q_count, variant, 1 if keyword_filter else 0)
     st = SearchStats()
     _check(lib().apoe_search(ctx.h, corpus.h, queries.h, graph.h, kg.h if kg is not None else C.c_void_p(0), C.byref(p), ki[1], kd[1],
                              C.byref(st)))

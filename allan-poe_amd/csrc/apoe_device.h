@@ -12,6 +12,8 @@ constexpr int WAVE = 64;
 constexpr uint32_t EMPTY = 0xFFFFFFFFu;
 constexpr uint32_t FLAG = 0x80000000u;     // "explored"/"sampled" bit on a doc id
 constexpr uint32_t BM25_BIT = 0x80000000u; // unified term key: bit31 set = BM25 term
+constexpr uint32_t KW_HIT = 0x40000000u;   // keyword-filter search: pool id of a document that holds a required keyword
+constexpr uint32_t ID_MASK = 0x3FFFFFFFu;  // doc id without the two flag bits
 constexpr float INF_DIS = 1000000.0f;
 constexpr int DIM = 1024;
 constexpr int DENSE_BYTES = DIM * 4;
@@ -208,6 +210,17 @@ __device__ __forceinline__ bool id_set_contains(const uint32_t* set, uint32_t ma
     }
 }
 
+// Insert into a plain id set; false if the key was already there.
+__device__ __forceinline__ bool id_set_insert(uint32_t* set, uint32_t mask, uint32_t id) {
+    uint32_t h = term_hash(id, mask);
+    while (true) {
+        uint32_t old = atomicCAS(&set[h], EMPTY, id);
+        if (old == EMPTY) return true;
+        if (old == id) return false;
+        h = (h + 1) & mask;
+    }
+}
+
 // One pair of the candidate against the pivot's table. With KW, a BM25 term of the
 // candidate that the pivot lacks but the centre node's term set holds raises `kw`
 // (the test of the build-time cal_bm25_dist, index.cu:128-153).
@@ -281,6 +294,7 @@ struct BoundedOut {
     uint32_t nnz_s;  // SPLADE pairs read
     uint32_t nnz_b;  // BM25 pairs read
     bool dense_read; // the 4 KB dense row was read
+    bool kw_hit;     // keyword-filter search only: a BM25 term of the document is one of the query's required keywords
 };
 
 // Two-stage hybrid distance between the pivot and document `id` (wave-uniform).
@@ -301,6 +315,7 @@ __device__ __forceinline__ BoundedOut eval_wave_bounded(const CorpusView& C, uin
     o.nnz_s = (paths & PATH_SPARSE) ? ns : 0u;
     o.nnz_b = (paths & PATH_BM25) ? nb : 0u;
     o.dense_read = false;
+    o.kw_hit = false;
     float ssum = 0.f;
     const bool has_sparse = (paths & (PATH_SPARSE | PATH_BM25)) != 0;
     if (has_sparse) {
@@ -391,25 +406,39 @@ __device__ __forceinline__ float readlane_f32(float v, uint32_t src) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
 }
 
+// A pair of the candidate against the query's table. With KWD, a BM25 pair that hits the table and
+// whose term is in `kwset` (the query's required keywords, keys carry BM25_BIT) raises `hit`
+// (the test of the search-time cal_bm25_dist, utils.cuh:318-340).
+template <bool KWD>
+__device__ __forceinline__ void probe_query_pair(const uint2* tab, uint32_t mask, uint2 kv, float& acc, const uint32_t* kwset, uint32_t kwmask,
+                                                 bool& hit) {
+    const bool found = term_table_probe(tab, mask, kv.x, __uint_as_float(kv.y), acc);
+    if (KWD) {
+        if (found && (kv.x & BM25_BIT) && id_set_contains(kwset, kwmask, kv.x)) hit = true;
+    }
+}
+
+template <bool KWD = false>
 __device__ __forceinline__ BoundedOut eval_finish(const PendingEval& p, const PivotDense& pv, const uint2* tab, uint32_t mask, uint32_t paths,
-                                                  float dense_mul, float bonus, float thr) {
+                                                  float dense_mul, float bonus, float thr, const uint32_t* kwset = nullptr,
+                                                  uint32_t kwmask = 0) {
     const int lane = lane_id();
     BoundedOut o;
     o.nnz_s = (paths & PATH_SPARSE) ? p.ns : 0u;
     o.nnz_b = (paths & PATH_BM25) ? p.nb : 0u;
     o.dense_read = false;
+    o.kw_hit = false;
     float ssum = 0.f;
     if (paths & (PATH_SPARSE | PATH_BM25)) {
         const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
         const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
         float acc = 0.f;
-        if (j0 < p.end) term_table_probe(tab, mask, p.kv0.x, __uint_as_float(p.kv0.y), acc);
-        if (j1 < p.end) term_table_probe(tab, mask, p.kv1.x, __uint_as_float(p.kv1.y), acc);
-        if (j2 < p.end) term_table_probe(tab, mask, p.kv2.x, __uint_as_float(p.kv2.y), acc);
-        for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) {
-            const uint2 kv = sp[j];
-            term_table_probe(tab, mask, kv.x, __uint_as_float(kv.y), acc);
-        }
+        bool hit = false;
+        if (j0 < p.end) probe_query_pair<KWD>(tab, mask, p.kv0, acc, kwset, kwmask, hit);
+        if (j1 < p.end) probe_query_pair<KWD>(tab, mask, p.kv1, acc, kwset, kwmask, hit);
+        if (j2 < p.end) probe_query_pair<KWD>(tab, mask, p.kv2, acc, kwset, kwmask, hit);
+        for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) probe_query_pair<KWD>(tab, mask, sp[j], acc, kwset, kwmask, hit);
+        if (KWD) o.kw_hit = __ballot(hit) != 0;
         ssum = wave_sum_dpp(acc);
         if (!(paths & PATH_DENSE)) {
             o.dist = 1.0f - ssum - bonus;

@@ -223,6 +223,15 @@ int apoe_queries_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* de
         q->max_nnz = std::max(q->max_nnz, (q->h_s_off[i + 1] - q->h_s_off[i]) + (q->h_b_off[i + 1] - q->h_b_off[i]));
     q->total_nnz_s = nnz_s;
     q->total_nnz_b = nnz_b;
+    if (nnz_b) {
+        std::vector<uint32_t> h_idx(nnz_b);
+        APOE_HIP(hipMemcpy(h_idx.data(), b_idx, (size_t)nnz_b * sizeof(uint32_t), hipMemcpyDefault));
+        for (uint32_t i = 0; i < n; i++) {
+            uint32_t k = 0;
+            for (uint32_t j = q->h_b_off[i]; j < q->h_b_off[i + 1]; j++) k += h_idx[j] >> 31;
+            q->max_keywords = std::max(q->max_keywords, k);
+        }
+    }
     APOE_TRY(q->dense.alloc((size_t)n * dim));
     APOE_TRY(q->s_off.alloc(n + 1));
     APOE_TRY(q->b_off.alloc(n + 1));

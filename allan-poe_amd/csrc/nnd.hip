@@ -17,17 +17,6 @@ __device__ __forceinline__ float key_dist(uint64_t key) {
     return __uint_as_float(u);
 }
 
-// ---- id set in LDS (dedupe of gathered candidates) ----
-__device__ __forceinline__ bool id_set_insert(uint32_t* set, uint32_t mask, uint32_t id) {
-    uint32_t h = term_hash(id, mask);
-    while (true) {
-        uint32_t old = atomicCAS(&set[h], EMPTY, id);
-        if (old == EMPTY) return true;
-        if (old == id) return false;
-        h = (h + 1) & mask;
-    }
-}
-
 __global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t n, uint32_t K, uint64_t seed, uint32_t* ids, float* dist,
                                                        unsigned long long* rev, uint32_t* rev_cnt) {
     const uint64_t total = (uint64_t)n * K;

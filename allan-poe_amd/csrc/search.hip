@@ -7,6 +7,10 @@ namespace apoe {
 
 constexpr int MAX_NEW = 64;   // fresh candidates per step: one lane each in wave 0
 constexpr int EVAL_BATCH = 2; // candidates whose sparse parts a wave keeps in flight together
+constexpr int RING = 32;      // keyword-filter search: evicted keyword hits kept beside the pool (query.cu:18)
+
+// What the kernel does on top of the plain beam search.
+enum SearchMode { MODE_PLAIN = 0, MODE_KG = 1, MODE_KEYWORD = 2 };
 
 struct SearchArgs {
     CorpusView C;
@@ -29,12 +33,15 @@ struct SearchArgs {
     const uint32_t *e2e_off, *e2e_idx, *e2d_off, *e2d_idx, *q2e_off, *q2e_idx;
     uint32_t n_entities;
     float kg_weight;
+    uint32_t kw_slots; // keyword-filter kernels only: slots of the per-query keyword term set
 };
 
 // LDS carve-up shared by host (size) and device (pointers).
 struct SearchLds {
-    uint32_t tab, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ctl, total;
-    __host__ __device__ SearchLds(uint32_t slots, uint32_t cands, bool kg) {
+    uint32_t tab, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ring_id,
+        ring_dist, kwset, ctl, total;
+    __host__ __device__ SearchLds(uint32_t slots, uint32_t cands, int mode, uint32_t kw_slots) {
+        const bool kg = mode == MODE_KG, kwd = mode == MODE_KEYWORD;
         uint32_t o = 0;
         tab = o; o += slots * 8;
         pool_id = o; o += cands * 4;
@@ -44,12 +51,15 @@ struct SearchLds {
         new_lb = o; o += MAX_NEW * 4;
         new_id = o; o += MAX_NEW * 4;
         new_dist = o; o += MAX_NEW * 4;
-        new_ent = o; o += kg ? MAX_NEW * 4 : 0;
+        new_ent = o; o += (kg || kwd) ? MAX_NEW * 4 : 0; // keyword search: the hit flag of a fresh candidate
         new_hop = o; o += kg ? MAX_NEW * 4 : 0;
         seed_id = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
         seed_ent = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
         seed_dist = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
         link = o; o += kg ? MAX_NEW * 4 : 0;
+        ring_id = o; o += kwd ? RING * 4 : 0;
+        ring_dist = o; o += kwd ? RING * 4 : 0;
+        kwset = o; o += kwd ? kw_slots * 4 : 0;
         ctl = o; o += 16 * 4;
         total = o;
     }
@@ -66,6 +76,16 @@ struct Pool {
     uint32_t cands;
 };
 
+// Keyword-filter search: pool entries that carry KW_HIT and fall off the pool. Entries are
+// appended merge by merge, within one merge from the worst to the best, and slot (count % RING)
+// is overwritten, so the ring holds the RING most recent ones: distances never grow along that
+// sequence, which makes them the closest evicted hits (query.cu:244-248 appends in atomic order).
+struct Ring {
+    uint32_t* id;
+    float* dist;
+    uint32_t n; // appended so far (wave-uniform, wave 0)
+};
+
 __device__ __forceinline__ void wave_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -79,8 +99,11 @@ __device__ __forceinline__ void wave_fence() {
 // moves at all -- only the 64-element rounds from the top down to lb_0 are touched (each round
 // is read into registers before anything at or above it is written). Returns the lowest rank a
 // new element took (cands if none entered).
-template <bool KG>
-__device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, float* ndist, uint32_t* nent, uint32_t* nhop, uint32_t n) {
+// Keyword-filter search: nent[i] != 0 says that new candidate i holds a required keyword; it
+// enters the pool with KW_HIT set on its id (ordering uses the plain id).
+template <int MODE>
+__device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, float* ndist, uint32_t* nent, uint32_t* nhop, uint32_t n, Ring& R) {
+    constexpr bool KG = MODE == MODE_KG, KWD = MODE == MODE_KEYWORD;
     const int lane = lane_id();
     const uint32_t cands = P.cands;
     if (n == 0) return cands;
@@ -91,6 +114,7 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
         d = ndist[lane];
         id = nid[lane];
         if (KG) { ent = nent[lane]; hop = nhop[lane]; }
+        if (KWD) ent = nent[lane];
         for (uint32_t i = 0; i < n; i++) {
             const float di = ndist[i];
             const uint32_t ii = nid[i];
@@ -102,6 +126,7 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
         ndist[rank] = d;
         nid[rank] = id;
         if (KG) { nent[rank] = ent; nhop[rank] = hop; }
+        if (KWD) nent[rank] = ent;
     }
     wave_fence();
     // lane i now takes the i-th smallest
@@ -110,6 +135,7 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
         d = ndist[lane];
         id = nid[lane];
         if (KG) { ent = nent[lane]; hop = nhop[lane]; }
+        if (KWD) id |= nent[lane] ? KW_HIT : 0u;
         if (d <= P.dist[cands - 1]) {
             uint32_t lo = 0, len = cands;
             while (len > 0) {
@@ -124,6 +150,22 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
     const uint32_t n_in = __popcll(__ballot(enters)); // ranks grow with the lane: the first n_in enter
     if (n_in == 0) return cands;
     wave_fence();
+    if (KWD) {
+        // exactly the last n_in pool entries fall off; lane l looks at the l-th from the end
+        uint32_t eid = EMPTY;
+        float ed = 0.f;
+        if ((uint32_t)lane < n_in) { eid = P.id[cands - 1 - lane]; ed = P.dist[cands - 1 - lane]; }
+        const bool hit = eid != EMPTY && (eid & KW_HIT);
+        const uint64_t hb = __ballot(hit);
+        const uint32_t cnt = __popcll(hb), rank = __popcll(hb & ((1ull << lane) - 1));
+        if (hit && rank + RING >= cnt) {
+            const uint32_t slot = (R.n + rank) % RING;
+            R.id[slot] = eid & ID_MASK;
+            R.dist[slot] = ed;
+        }
+        R.n += cnt;
+        wave_fence();
+    }
     const uint32_t lo0 = P.lb[0];
     for (int base = (int)((cands - 1) & ~(uint32_t)(WAVE - 1)); base >= 0 && (uint32_t)base + WAVE > lo0; base -= WAVE) {
         const uint32_t p = base + lane;
@@ -153,10 +195,11 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
     return lo0;
 }
 
-template <int NW, bool KG>
+template <int NW, int MODE>
 __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))) void search_kernel(SearchArgs a) {
+    constexpr bool KG = MODE == MODE_KG, KWD = MODE == MODE_KEYWORD;
     extern __shared__ __align__(16) char smem[];
-    const SearchLds L(a.slots, a.cands, KG);
+    const SearchLds L(a.slots, a.cands, MODE, a.kw_slots);
     uint2* tab = reinterpret_cast<uint2*>(smem + L.tab);
     Pool P;
     P.id = reinterpret_cast<uint32_t*>(smem + L.pool_id);
@@ -173,6 +216,11 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
     uint32_t* seed_ent = reinterpret_cast<uint32_t*>(smem + L.seed_ent);
     float* seed_dist = reinterpret_cast<float*>(smem + L.seed_dist);
     uint32_t* link = reinterpret_cast<uint32_t*>(smem + L.link);
+    uint32_t* kwset = reinterpret_cast<uint32_t*>(smem + L.kwset);
+    Ring R;
+    R.id = reinterpret_cast<uint32_t*>(smem + L.ring_id);
+    R.dist = reinterpret_cast<float*>(smem + L.ring_dist);
+    R.n = 0;
     volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
 
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
@@ -194,6 +242,10 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             for (uint32_t i = tid; i < a.bitmap_words / 4; i += NW * WAVE) b4[i] = make_uint4(0, 0, 0, 0);
         }
         term_table_clear(tab, a.slots, tid, NW * WAVE);
+        if (KWD) {
+            for (uint32_t i = tid; i < a.kw_slots; i += NW * WAVE) kwset[i] = EMPTY;
+            R.n = 0;
+        }
         for (uint32_t i = tid; i < cands; i += NW * WAVE) {
             P.id[i] = EMPTY;
             P.dist[i] = INF_DIS;
@@ -204,6 +256,13 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
         __threadfence();
         __syncthreads();
         pivot_terms_from_query(tab, mask, a.Q, q, a.w_s, a.w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
+        if (KWD) {
+            // required keywords: BM25 query terms whose id arrives with bit 31 set (query.cu:1828-1843)
+            for (uint32_t j = a.Q.b_off[q] + tid; j < a.Q.b_off[q + 1]; j += NW * WAVE) {
+                const uint32_t t = a.Q.b_idx[j];
+                if (t & BM25_BIT) id_set_insert(kwset, a.kw_slots - 1, t);
+            }
+        }
 
         const float pv_norm = pivot_dense_norm(pv);
         uint64_t st_exp = 0, st_eval = 0, st_ns = 0, st_nb = 0, st_dense = 0; // wave-uniform counters
@@ -285,7 +344,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                         new_hop[lane] = 0;
                     }
                     wave_fence();
-                    sort_merge<KG>(P, new_id, new_dist, new_ent, new_hop, nb);
+                    sort_merge<MODE>(P, new_id, new_dist, new_ent, new_hop, nb, R);
                 }
                 if (lane == 0) { ctl[CTL_NNEW] = 0; ctl[CTL_PARENT] = 0; }
             }
@@ -323,19 +382,22 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                         if (KG) {
                             if (new_ent[jj] != EMPTY) bonus = a.kg_weight / (float)new_hop[jj]; // query.cu:1759-1760
                         }
-                        BoundedOut e = eval_finish(pe[b], pv, tab, mask, a.paths, 1.0f, bonus, thr_eff);
+                        BoundedOut e = eval_finish<KWD>(pe[b], pv, tab, mask, a.paths, 1.0f, bonus, thr_eff, kwset, a.kw_slots - 1);
                         st_eval++;
                         st_ns += e.nnz_s;
                         st_nb += e.nnz_b;
                         st_dense += e.dense_read;
-                        if (lane == 0) new_dist[jj] = e.dist;
+                        if (lane == 0) {
+                            new_dist[jj] = e.dist;
+                            if (KWD) new_ent[jj] = e.kw_hit ? 1u : 0u;
+                        }
                     }
                 }
             }
             __syncthreads();
             // ---- wave 0: merge, pick the next parent, fetch its neighbours ----
             if (wave == 0) {
-                hint = min(hint, sort_merge<KG>(P, new_id, new_dist, new_ent, new_hop, n_new));
+                hint = min(hint, sort_merge<MODE>(P, new_id, new_dist, new_ent, new_hop, n_new, R));
                 uint32_t parent = EMPTY, slot = 0, n_next = 0;
                 if (it < a.max_iter) {
                     for (uint32_t base = hint & ~(uint32_t)(WAVE - 1); base < cands; base += WAVE) {
@@ -354,6 +416,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                     uint32_t p_ent = EMPTY, p_hop = 0;
                     if (KG) { p_ent = P.ent[slot]; p_hop = P.hop[slot]; }
                     if (lane == 0) P.id[slot] = parent | FLAG;
+                    if (KWD) parent &= ID_MASK;
                     st_exp++;
                     uint32_t c = lane < (int)a.degree ? a.graph[(size_t)parent * a.W + lane] : EMPTY;
                     bool fresh = false;
@@ -363,6 +426,21 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                     }
                     bool alive = fresh;
                     uint32_t ent = EMPTY;
+                    if (KWD) {
+                        // slots whose graph neighbour was already visited (or invalid) are recycled with
+                        // the parent's keyword edges: the t-th such slot takes keyword edge t
+                        // (query.cu:1397-1409; which slot gets which edge does not matter)
+                        const bool dup = lane < (int)a.degree && !fresh;
+                        const uint32_t t = __popcll(__ballot(dup) & lane_lt);
+                        const uint32_t n_kw = min(uniform(a.graph[(size_t)parent * a.W + a.degree]), (uint32_t)APOE_KW_SLOTS - 1u);
+                        if (dup && t < n_kw) {
+                            const uint32_t c2 = a.graph[(size_t)parent * a.W + a.degree + 1 + t];
+                            if (c2 < a.C.n) {
+                                const uint32_t bit = 1u << (c2 & 31);
+                                if (!(atomicOr(&bitmap[c2 >> 5], bit) & bit)) { c = c2; alive = true; }
+                            }
+                        }
+                    }
                     if (KG) {
                         // logical edges: parent's entity -> neighbour entity -> document
                         if (p_hop < 3 && p_ent < a.n_entities) {
@@ -449,9 +527,41 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             __syncthreads();
         }
         // ---- results (query.cu:566-569) ----
-        for (uint32_t i = tid; i < cands; i += NW * WAVE) {
-            a.out_ids[(size_t)qi * cands + i] = P.id[i] & ~FLAG;
-            a.out_dist[(size_t)qi * cands + i] = P.dist[i];
+        if (!KWD) {
+            for (uint32_t i = tid; i < cands; i += NW * WAVE) {
+                a.out_ids[(size_t)qi * cands + i] = P.id[i] & ~FLAG;
+                a.out_dist[(size_t)qi * cands + i] = P.dist[i];
+            }
+        } else if (wave == 0) {
+            // pool entries that hold a required keyword, in pool order, then the evicted hits by
+            // (distance, id); the rest of the row is empty (query.cu:1464-1481)
+            uint32_t* oid = a.out_ids + (size_t)qi * cands;
+            float* od = a.out_dist + (size_t)qi * cands;
+            uint32_t kn = 0;
+            for (uint32_t base = 0; base < cands; base += WAVE) {
+                const uint32_t id = base + lane < cands ? P.id[base + lane] : EMPTY;
+                const bool hit = id != EMPTY && (id & KW_HIT);
+                const uint64_t hb = __ballot(hit);
+                if (hit) {
+                    const uint32_t pos = kn + __popcll(hb & lane_lt);
+                    oid[pos] = id & ID_MASK;
+                    od[pos] = P.dist[base + lane];
+                }
+                kn += __popcll(hb);
+            }
+            const uint32_t m = min(R.n, (uint32_t)RING);
+            if ((uint32_t)lane < m) {
+                const float d = R.dist[lane];
+                const uint32_t id = R.id[lane];
+                uint32_t rank = 0;
+                for (uint32_t i = 0; i < m; i++) {
+                    const float di = R.dist[i];
+                    const uint32_t ii = R.id[i];
+                    rank += (di < d) || (di == d && ii < id);
+                }
+                if (kn + rank < cands) { oid[kn + rank] = id; od[kn + rank] = d; }
+            }
+            for (uint32_t i = kn + m + lane; i < cands; i += WAVE) { oid[i] = EMPTY & ~FLAG; od[i] = INF_DIS; }
         }
         if (lane == 0) {
             if (st_exp) atomicAdd(a.work + 1, st_exp);
@@ -463,12 +573,35 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
     }
 }
 
-template <int NW, bool KG>
-static int launch_variant(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, size_t lds) {
-    APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&search_kernel<NW, KG>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    search_kernel<NW, KG><<<grid, NW * WAVE, lds, ctx->stream>>>(a);
+template <int NW, int MODE>
+static int launch_variant(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, size_t lds, int* per_cu) {
+    const void* fn = reinterpret_cast<const void*>(&search_kernel<NW, MODE>);
+    APOE_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (per_cu) { // occupancy query only
+        APOE_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, fn, NW * WAVE, lds));
+        return APOE_OK;
+    }
+    search_kernel<NW, MODE><<<grid, NW * WAVE, lds, ctx->stream>>>(a);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
+}
+
+template <int MODE>
+static int launch_shape(apoe_ctx* ctx, int nw, const SearchArgs& a, uint32_t grid, size_t lds, int* per_cu) {
+    switch (nw) {
+        case 1: return launch_variant<1, MODE>(ctx, a, grid, lds, per_cu);
+        case 4: return launch_variant<4, MODE>(ctx, a, grid, lds, per_cu);
+        case 8: return launch_variant<8, MODE>(ctx, a, grid, lds, per_cu);
+        default: return launch_variant<2, MODE>(ctx, a, grid, lds, per_cu);
+    }
+}
+
+static int launch_mode(apoe_ctx* ctx, int mode, int nw, const SearchArgs& a, uint32_t grid, size_t lds, int* per_cu) {
+    switch (mode) {
+        case MODE_KG: return launch_shape<MODE_KG>(ctx, nw, a, grid, lds, per_cu);
+        case MODE_KEYWORD: return launch_shape<MODE_KEYWORD>(ctx, nw, a, grid, lds, per_cu);
+        default: return launch_shape<MODE_PLAIN>(ctx, nw, a, grid, lds, per_cu);
+    }
 }
 
 int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g, const apoe_kg* kg,
@@ -505,6 +638,14 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     a.full_eval = (p->variant & 0x100u) ? 1u : 0u;
 
     const bool use_kg = kg != nullptr;
+    const bool use_kw = p->keyword_filter != 0;
+    APOE_REQUIRE(!(use_kg && use_kw), "keyword-filter search cannot be combined with a knowledge graph");
+    const int mode = use_kg ? MODE_KG : use_kw ? MODE_KEYWORD : MODE_PLAIN;
+    if (use_kw) {
+        APOE_REQUIRE(c->n < (1u << 30), "keyword-filter search keeps two flag bits on a document id: %u documents are too many", c->n);
+        a.paths = PATH_DENSE | PATH_SPARSE | PATH_BM25; // query.cu:2005-2007: always the three-path loop
+        a.kw_slots = next_pow2(std::max(64u, 2 * q->max_keywords));
+    }
     if (use_kg) {
         APOE_REQUIRE(kg->n_queries >= p->q_begin + q_count, "knowledge graph holds entities for %u queries, %u needed", kg->n_queries, p->q_begin + q_count);
         a.e2e_off = kg->e2e_off.p;
@@ -515,7 +656,7 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
         a.q2e_idx = kg->q2e_idx.p;
         a.n_entities = kg->n_entities;
     }
-    const SearchLds L(a.slots, a.cands, use_kg);
+    const SearchLds L(a.slots, a.cands, mode, a.kw_slots);
     APOE_REQUIRE(L.total <= 64 * 1024, "search needs %u bytes of LDS (query rows with up to %u sparse terms)", L.total, q->max_nnz);
 
     // variant 0: two waves per query (the measured best); 1, 2, 3: one, four, eight waves
@@ -526,14 +667,8 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     else if (shape == 3) nw = 8;
     // persistent grid: as many workgroups as can be resident, never more than queries
     int per_cu = 1;
-    {
-        const void* fn = nullptr;
-        if (use_kg) fn = nw == 1 ? (const void*)&search_kernel<1, true> : nw == 2 ? (const void*)&search_kernel<2, true> : nw == 8 ? (const void*)&search_kernel<8, true> : (const void*)&search_kernel<4, true>;
-        else fn = nw == 1 ? (const void*)&search_kernel<1, false> : nw == 2 ? (const void*)&search_kernel<2, false> : nw == 8 ? (const void*)&search_kernel<8, false> : (const void*)&search_kernel<4, false>;
-        APOE_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
-        APOE_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, nw * WAVE, L.total));
-        if (per_cu < 1) per_cu = 1;
-    }
+    APOE_TRY(launch_mode(ctx, mode, nw, a, 0, L.total, &per_cu));
+    if (per_cu < 1) per_cu = 1;
     const uint32_t grid = std::min<uint32_t>(q_count, (uint32_t)per_cu * (uint32_t)ctx->num_cus);
 
     a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;
@@ -546,22 +681,7 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     a.work = work.p;
 
     float ms = 0.f;
-    APOE_TRY(timed(ctx, &ms, [&]() {
-        if (use_kg) {
-            switch (nw) {
-                case 1: return launch_variant<1, true>(ctx, a, grid, L.total);
-                case 8: return launch_variant<8, true>(ctx, a, grid, L.total);
-                case 4: return launch_variant<4, true>(ctx, a, grid, L.total);
-                default: return launch_variant<2, true>(ctx, a, grid, L.total);
-            }
-        }
-        switch (nw) {
-            case 1: return launch_variant<1, false>(ctx, a, grid, L.total);
-            case 8: return launch_variant<8, false>(ctx, a, grid, L.total);
-            case 4: return launch_variant<4, false>(ctx, a, grid, L.total);
-            default: return launch_variant<2, false>(ctx, a, grid, L.total);
-        }
-    }));
+    APOE_TRY(timed(ctx, &ms, [&]() { return launch_mode(ctx, mode, nw, a, grid, L.total, nullptr); }));
     APOE_HIP(hipStreamSynchronize(ctx->stream));
     if (stats) {
         unsigned long long h[8];

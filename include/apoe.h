@@ -160,6 +160,8 @@ typedef struct {
                                         default a candidate whose sparse part plus the Cauchy-Schwarz
                                         bound of its dense part cannot beat the worst entry of the full
                                         pool is dropped without reading its dense row (same results) */
+    uint32_t keyword_filter;         /* 1: keyword-filter search (search_with_keyword, query.cu:1271-1483);
+                                        kg must be NULL */
 } apoe_search_params;
 
 typedef struct {
@@ -174,7 +176,16 @@ typedef struct {
 } apoe_search_stats;
 
 /* out_ids/out_dist are [q_count][cands], ascending distance; top_k is the row
- * prefix (query.cu:2070-2075). Empty slots hold id 0x7FFFFFFF, distance INF_DIS. */
+ * prefix (query.cu:2070-2075). Empty slots hold id 0x7FFFFFFF, distance INF_DIS.
+ *
+ * Keyword-filter search (keyword_filter = 1): a BM25 term id of a QUERY row with bit 31 set is a
+ * required keyword (the host sets the bit, query.cu:1828-1843; every search compares term ids
+ * under the mask 0x7FFFFFFF, so a flagged term scores like an unflagged one). A document "hits"
+ * when one of its BM25 terms is a required keyword of the query. All three paths are computed
+ * whatever the weights (the reference runs its three-path loop), slots of a graph row whose
+ * neighbour was already visited are refilled from the row's keyword edges, and a result row holds
+ * only hits: the hits of the final pool in pool order, then up to 32 hits that were pushed out of
+ * the pool (the closest ones, ascending), then empty slots. Needs n < 2^30 documents. */
 int apoe_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g,
                 const apoe_kg* kg, const apoe_search_params* p, uint32_t* out_ids, float* out_dist,
                 apoe_search_stats* stats);

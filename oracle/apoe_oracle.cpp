@@ -309,6 +309,147 @@ void orc_search(const orc_set* corpus, const orc_set* queries, const uint32_t* g
 }
 
 /*
+ * query.cu:1271-1483 (search_with_keyword), merge_top_keyword query.cu:227-275, cal_bm25_dist
+ * utils.cuh:318-340, host flagging query.cu:1828-1843. On top of orc_search's semantics:
+ *  - a BM25 term id of a query row with bit 31 set is a required keyword; term ids are compared
+ *    under the mask 0x7FFFFFFF; a document "hits" when one of its BM25 terms is a required keyword
+ *    of the query (utils.cuh:330-336), and carries that as a flag beside its pool entry (bit 30 of
+ *    the id in the reference, query.cu:1349,1450);
+ *  - all three paths are computed whatever the weights (query.cu:2005-2007 always launches the
+ *    three-path loop; the weights are already folded into the query values);
+ *  - expansion (query.cu:1386-1410): the slots of the parent's row whose neighbour was already
+ *    visited (or is not a document) are refilled from the row's keyword edges, the t-th such
+ *    slot with keyword edge t, if that one is unvisited; the set of candidates this yields does
+ *    not depend on the reference's atomic slot order;
+ *  - merge (query.cu:243-248): a POOL entry that falls off the pool and is a hit goes to a ring
+ *    of 32 (new candidates that never enter are not kept, as in the reference). The reference
+ *    tests `id & 0x40000000 != 0`, which C parses as `id & 1`; here the flag is tested. The ring is
+ *    filled merge by merge, within a merge from the worst to the best, slot = count % 32, so it
+ *    ends up holding the 32 closest evicted hits (the reference's order inside a merge is the
+ *    arrival order of atomics);
+ *  - result row (query.cu:1464-1481): hits of the final pool in pool order, then the ring by
+ *    (distance, id), then empty slots (the reference sorts and reads all 32 ring slots, written
+ *    or not, and reads past the ring when cands > 32 + hits).
+ */
+void orc_search_keyword(const orc_set* corpus, const orc_set* queries, const uint32_t* graph,
+                        uint32_t W, const uint32_t* entry, uint32_t n_entry, const float* w3,
+                        uint32_t cands, uint32_t max_iter, uint32_t* out_ids, float* out_dist,
+                        uint64_t* counters, int threads) {
+    const uint32_t d = W - ORC_KW_SLOTS;
+    const uint32_t RING = 32; /* query.cu:18 */
+    /* queries with the keyword bit stripped, for the metric */
+    const uint32_t nnz_qb = queries->b_off[queries->n];
+    std::vector<uint32_t> plain_idx(nnz_qb);
+    for (uint32_t j = 0; j < nnz_qb; j++) plain_idx[j] = queries->b_idx[j] & 0x7FFFFFFFu;
+    orc_set Qp = *queries;
+    Qp.b_idx = plain_idx.data();
+    QW w(w3);
+    for (int i = 0; i < 3; i++) w.on[i] = true;
+#pragma omp parallel num_threads(nthreads(threads))
+    {
+        Bitset visited(corpus->n);
+        std::vector<Cand> pool, fresh, merged, ring(RING);
+#pragma omp for schedule(dynamic, 4)
+        for (int64_t q = 0; q < (int64_t)queries->n; q++) {
+            visited.clear();
+            pool.assign(cands, Cand{ORC_INF_DIS, ORC_EMPTY, 0, 0});
+            uint64_t n_exp = 0, n_eval = 0, nnz_s = 0, nnz_b = 0, ring_n = 0;
+            auto is_hit = [&](uint32_t c) -> uint32_t {
+                uint32_t a = corpus->b_off[c], a1 = corpus->b_off[c + 1];
+                uint32_t b = queries->b_off[q], b1 = queries->b_off[q + 1];
+                while (a < a1 && b < b1) {
+                    const uint32_t tq = queries->b_idx[b] & 0x7FFFFFFFu;
+                    if (corpus->b_idx[a] < tq) a++;
+                    else if (corpus->b_idx[a] > tq) b++;
+                    else {
+                        if (queries->b_idx[b] & 0x80000000u) return 1;
+                        a++; b++;
+                    }
+                }
+                return 0;
+            };
+            auto eval = [&](uint32_t c) {
+                n_eval++;
+                nnz_s += corpus->s_off[c + 1] - corpus->s_off[c];
+                nnz_b += corpus->b_off[c + 1] - corpus->b_off[c];
+                fresh.push_back({qdist(corpus, c, &Qp, (uint32_t)q, w), c, is_hit(c), 0}); /* ent = hit flag */
+            };
+            /* merge with the ring fed by the pool entries that fall off */
+            auto merge_kw = [&]() {
+                std::sort(fresh.begin(), fresh.end(), cand_less);
+                /* the rank merge of merge_cands, counting how many new ones enter: exactly that
+                 * many entries fall off the end of the old pool */
+                merged.clear();
+                size_t p = 0, f = 0;
+                while (merged.size() < cands && (p < cands || f < fresh.size())) {
+                    if (f < fresh.size() && (p >= cands || fresh[f].dist <= pool[p].dist)) merged.push_back(fresh[f++]);
+                    else merged.push_back(pool[p++]);
+                }
+                for (size_t l = 0; l < f; l++) { /* worst first */
+                    const Cand& e = pool[cands - 1 - l];
+                    if (e.id != ORC_EMPTY && e.ent) ring[ring_n++ % RING] = e;
+                }
+                pool.swap(merged);
+            };
+            fresh.clear();
+            for (uint32_t i = 0; i < n_entry; i++) {
+                uint32_t e = entry[i];
+                if (e >= corpus->n || visited.test_and_set(e)) continue;
+                eval(e);
+            }
+            merge_kw();
+            for (uint32_t it = 0; it < max_iter; it++) {
+                uint32_t j = 0;
+                while (j < cands && (pool[j].id & ORC_FLAG)) j++;
+                if (j == cands) break;
+                uint32_t parent = pool[j].id;
+                pool[j].id |= ORC_FLAG;
+                n_exp++;
+                fresh.clear();
+                const uint32_t* row = graph + (size_t)parent * W;
+                uint32_t n_dup = 0;
+                for (uint32_t t = 0; t < d; t++) {
+                    uint32_t c = row[t];
+                    if (c >= corpus->n || visited.test_and_set(c)) { n_dup++; continue; }
+                    eval(c);
+                }
+                const uint32_t n_kw = std::min<uint32_t>(row[d], ORC_KW_SLOTS - 1);
+                for (uint32_t t = 0; t < std::min(n_dup, n_kw); t++) {
+                    uint32_t c = row[d + 1 + t];
+                    if (c >= corpus->n || visited.test_and_set(c)) continue;
+                    eval(c);
+                }
+                merge_kw();
+            }
+            uint32_t o = 0;
+            for (uint32_t i = 0; i < cands; i++)
+                if (pool[i].id != ORC_EMPTY && pool[i].ent) {
+                    out_ids[q * cands + o] = pool[i].id & ~ORC_FLAG;
+                    out_dist[q * cands + o] = pool[i].dist;
+                    o++;
+                }
+            std::vector<Cand> tail(ring.begin(), ring.begin() + std::min<uint64_t>(ring_n, RING));
+            for (Cand& c : tail) c.id &= ~ORC_FLAG;
+            std::sort(tail.begin(), tail.end(), cand_less);
+            for (size_t i = 0; i < tail.size() && o < cands; i++, o++) {
+                out_ids[q * cands + o] = tail[i].id;
+                out_dist[q * cands + o] = tail[i].dist;
+            }
+            for (; o < cands; o++) {
+                out_ids[q * cands + o] = ORC_EMPTY & ~ORC_FLAG;
+                out_dist[q * cands + o] = ORC_INF_DIS;
+            }
+            if (counters) {
+                counters[q * 4 + 0] = n_exp;
+                counters[q * 4 + 1] = n_eval;
+                counters[q * 4 + 2] = nnz_s;
+                counters[q * 4 + 3] = nnz_b;
+            }
+        }
+    }
+}
+
+/*
  * query.cu:1541-1779. On top of orc_search's semantics:
  *  - "current" means the pool slot of the parent picked in this iteration (the
  *    reference reads kg_cur_id, which is never written, query.cu:1559,1694);

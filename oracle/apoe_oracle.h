@@ -83,6 +83,13 @@ void orc_search(const orc_set* corpus, const orc_set* queries, const uint32_t* g
                 uint32_t max_iter, uint32_t* out_ids, float* out_dist, uint64_t* counters,
                 int threads);
 
+/* Keyword-filter beam search (query.cu:1271-1483): query BM25 term ids with bit 31 set are the
+ * required keywords; rows hold only documents with such a term (pool hits, then evicted hits). */
+void orc_search_keyword(const orc_set* corpus, const orc_set* queries, const uint32_t* graph,
+                        uint32_t W, const uint32_t* entry, uint32_t n_entry, const float* w3,
+                        uint32_t cands, uint32_t max_iter, uint32_t* out_ids, float* out_dist,
+                        uint64_t* counters, int threads);
+
 /* Beam search with KG seeding and logical-edge expansion (query.cu:1541-1779). */
 void orc_search_kg(const orc_set* corpus, const orc_set* queries, const orc_kg* kg,
                    const uint32_t* graph, uint32_t W, const uint32_t* entry, uint32_t n_entry,

@@ -175,7 +175,7 @@ def merge_top(pool_ids, pool_dist, new_ids, new_dist):
     return pi, pd
 
 
-def search(corpus, queries, rows, entry, w3, cands, max_iter=1000, kg=None, kg_weight=0.0, threads=0):
+def search(corpus, queries, rows, entry, w3, cands, max_iter=1000, kg=None, kg_weight=0.0, threads=0, keyword_filter=False):
     rows, pr = _u32(rows)
     entry, pe = _u32(entry)
     n, W = rows.shape
@@ -184,7 +184,12 @@ def search(corpus, queries, rows, entry, w3, cands, max_iter=1000, kg=None, kg_w
     dist = np.empty((queries.n, cands), np.float32)
     counters = np.zeros((queries.n, 4), np.uint64)
     w, pw = _w3(w3)
-    if kg is None:
+    if keyword_filter:
+        assert kg is None
+        lib().orc_search_keyword(corpus.ref(), queries.ref(), pr, C.c_uint32(W), pe, C.c_uint32(len(entry)), pw, C.c_uint32(cands),
+                                 C.c_uint32(max_iter), ids.ctypes.data_as(u32p), dist.ctypes.data_as(f32p),
+                                 counters.ctypes.data_as(u64p), threads)
+    elif kg is None:
         lib().orc_search(corpus.ref(), queries.ref(), pr, C.c_uint32(W), pe, C.c_uint32(len(entry)), pw, C.c_uint32(cands),
                          C.c_uint32(max_iter), ids.ctypes.data_as(u32p), dist.ctypes.data_as(f32p), counters.ctypes.data_as(u64p), threads)
     else:
