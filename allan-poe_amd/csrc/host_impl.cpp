@@ -253,7 +253,22 @@ SearchResult search_index_impl(const std::string& dense_data_path, const std::st
     // the reference searches the first 100 queries only (query.cu:1825)
     query_num = std::min(query_num, opt.max_queries);
     std::cout << "query num: " << query_num << std::endl;
-    if (!keyword_id_path.empty()) fail("keyword-filtered search (keyword_id_path) is not available in this build");
+    // query.cu:1828-1843: a BM25 term of query i that line i of the keyword file lists becomes a
+    // required keyword (bit 31 of its id)
+    const bool have_keywords = !keyword_id_path.empty();
+    if (have_keywords) {
+        std::vector<std::vector<unsigned>> keyword_vec(query_num);
+        load_txt(keyword_id_path, keyword_vec, query_num);
+        unsigned t_count = 0;
+        for (unsigned i = 0; i < query_num; i++)
+            for (unsigned j = qbm25.off[i]; j < qbm25.off[i + 1]; j++)
+                for (unsigned kw : keyword_vec[i])
+                    if (kw == qbm25.idx[j]) {
+                        qbm25.idx[j] |= 0x80000000u;
+                        t_count += 1;
+                    }
+        std::cout << "keywords: " << t_count << std::endl;
+    }
     if (have_kg && query_entity_num < query_num + 1) fail("query entity file has fewer rows than queries");
 
     std::cout << "Dense weight: " << dense_weight << ", Sparse weight: " << sparse_weight << ", BM25 weight: " << bm25_weight
@@ -292,9 +307,13 @@ SearchResult search_index_impl(const std::string& dense_data_path, const std::st
     std::cout << "Begin search" << std::endl;
     const bool on_d = !(w3[0] < 1e-5f), on_s = !(w3[1] < 1e-5f), on_b = !(w3[2] < 1e-5f);
     const bool use_kg = !(kg_weight < 1e-5f);
+    // query.cu:2004-2047: the knowledge-graph search wins over the keyword filter, which wins over the weights
+    const bool use_keywords = have_keywords && !use_kg;
     if (use_kg) {
         std::cout << "Search with dense + sparse + bm25 + kg" << std::endl;
         if (!have_kg) fail("kg_weight is set but knowledge_path is empty"); // the reference launches nothing here (query.cu:2042-2047)
+    } else if (use_keywords) {
+        std::cout << "Search with dense + sparse + bm25 + keyword" << std::endl;
     } else {
         if (!on_d && !on_s && !on_b) fail("all three weights are zero"); // the reference launches nothing here
         std::string what;
@@ -314,6 +333,7 @@ SearchResult search_index_impl(const std::string& dense_data_path, const std::st
     p.w_bm25 = w3[2];
     p.kg_weight = kg_weight;
     p.cands = (unsigned)cands;
+    p.keyword_filter = use_keywords ? 1u : 0u;
     apoe_search_stats st{};
     const auto start = std::chrono::high_resolution_clock::now();
     check(apoe_search(h.ctx, h.corpus, h.queries, h.graph, use_kg ? h.kg : nullptr, &p, res.ids.data(), res.dist.data(), &st), "apoe_search");

@@ -84,6 +84,47 @@ def test_build_and_search_roundtrip(files, capfd):
     assert (rk["ids"][:, :10] == kid[:, :10]).mean() > 0.97
 
 
+def test_keyword_file_search(files, capfd):
+    """keyword_id_path: line i lists term ids; those that are BM25 terms of query i become required keywords
+    (query.cu:1828-1843) and the keyword-filter search runs (query.cu:2005-2007)."""
+    import hybrid_search
+    import oracle as O
+    p, C, Q = files["paths"], files["C"], files["Q"]
+    if not os.path.exists(p["index.poe"]):
+        hybrid_search.build_index(dense_data_path=p["dense.fvecs"], sparse_data_path=p["sparse.bin"], bm25_data_path=p["bm25.bin"],
+                                  output_graph_path=p["index.poe"], nnd_iters=8)
+    rows, entry = O.read_poe(p["index.poe"])
+    df = np.bincount(C.b_idx, minlength=int(max(C.b_idx.max(), Q.b_idx.max())) + 2)
+    kw_path = os.path.join(os.path.dirname(p["index.poe"]), "keywords.txt")
+    flagged = Q.b_idx.copy()
+    n_flag = 0
+    with open(kw_path, "w") as f:
+        for q in range(100):
+            terms = Q.b_idx[Q.b_off[q]:Q.b_off[q + 1]]
+            present = [int(t) for t in terms if df[t] > 0]
+            # the rarest term of the query that some document holds, plus an id no query has
+            pick = min(present, key=lambda t: df[t]) if present else None
+            f.write(" ".join(str(x) for x in ([pick] if pick is not None else []) + [4000000]) + "\n")
+            if pick is not None:
+                flagged[Q.b_off[q] + list(terms).index(pick)] |= 0x80000000
+                n_flag += 1
+    with open(p["qrels.txt"], "w") as f:
+        for q in range(100):
+            f.write("0\n")
+    r = hybrid_search.search(dense_data_path=p["dense.fvecs"], dense_query_path=p["qdense.fvecs"], sparse_data_path=p["sparse.bin"],
+                             sparse_query_path=p["qsparse.bin"], bm25_data_path=p["bm25.bin"], bm25_query_path=p["qbm25.bin"],
+                             keyword_id_path=kw_path, knowledge_path="", entity2doc_path="", query_entity_path="", graph_path=p["index.poe"],
+                             ground_truth_path=p["qrels.txt"], top_k=10, cands=64, sparse_weight=1.0, bm25_weight=1.0, dense_weight=1.0,
+                             kg_weight=0.0, calibrate=False)
+    out = capfd.readouterr().out
+    assert f"keywords: {n_flag}" in out and "Search with dense + sparse + bm25 + keyword" in out
+    assert out.index("query num: 100") < out.index("keywords:") < out.index("Dense weight:")
+    Qk = O.HybridSet(Q.dense, Q.s_off, Q.s_idx, Q.s_val, Q.b_off, flagged, Q.b_val).head(100)
+    oid, odist, _ = O.search(C, Qk, rows, entry, (1.0, 1.0, 1.0), 64, keyword_filter=True)
+    assert (r["ids"] == oid).all(axis=1).mean() > 0.97
+    assert (oid != 0x7FFFFFFF).any()
+
+
 def test_errors_raise(files):
     import hybrid_search
     p = files["paths"]
