@@ -471,6 +471,180 @@ __device__ __forceinline__ BoundedOut eval_finish(const PendingEval& p, const Pi
     return o;
 }
 
+// ---- bucket table: the query's terms for the search kernels ----
+// Two (key, value) entries per 16-byte bucket, so a lookup is ONE ds_read_b128 and no probe loop:
+// every lane can issue the reads for all its pairs (of several candidates) back to back instead of
+// walking a chain of dependent LDS reads whose length is set by the unluckiest lane. A term whose
+// bucket is already full goes to an overflow list that holds up to every term of the row (with
+// at least twice as many buckets as terms it is empty for most rows); its length is wave-uniform
+// and the list is only walked when it is not zero.
+struct BucketTab {
+    uint4* b;        // [mask + 1] buckets: (key0, value0, key1, value1)
+    uint2* ovf;      // overflow entries
+    uint32_t* n_ovf; // their number
+    uint32_t mask;
+};
+
+__device__ __forceinline__ void bucket_tab_clear(const BucketTab& T, int tid, int nthreads) {
+    for (uint32_t i = tid; i <= T.mask; i += nthreads) T.b[i] = make_uint4(EMPTY, 0u, EMPTY, 0u);
+    if (tid == 0) *T.n_ovf = 0;
+}
+
+// Keys inserted into one table are distinct.
+__device__ __forceinline__ void bucket_tab_insert(const BucketTab& T, uint32_t key, float val) {
+    uint4* e = T.b + term_hash(key, T.mask);
+    if (atomicCAS(&e->x, EMPTY, key) == EMPTY) { e->y = __float_as_uint(val); return; }
+    if (atomicCAS(&e->z, EMPTY, key) == EMPTY) { e->w = __float_as_uint(val); return; }
+    T.ovf[atomicAdd(T.n_ovf, 1u)] = make_uint2(key, __float_as_uint(val));
+}
+
+__device__ __forceinline__ void bucket_terms_from_query(const BucketTab& T, const SetView& Q, uint32_t q, float w_s, float w_b, bool use_s,
+                                                        bool use_b, int tid, int nthreads) {
+    if (use_s)
+        for (uint32_t j = Q.s_off[q] + tid; j < Q.s_off[q + 1]; j += nthreads) bucket_tab_insert(T, Q.s_idx[j], Q.s_val[j] * w_s);
+    if (use_b)
+        for (uint32_t j = Q.b_off[q] + tid; j < Q.b_off[q + 1]; j += nthreads)
+            bucket_tab_insert(T, Q.b_idx[j] | BM25_BIT, Q.b_val[j] * w_b);
+}
+
+// The per-lane part of stage 1: this lane's pairs of the candidate against the query's table.
+// Straight-line code on purpose: the three bucket reads of a candidate are issued back to back
+// and a lane without a pair at some position computes on a (0, 0) pair whose result is masked.
+template <bool KWD>
+__device__ __forceinline__ void bucket_match(const uint4 e, uint2 kv, bool valid, float& acc, const uint32_t* kwset, uint32_t kwmask, bool& hit) {
+    const bool m0 = e.x == kv.x, m1 = e.z == kv.x;
+    const float v = __uint_as_float(m0 ? e.y : e.w);
+    const bool found = valid && (m0 || m1);
+    const float next = fmaf(__uint_as_float(kv.y), v, acc);
+    acc = found ? next : acc;
+    if (KWD) {
+        if (found && (kv.x & BM25_BIT) && id_set_contains(kwset, kwmask, kv.x)) hit = true;
+    }
+}
+
+template <bool KWD>
+__device__ __forceinline__ void overflow_match(const BucketTab& T, uint32_t n_ovf, uint2 kv, bool valid, float& acc, const uint32_t* kwset,
+                                               uint32_t kwmask, bool& hit) {
+    for (uint32_t i = 0; i < n_ovf; i++) {
+        const uint2 o = T.ovf[i];
+        if (valid && o.x == kv.x) {
+            acc = fmaf(__uint_as_float(kv.y), __uint_as_float(o.y), acc);
+            if (KWD) {
+                if ((kv.x & BM25_BIT) && id_set_contains(kwset, kwmask, kv.x)) hit = true;
+            }
+        }
+    }
+}
+
+// n_ovf is the (wave-uniform) overflow count read after the table was built.
+template <bool KWD>
+__device__ __forceinline__ float sparse_probe(const PendingEval& p, const BucketTab& T, uint32_t n_ovf, uint32_t paths, const uint32_t* kwset,
+                                              uint32_t kwmask, bool& hit) {
+    const int lane = lane_id();
+    float acc = 0.f;
+    if (!(paths & (PATH_SPARSE | PATH_BM25))) return acc;
+    const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
+    const bool in0 = j0 < p.end, in1 = j1 < p.end, in2 = j2 < p.end;
+    uint4 e0 = T.b[term_hash(p.kv0.x, T.mask)];
+    uint4 e1 = T.b[term_hash(p.kv1.x, T.mask)];
+    uint4 e2 = T.b[term_hash(p.kv2.x, T.mask)];
+    // keep the three reads together: nothing below may be scheduled between them
+    asm volatile("" : "+v"(e0.x), "+v"(e1.x), "+v"(e2.x));
+    bucket_match<KWD>(e0, p.kv0, in0, acc, kwset, kwmask, hit);
+    bucket_match<KWD>(e1, p.kv1, in1, acc, kwset, kwmask, hit);
+    bucket_match<KWD>(e2, p.kv2, in2, acc, kwset, kwmask, hit);
+    if (n_ovf) {
+        overflow_match<KWD>(T, n_ovf, p.kv0, in0, acc, kwset, kwmask, hit);
+        overflow_match<KWD>(T, n_ovf, p.kv1, in1, acc, kwset, kwmask, hit);
+        overflow_match<KWD>(T, n_ovf, p.kv2, in2, acc, kwset, kwmask, hit);
+    }
+    if (p.begin + 3 * WAVE < p.end) { // rows with more than 192 pairs
+        const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
+        for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) {
+            const uint2 kv = sp[j];
+            bucket_match<KWD>(T.b[term_hash(kv.x, T.mask)], kv, true, acc, kwset, kwmask, hit);
+            overflow_match<KWD>(T, n_ovf, kv, true, acc, kwset, kwmask, hit);
+        }
+    }
+    return acc;
+}
+
+// The wave-level part of stage 1: reduce, then decide whether the dense row is needed at all.
+struct SparseOut {
+    float v;      // decided: the distance to report (INF_DIS if the bound rejects); else the sparse sum
+    bool decided; // no dense row needed
+};
+
+__device__ __forceinline__ SparseOut sparse_decide(const PendingEval& p, float acc, uint32_t paths, float bonus, float thr) {
+    SparseOut o;
+    float ssum = 0.f;
+    if (paths & (PATH_SPARSE | PATH_BM25)) {
+        ssum = wave_sum_dpp(acc);
+        if (!(paths & PATH_DENSE)) {
+            o.v = 1.0f - ssum - bonus;
+            o.decided = true;
+            return o;
+        }
+        const float lb = 1.0f - (ssum + p.dub) - bonus;
+        if (lb > thr + 1e-5f * (fabsf(ssum) + p.dub + fabsf(bonus) + 1.0f)) {
+            o.v = INF_DIS;
+            o.decided = true;
+            return o;
+        }
+    }
+    o.v = ssum;
+    o.decided = false;
+    return o;
+}
+
+struct DenseRow {
+    float4 x[NV];
+};
+__device__ __forceinline__ void dense_issue(DenseRow& d, const char* rec) {
+    const float4* r = reinterpret_cast<const float4*>(rec);
+    const int lane = lane_id();
+#pragma unroll
+    for (int i = 0; i < NV; i++) d.x[i] = r[lane + WAVE * i];
+}
+// dense_mul * <row, pivot>, the same FMA chain and reduction as eval_finish.
+__device__ __forceinline__ float dense_finish(const DenseRow& d, const PivotDense& pv, float dense_mul) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        acc = fmaf(d.x[i].x, pv.v[i].x, acc);
+        acc = fmaf(d.x[i].y, pv.v[i].y, acc);
+        acc = fmaf(d.x[i].z, pv.v[i].z, acc);
+        acc = fmaf(d.x[i].w, pv.v[i].w, acc);
+    }
+    return dense_mul * wave_sum_dpp(acc);
+}
+
+// The same with the pivot's dense row in LDS (float4 number l + 64*i belongs to lane l, as in
+// PivotDense): frees 64 registers per lane for kernels that need the occupancy more.
+__device__ __forceinline__ float dense_finish_lds(const DenseRow& d, const float4* pivot, float dense_mul) {
+    const int lane = lane_id();
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const float4 p = pivot[lane + WAVE * i];
+        acc = fmaf(d.x[i].x, p.x, acc);
+        acc = fmaf(d.x[i].y, p.y, acc);
+        acc = fmaf(d.x[i].z, p.z, acc);
+        acc = fmaf(d.x[i].w, p.w, acc);
+    }
+    return dense_mul * wave_sum_dpp(acc);
+}
+__device__ __forceinline__ float pivot_dense_norm_lds(const float4* pivot) {
+    const int lane = lane_id();
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const float4 p = pivot[lane + WAVE * i];
+        a += p.x * p.x + p.y * p.y + p.z * p.z + p.w * p.w;
+    }
+    return sqrtf(wave_sum_dpp(a));
+}
+
 // splitmix64 finaliser (random initial neighbours).
 __host__ __device__ inline uint64_t mix64(uint64_t z) {
     z += 0x9E3779B97F4A7C15ull;

@@ -6,7 +6,8 @@
 namespace apoe {
 
 constexpr int MAX_NEW = 64;   // fresh candidates per step: one lane each in wave 0
-constexpr int EVAL_BATCH = 2; // candidates whose sparse parts a wave keeps in flight together
+constexpr int EVAL_BATCH = 3;  // candidates whose sparse parts a wave keeps in flight together
+constexpr int DENSE_BATCH = 1; // dense rows a wave keeps in flight together
 constexpr int RING = 32;      // keyword-filter search: evicted keyword hits kept beside the pool (query.cu:18)
 
 // What the kernel does on top of the plain beam search.
@@ -38,34 +39,37 @@ struct SearchArgs {
 
 // LDS carve-up shared by host (size) and device (pointers).
 struct SearchLds {
-    uint32_t tab, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ring_id,
+    uint32_t qd, tab, ovf, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ring_id,
         ring_dist, kwset, ctl, total;
     __host__ __device__ SearchLds(uint32_t slots, uint32_t cands, int mode, uint32_t kw_slots) {
         const bool kg = mode == MODE_KG, kwd = mode == MODE_KEYWORD;
+        // fixed-size arrays first: their offsets are compile-time constants
         uint32_t o = 0;
-        tab = o; o += slots * 8;
+        qd = o; o += DENSE_BYTES;       // the query's dense row, weight applied
+        ctl = o; o += 16 * 4;
+        new_lb = o; o += MAX_NEW * 4;
+        new_id = o; o += MAX_NEW * 4;
+        new_dist = o; o += MAX_NEW * 4;
+        new_ent = o; o += MAX_NEW * 4;  // KG: linking entity; keyword search: the hit flag of a fresh candidate
+        new_hop = o; o += MAX_NEW * 4;
+        link = o; o += MAX_NEW * 4;
+        ring_id = o; o += RING * 4;
+        ring_dist = o; o += RING * 4;
+        tab = o; o += slots * 16;     // buckets of two (key, value) entries
+        ovf = o; o += slots / 2 * 8;  // overflow entries: up to every term of the longest query row
         pool_id = o; o += cands * 4;
         pool_dist = o; o += cands * 4;
         pool_ent = o; o += kg ? cands * 4 : 0;
         pool_hop = o; o += kg ? cands * 4 : 0;
-        new_lb = o; o += MAX_NEW * 4;
-        new_id = o; o += MAX_NEW * 4;
-        new_dist = o; o += MAX_NEW * 4;
-        new_ent = o; o += (kg || kwd) ? MAX_NEW * 4 : 0; // keyword search: the hit flag of a fresh candidate
-        new_hop = o; o += kg ? MAX_NEW * 4 : 0;
         seed_id = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
         seed_ent = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
         seed_dist = o; o += kg ? (cands + MAX_NEW) * 4 : 0;
-        link = o; o += kg ? MAX_NEW * 4 : 0;
-        ring_id = o; o += kwd ? RING * 4 : 0;
-        ring_dist = o; o += kwd ? RING * 4 : 0;
         kwset = o; o += kwd ? kw_slots * 4 : 0;
-        ctl = o; o += 16 * 4;
         total = o;
     }
 };
 
-enum { CTL_QUERY = 0, CTL_PARENT = 1, CTL_NNEW = 2, CTL_NSEED = 3 };
+enum { CTL_QUERY = 0, CTL_PARENT = 1, CTL_NNEW = 2, CTL_NSEED = 3, CTL_NOVF = 4 };
 
 struct Pool {
     uint32_t* id;   // [cands], ascending distance
@@ -200,7 +204,13 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
     constexpr bool KG = MODE == MODE_KG, KWD = MODE == MODE_KEYWORD;
     extern __shared__ __align__(16) char smem[];
     const SearchLds L(a.slots, a.cands, MODE, a.kw_slots);
-    uint2* tab = reinterpret_cast<uint2*>(smem + L.tab);
+    volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
+    float4* qd = reinterpret_cast<float4*>(smem + L.qd);
+    BucketTab T;
+    T.b = reinterpret_cast<uint4*>(smem + L.tab);
+    T.ovf = reinterpret_cast<uint2*>(smem + L.ovf);
+    T.n_ovf = const_cast<uint32_t*>(&ctl[CTL_NOVF]);
+    T.mask = a.slots - 1;
     Pool P;
     P.id = reinterpret_cast<uint32_t*>(smem + L.pool_id);
     P.dist = reinterpret_cast<float*>(smem + L.pool_dist);
@@ -221,10 +231,9 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
     R.id = reinterpret_cast<uint32_t*>(smem + L.ring_id);
     R.dist = reinterpret_cast<float*>(smem + L.ring_dist);
     R.n = 0;
-    volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
 
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
-    const uint32_t mask = a.slots - 1, cands = a.cands;
+    const int tid = threadIdx.x, wave = (int)uniform(tid / WAVE), lane = lane_id();
+    const uint32_t cands = a.cands;
     uint32_t* bitmap = a.bitmaps + (size_t)blockIdx.x * a.bitmap_words;
     const uint64_t lane_lt = (1ull << lane) - 1;
 
@@ -241,7 +250,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             uint4* b4 = reinterpret_cast<uint4*>(bitmap);
             for (uint32_t i = tid; i < a.bitmap_words / 4; i += NW * WAVE) b4[i] = make_uint4(0, 0, 0, 0);
         }
-        term_table_clear(tab, a.slots, tid, NW * WAVE);
+        bucket_tab_clear(T, tid, NW * WAVE);
         if (KWD) {
             for (uint32_t i = tid; i < a.kw_slots; i += NW * WAVE) kwset[i] = EMPTY;
             R.n = 0;
@@ -251,11 +260,16 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             P.dist[i] = INF_DIS;
             if (KG) { P.ent[i] = EMPTY; P.hop[i] = 0; }
         }
-        PivotDense pv;
-        pivot_dense_load(pv, a.Q.dense + (size_t)q * DIM, a.w_d);
+        {
+            const float4* src = reinterpret_cast<const float4*>(a.Q.dense + (size_t)q * DIM);
+            for (uint32_t i = tid; i < DIM / 4; i += NW * WAVE) {
+                const float4 x = src[i];
+                qd[i] = make_float4(x.x * a.w_d, x.y * a.w_d, x.z * a.w_d, x.w * a.w_d);
+            }
+        }
         __threadfence();
         __syncthreads();
-        pivot_terms_from_query(tab, mask, a.Q, q, a.w_s, a.w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
+        bucket_terms_from_query(T, a.Q, q, a.w_s, a.w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
         if (KWD) {
             // required keywords: BM25 query terms whose id arrives with bit 31 set (query.cu:1828-1843)
             for (uint32_t j = a.Q.b_off[q] + tid; j < a.Q.b_off[q + 1]; j += NW * WAVE) {
@@ -264,7 +278,8 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             }
         }
 
-        const float pv_norm = pivot_dense_norm(pv);
+        __syncthreads();
+        const float pv_norm = pivot_dense_norm_lds(qd);
         uint64_t st_exp = 0, st_eval = 0, st_ns = 0, st_nb = 0, st_dense = 0; // wave-uniform counters
         uint32_t hint = 0;                                       // wave 0: every pool slot below hint is explored
 
@@ -323,15 +338,26 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             }
             __syncthreads();
             const uint32_t n_seed = ctl[CTL_NSEED];
+            const uint32_t n_ovf_seed = uniform(ctl[CTL_NOVF]);
             for (uint32_t j = wave; j < n_seed; j += NW) {
                 const uint32_t id = uniform(seed_id[j]);
                 const float bonus = seed_ent[j] != EMPTY ? a.kg_weight : 0.0f; // query.cu:1637-1638
-                BoundedOut e = eval_wave_bounded(a.C, id, pv, pv_norm, tab, mask, a.paths, 1.0f, bonus, __builtin_inff());
+                PendingEval pe;
+                eval_issue(pe, a.C, id, pv_norm, a.paths, 1.0f);
+                bool hit = false;
+                const float acc = sparse_probe<false>(pe, T, n_ovf_seed, a.paths, nullptr, 0, hit);
+                const SparseOut so = sparse_decide(pe, acc, a.paths, bonus, __builtin_inff());
+                float dist = so.v;
+                if (!so.decided) {
+                    DenseRow row;
+                    dense_issue(row, pe.rec);
+                    dist = 1.0f - (dense_finish_lds(row, qd, 1.0f) + so.v) - bonus;
+                    st_dense++;
+                }
                 st_eval++;
-                st_ns += e.nnz_s;
-                st_nb += e.nnz_b;
-                st_dense += e.dense_read;
-                if (lane == 0) seed_dist[j] = e.dist;
+                st_ns += (a.paths & PATH_SPARSE) ? pe.ns : 0u;
+                st_nb += (a.paths & PATH_BM25) ? pe.nb : 0u;
+                if (lane == 0) seed_dist[j] = dist;
             }
             __syncthreads();
             if (wave == 0) {
@@ -359,6 +385,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             // it is reported as INF_DIS and falls off the end of the merge like any other loser
             const float thr = a.full_eval ? __builtin_inff() : P.dist[cands - 1];
             const float thr_eff = thr < INF_DIS ? thr : __builtin_inff();
+            const uint32_t n_ovf = uniform(ctl[CTL_NOVF]);
             // descriptors and dense norms of all fresh candidates in one gather: lane l holds candidate l's
             uint64_t my_desc = 0;
             float my_dn = 0.f;
@@ -367,30 +394,72 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                 my_desc = a.C.desc[cid];
                 my_dn = a.C.dnorm[cid];
             }
-            for (uint32_t j = wave; j < n_new; j += NW * EVAL_BATCH) {
-                PendingEval pe[EVAL_BATCH];
+            // stage 1: the sparse parts of this wave's candidates, EVAL_BATCH of them in flight
+            uint64_t need = 0; // bit t: the wave's t-th candidate (id wave + t*NW) still needs its dense row
+            {
+                uint32_t t0 = 0;
+                for (uint32_t j = wave; j < n_new; j += NW * EVAL_BATCH, t0 += EVAL_BATCH) {
+                    PendingEval pe[EVAL_BATCH];
 #pragma unroll
-                for (int b = 0; b < EVAL_BATCH; b++) {
-                    const uint32_t jj = j + b * NW;
-                    if (jj < n_new) eval_issue_desc(pe[b], a.C, readlane64(my_desc, jj), readlane_f32(my_dn, jj), pv_norm, a.paths, 1.0f);
+                    for (int b = 0; b < EVAL_BATCH; b++) {
+                        const uint32_t jj = j + b * NW;
+                        if (jj < n_new) eval_issue_desc(pe[b], a.C, readlane64(my_desc, jj), readlane_f32(my_dn, jj), pv_norm, a.paths, 1.0f);
+                    }
+                    float acc[EVAL_BATCH];
+                    bool hit[EVAL_BATCH];
+#pragma unroll
+                    for (int b = 0; b < EVAL_BATCH; b++) {
+                        hit[b] = false;
+                        acc[b] = 0.f;
+                        if (j + b * NW < n_new) acc[b] = sparse_probe<KWD>(pe[b], T, n_ovf, a.paths, kwset, a.kw_slots - 1, hit[b]);
+                    }
+#pragma unroll
+                    for (int b = 0; b < EVAL_BATCH; b++) {
+                        const uint32_t jj = j + b * NW;
+                        if (jj < n_new) {
+                            float bonus = 0.f;
+                            if (KG) {
+                                if (new_ent[jj] != EMPTY) bonus = a.kg_weight / (float)new_hop[jj]; // query.cu:1759-1760
+                            }
+                            const SparseOut so = sparse_decide(pe[b], acc[b], a.paths, bonus, thr_eff);
+                            const bool kw_hit = KWD ? __ballot(hit[b]) != 0 : false;
+                            st_eval++;
+                            st_ns += (a.paths & PATH_SPARSE) ? pe[b].ns : 0u;
+                            st_nb += (a.paths & PATH_BM25) ? pe[b].nb : 0u;
+                            if (lane == 0) {
+                                new_dist[jj] = so.v;
+                                if (KWD) new_ent[jj] = kw_hit ? 1u : 0u;
+                            }
+                            if (!so.decided) need |= 1ull << (t0 + b);
+                        }
+                    }
+                }
+            }
+            wave_fence();
+            // stage 2: the dense rows of the survivors, DENSE_BATCH rows in flight
+            while (need) {
+                DenseRow row[DENSE_BATCH];
+                uint32_t jj[DENSE_BATCH];
+#pragma unroll
+                for (int b = 0; b < DENSE_BATCH; b++) {
+                    jj[b] = EMPTY;
+                    if (need) {
+                        const uint32_t t = __builtin_ctzll(need);
+                        need &= need - 1;
+                        jj[b] = wave + t * NW;
+                        dense_issue(row[b], a.C.recs + desc_off(readlane64(my_desc, jj[b])) * 16);
+                    }
                 }
 #pragma unroll
-                for (int b = 0; b < EVAL_BATCH; b++) {
-                    const uint32_t jj = j + b * NW;
-                    if (jj < n_new) {
+                for (int b = 0; b < DENSE_BATCH; b++) {
+                    if (jj[b] != EMPTY) {
                         float bonus = 0.f;
                         if (KG) {
-                            if (new_ent[jj] != EMPTY) bonus = a.kg_weight / (float)new_hop[jj]; // query.cu:1759-1760
+                            if (new_ent[jj[b]] != EMPTY) bonus = a.kg_weight / (float)new_hop[jj[b]];
                         }
-                        BoundedOut e = eval_finish<KWD>(pe[b], pv, tab, mask, a.paths, 1.0f, bonus, thr_eff, kwset, a.kw_slots - 1);
-                        st_eval++;
-                        st_ns += e.nnz_s;
-                        st_nb += e.nnz_b;
-                        st_dense += e.dense_read;
-                        if (lane == 0) {
-                            new_dist[jj] = e.dist;
-                            if (KWD) new_ent[jj] = e.kw_hit ? 1u : 0u;
-                        }
+                        const float dsum = dense_finish_lds(row[b], qd, 1.0f);
+                        st_dense++;
+                        if (lane == 0) new_dist[jj[b]] = 1.0f - (dsum + new_dist[jj[b]]) - bonus;
                     }
                 }
             }
