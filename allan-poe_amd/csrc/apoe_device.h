@@ -645,6 +645,100 @@ __device__ __forceinline__ float pivot_dense_norm_lds(const float4* pivot) {
     return sqrtf(wave_sum_dpp(a));
 }
 
+// ---- four-entry bucket table: a document's terms as pivot (NN-Descent) ----
+// Same idea as BucketTab with 32-byte buckets (two ds_read_b128 per lookup), which keeps the table
+// at 8 bytes per slot for rows of several hundred terms. A term whose bucket is full goes to the
+// overflow list (wave-uniform length, walked only when not empty); should even that list be full,
+// lookups fall back to scanning the pivot's own pair array in global memory (correct, slow, and
+// not reachable with a hash that spreads the row's terms).
+struct Bucket4Tab {
+    uint4* b;        // [2 * (mask + 1)]: bucket i is b[2i], b[2i+1] = (k0, v0, k1, v1), (k2, v2, k3, v3)
+    uint2* ovf;      // [ovf_cap]
+    uint32_t* n_ovf; // terms that found their bucket full (may exceed ovf_cap)
+    uint32_t mask, ovf_cap;
+};
+
+__device__ __forceinline__ void bucket4_clear(const Bucket4Tab& T, int tid, int nthreads) {
+    for (uint32_t i = tid; i < 2 * (T.mask + 1); i += nthreads) T.b[i] = make_uint4(EMPTY, 0u, EMPTY, 0u);
+    if (tid == 0) *T.n_ovf = 0;
+}
+
+__device__ __forceinline__ void bucket4_insert(const Bucket4Tab& T, uint32_t key, uint32_t val_bits) {
+    uint4* e = T.b + 2 * term_hash(key, T.mask);
+    if (atomicCAS(&e[0].x, EMPTY, key) == EMPTY) { e[0].y = val_bits; return; }
+    if (atomicCAS(&e[0].z, EMPTY, key) == EMPTY) { e[0].w = val_bits; return; }
+    if (atomicCAS(&e[1].x, EMPTY, key) == EMPTY) { e[1].y = val_bits; return; }
+    if (atomicCAS(&e[1].z, EMPTY, key) == EMPTY) { e[1].w = val_bits; return; }
+    const uint32_t at = atomicAdd(T.n_ovf, 1u);
+    if (at < T.ovf_cap) T.ovf[at] = make_uint2(key, val_bits);
+}
+
+__device__ __forceinline__ void bucket4_terms_from_record(const Bucket4Tab& T, const char* rec, uint32_t nnz, int tid, int nthreads) {
+    const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
+    for (uint32_t j = tid; j < nnz; j += nthreads) {
+        const uint2 kv = sp[j];
+        bucket4_insert(T, kv.x, kv.y);
+    }
+}
+
+__device__ __forceinline__ bool bucket4_match(const uint4 e0, const uint4 e1, uint2 kv, bool valid, float& acc) {
+    const bool m0 = e0.x == kv.x, m1 = e0.z == kv.x, m2 = e1.x == kv.x, m3 = e1.z == kv.x;
+    const float v = __uint_as_float(m0 ? e0.y : m1 ? e0.w : m2 ? e1.y : e1.w);
+    const bool found = valid && (m0 || m1 || m2 || m3);
+    const float next = fmaf(__uint_as_float(kv.y), v, acc);
+    acc = found ? next : acc;
+    return found;
+}
+
+// Terms that are not in their bucket: the overflow list, or the pivot's pair array if the list overflowed.
+__device__ __forceinline__ void bucket4_overflow(const Bucket4Tab& T, uint32_t n_ovf, const uint2* pivot_pairs, uint32_t pivot_nnz, uint2 kv,
+                                                 bool pending, float& acc) {
+    if (n_ovf <= T.ovf_cap) {
+        for (uint32_t i = 0; i < n_ovf; i++) {
+            const uint2 o = T.ovf[i];
+            if (pending && o.x == kv.x) acc = fmaf(__uint_as_float(kv.y), __uint_as_float(o.y), acc);
+        }
+    } else {
+        for (uint32_t i = 0; i < pivot_nnz; i++) {
+            const uint2 o = pivot_pairs[i];
+            if (pending && o.x == kv.x) acc = fmaf(__uint_as_float(kv.y), __uint_as_float(o.y), acc);
+        }
+    }
+}
+
+// Per-lane part of stage 1 against a document pivot (all paths on).
+__device__ __forceinline__ float doc_sparse_probe(const PendingEval& p, const Bucket4Tab& T, uint32_t n_ovf, const uint2* pivot_pairs,
+                                                  uint32_t pivot_nnz) {
+    const int lane = lane_id();
+    float acc = 0.f;
+    const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
+    const bool in0 = j0 < p.end, in1 = j1 < p.end, in2 = j2 < p.end;
+    const uint4* b0 = T.b + 2 * term_hash(p.kv0.x, T.mask);
+    const uint4* b1 = T.b + 2 * term_hash(p.kv1.x, T.mask);
+    const uint4* b2 = T.b + 2 * term_hash(p.kv2.x, T.mask);
+    uint4 e00 = b0[0], e01 = b0[1], e10 = b1[0], e11 = b1[1], e20 = b2[0], e21 = b2[1];
+    // keep the six reads together: nothing below may be scheduled between them
+    asm volatile("" : "+v"(e00.x), "+v"(e01.x), "+v"(e10.x), "+v"(e11.x), "+v"(e20.x), "+v"(e21.x));
+    const bool f0 = bucket4_match(e00, e01, p.kv0, in0, acc);
+    const bool f1 = bucket4_match(e10, e11, p.kv1, in1, acc);
+    const bool f2 = bucket4_match(e20, e21, p.kv2, in2, acc);
+    if (n_ovf) {
+        bucket4_overflow(T, n_ovf, pivot_pairs, pivot_nnz, p.kv0, in0 && !f0, acc);
+        bucket4_overflow(T, n_ovf, pivot_pairs, pivot_nnz, p.kv1, in1 && !f1, acc);
+        bucket4_overflow(T, n_ovf, pivot_pairs, pivot_nnz, p.kv2, in2 && !f2, acc);
+    }
+    if (p.begin + 3 * WAVE < p.end) { // rows with more than 192 pairs
+        const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
+        for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) {
+            const uint2 kv = sp[j];
+            const uint4* bb = T.b + 2 * term_hash(kv.x, T.mask);
+            const bool f = bucket4_match(bb[0], bb[1], kv, true, acc);
+            if (n_ovf) bucket4_overflow(T, n_ovf, pivot_pairs, pivot_nnz, kv, !f, acc);
+        }
+    }
+    return acc;
+}
+
 // splitmix64 finaliser (random initial neighbours).
 __host__ __device__ inline uint64_t mix64(uint64_t z) {
     z += 0x9E3779B97F4A7C15ull;

@@ -9,6 +9,8 @@ namespace apoe {
 
 constexpr int NND_THREADS = 256;
 constexpr int NND_PICKS = 4; // neighbours sampled per node and step (index.cu:157,171-181)
+constexpr int NND_EVAL_BATCH = 4;  // candidates whose sparse parts a wave keeps in flight
+constexpr int NND_DENSE_BATCH = 2; // dense rows a wave keeps in flight
 constexpr uint32_t ALLP = PATH_DENSE | PATH_SPARSE | PATH_BM25;
 
 __device__ __forceinline__ float key_dist(uint64_t key) {
@@ -105,7 +107,11 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
                                                                   uint32_t seen_slots, unsigned long long* inserted) {
     extern __shared__ __align__(16) char smem[];
     const NndLds L(term_slots, seen_slots, K);
-    uint2* tab = reinterpret_cast<uint2*>(smem + L.tab);
+    // the dedupe set is dead once the candidates are gathered: the pivot's dense row and the overflow
+    // list of its term table take its place; the survivor array doubles as the list of candidates
+    // that need their dense row
+    float4* qd = reinterpret_cast<float4*>(smem + L.seen);
+    unsigned long long* need = reinterpret_cast<unsigned long long*>(smem + L.surv);
     uint64_t* surv = reinterpret_cast<uint64_t*>(smem + L.surv);
     uint64_t* new_sorted = reinterpret_cast<uint64_t*>(smem + L.new_sorted);
     uint32_t* seen = reinterpret_cast<uint32_t*>(smem + L.seen);
@@ -117,14 +123,21 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
     float* m_dist = reinterpret_cast<float*>(smem + L.m_dist);
     uint32_t* ctl = reinterpret_cast<uint32_t*>(smem + L.ctl); // [0..3] picks, [4] n_picks, [5] n_cand, [6] n_surv, [7] n_ins
 
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
-    const uint32_t u = blockIdx.x, tmask = term_slots - 1, smask = seen_slots - 1;
+    const int tid = threadIdx.x, wave = (int)uniform(tid / WAVE), lane = lane_id();
+    const uint32_t u = blockIdx.x, smask = seen_slots - 1;
+    Bucket4Tab T;
+    T.b = reinterpret_cast<uint4*>(smem + L.tab);
+    T.ovf = reinterpret_cast<uint2*>(smem + L.seen + DENSE_BYTES);
+    T.n_ovf = &ctl[8];
+    T.mask = term_slots / 4 - 1;
+    T.ovf_cap = min(term_slots / 8, (seen_slots * 4 - DENSE_BYTES) / 8);
     const size_t base = (size_t)u * K;
 
     for (uint32_t i = tid; i < K; i += NND_THREADS) { own_id[i] = ids[base + i]; own_dist[i] = dist[base + i]; }
-    term_table_clear(tab, term_slots, tid, NND_THREADS);
+    bucket4_clear(T, tid, NND_THREADS);
     for (uint32_t i = tid; i < seen_slots; i += NND_THREADS) seen[i] = EMPTY;
     if (tid < 8) ctl[tid] = 0;
+    if (tid == 9) ctl[9] = 0;
     __syncthreads();
 
     // 1. picks: group g takes the first unsampled slot >= g; none left -> slot 0
@@ -163,35 +176,93 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
         else c = (uint32_t)rev[(size_t)v * K + (r - K)];
         if (c < C.n && id_set_insert(seen, smask, c)) cand_id[atomicAdd(&ctl[5], 1u)] = c;
     }
-    // pivot = u
+    __syncthreads();
+    // pivot = u: dense row into LDS (float4 number l + 64*i belongs to lane l), terms into the bucket table
     const uint64_t du = C.desc[u];
     const char* rec = C.recs + desc_off(du) * 16;
-    PivotDense pv;
-    pivot_dense_load(pv, reinterpret_cast<const float*>(rec), 1.0f);
-    pivot_terms_from_record(tab, tmask, rec, desc_nnz_s(du) + desc_nnz_b(du), tid, NND_THREADS);
+    const uint32_t u_nnz = desc_nnz_s(du) + desc_nnz_b(du);
+    {
+        const float4* src = reinterpret_cast<const float4*>(rec);
+        for (uint32_t i = tid; i < DIM / 4; i += NND_THREADS) qd[i] = src[i];
+    }
+    bucket4_terms_from_record(T, rec, u_nnz, tid, NND_THREADS);
     __syncthreads();
 
     // 4. distances; only those below the current worst matter (step 5), so a candidate whose
-    //    sparse part plus the bound of its dense part cannot get there is not read in full
+    //    sparse part plus the bound of its dense part cannot get there is not read in full.
+    //    Stage 1 settles the sparse parts (EVAL_BATCH candidates of a wave in flight), stage 2 reads
+    //    the dense rows of the rest (DENSE_BATCH rows in flight), shared out again over the waves.
+    constexpr int NW = NND_THREADS / WAVE;
     const uint32_t n_cand = ctl[5];
     const float worst = own_dist[K - 1];
     const float thr = worst < INF_DIS ? worst : __builtin_inff();
-    const float pv_norm = pivot_dense_norm(pv);
-    unsigned long long n_dense = 0;
-    for (uint32_t j = wave; j < n_cand; j += (NND_THREADS / WAVE) * 2) {
-        const uint32_t j2 = j + NND_THREADS / WAVE;
-        PendingEval p0, p1;
-        eval_issue(p0, C, uniform(cand_id[j]), pv_norm, ALLP, dense_mul);
-        if (j2 < n_cand) eval_issue(p1, C, uniform(cand_id[j2]), pv_norm, ALLP, dense_mul);
-        BoundedOut e0 = eval_finish(p0, pv, tab, tmask, ALLP, dense_mul, 0.f, thr);
-        n_dense += e0.dense_read;
-        if (lane == 0) cand_dist[j] = e0.dist;
-        if (j2 < n_cand) {
-            BoundedOut e1 = eval_finish(p1, pv, tab, tmask, ALLP, dense_mul, 0.f, thr);
-            n_dense += e1.dense_read;
-            if (lane == 0) cand_dist[j2] = e1.dist;
+    const float pv_norm = pivot_dense_norm_lds(qd);
+    const uint32_t n_ovf = uniform(ctl[8]);
+    const uint2* u_pairs = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
+    for (uint32_t c0 = 0; c0 * NW < n_cand; c0 += WAVE) {
+        // lane l fetches descriptor and dense norm of the wave's (c0 + l)-th candidate
+        uint64_t my_desc = 0;
+        float my_dn = 0.f;
+        {
+            const uint32_t jl = wave + (c0 + lane) * NW;
+            if (jl < n_cand) {
+                const uint32_t cid = cand_id[jl];
+                my_desc = C.desc[cid];
+                my_dn = C.dnorm[cid];
+            }
+        }
+        for (uint32_t t = 0; t < WAVE && wave + (c0 + t) * NW < n_cand; t += NND_EVAL_BATCH) {
+            PendingEval pe[NND_EVAL_BATCH];
+            float acc[NND_EVAL_BATCH];
+#pragma unroll
+            for (int b = 0; b < NND_EVAL_BATCH; b++) {
+                const uint32_t jj = wave + (c0 + t + b) * NW;
+                if (t + b < WAVE && jj < n_cand) eval_issue_desc(pe[b], C, readlane64(my_desc, t + b), readlane_f32(my_dn, t + b), pv_norm, ALLP, dense_mul);
+            }
+#pragma unroll
+            for (int b = 0; b < NND_EVAL_BATCH; b++) {
+                const uint32_t jj = wave + (c0 + t + b) * NW;
+                acc[b] = 0.f;
+                if (t + b < WAVE && jj < n_cand) acc[b] = doc_sparse_probe(pe[b], T, n_ovf, u_pairs, u_nnz);
+            }
+#pragma unroll
+            for (int b = 0; b < NND_EVAL_BATCH; b++) {
+                const uint32_t jj = wave + (c0 + t + b) * NW;
+                if (t + b < WAVE && jj < n_cand) {
+                    const SparseOut so = sparse_decide(pe[b], acc[b], ALLP, 0.f, thr);
+                    if (lane == 0) {
+                        cand_dist[jj] = so.v;
+                        if (!so.decided) need[atomicAdd(&ctl[9], 1u)] = ((unsigned long long)jj << 40) | desc_off(readlane64(my_desc, t + b));
+                    }
+                }
+            }
         }
     }
+    __syncthreads();
+    const uint32_t n_need = ctl[9];
+    for (uint32_t t = wave; t < n_need; t += NW * NND_DENSE_BATCH) {
+        DenseRow row[NND_DENSE_BATCH];
+        uint32_t jj[NND_DENSE_BATCH];
+#pragma unroll
+        for (int b = 0; b < NND_DENSE_BATCH; b++) {
+            const uint32_t tt = t + b * NW;
+            jj[b] = EMPTY;
+            if (tt < n_need) {
+                const unsigned long long e = need[tt];
+                const uint32_t lo = uniform((uint32_t)e), hi = uniform((uint32_t)(e >> 32));
+                jj[b] = hi >> 8;
+                dense_issue(row[b], C.recs + ((((uint64_t)(hi & 0xFFu)) << 32) | lo) * 16);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < NND_DENSE_BATCH; b++) {
+            if (jj[b] != EMPTY) {
+                const float dsum = dense_finish_lds(row[b], qd, dense_mul);
+                if (lane == 0) cand_dist[jj[b]] = 1.0f - (dsum + cand_dist[jj[b]]) - 0.f;
+            }
+        }
+    }
+    const unsigned long long n_dense = wave == 0 ? n_need : 0;
     if (lane == 0 && n_dense) atomicAdd(inserted + 3, n_dense);
     if (tid == 0) atomicAdd(inserted + 2, (unsigned long long)n_cand);
     __syncthreads();

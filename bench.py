@@ -101,6 +101,9 @@ def main():
     ap.add_argument("--cpu-queries", type=int, default=2000)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time the other search paths at cands=128: the query-time weight sweep, the knowledge-graph search "
+                         "(200k entities, 1-3 entities per query, kg_weight 40) and the keyword-filter search (rarest BM25 term of each query)")
     ap.add_argument("--calibrate", action="store_true",
                     help="apply the reference's query-time weight calibration to the 1/1/1 weights (off: the metric is literally 1/1/1)")
     ap.add_argument("--copy-calib", action="store_true",
@@ -204,6 +207,48 @@ def main():
     log(f"[bench] timed: {avg_kernel_ms:.2f} ms/launch, {achieved:.0f} GB/s algorithmic; every dense row read: {full_avg:.2f} ms, "
         f"{full_eval['achieved']:.0f} GB/s")
 
+    extras = None
+    if args.extras:
+        extras = {}
+        ec = 128
+        for wx in ((1.0, 0.0, 0.0), (0.0, 1.0, 0.0), (0.0, 0.0, 1.0), (1.0, 1.0, 1.0), (1.0, 0.5, 2.0)):
+            tx, _ = ground_truth(torch, corpus, queries, wx, 10, nq_truth)
+            apoe.search(ctx, gc, gq, graph, wx, ec, out_ids=None)
+            ids_x, _, sx = apoe.search(ctx, gc, gq, graph, wx, ec)
+            extras[f"weights {wx}"] = dict(kernel_ms=sx.kernel_ms, qps=args.queries / (sx.kernel_ms / 1e3), recall_at_10=recall_at_k(ids_x[:nq_truth], tx, 10),
+                                           algo_gbs=sx.algo_bytes / (sx.kernel_ms / 1e3) / 1e9)
+            log(f"[bench] extras: weights {wx} cands {ec}: {sx.kernel_ms:.2f} ms, recall {extras[f'weights {wx}']['recall_at_10']:.4f}")
+        kg = S.knowledge_graph(200_000, args.docs, args.queries, device=dev)
+        gkg = apoe.KnowledgeGraph(ctx, *kg)
+        apoe.search(ctx, gc, gq, graph, w3, ec, kg=gkg, kg_weight=40.0)
+        _, _, sk = apoe.search(ctx, gc, gq, graph, w3, ec, kg=gkg, kg_weight=40.0)
+        extras["knowledge graph, kg_weight 40"] = dict(kernel_ms=sk.kernel_ms, qps=args.queries / (sk.kernel_ms / 1e3), evaluations=int(sk.evaluations),
+                                                       algo_gbs=sk.algo_bytes / (sk.kernel_ms / 1e3) / 1e9)
+        log(f"[bench] extras: KG search cands {ec}: {sk.kernel_ms:.2f} ms")
+        # keyword filter: flag the rarest BM25 term of each query (by document frequency)
+        qb_off, qb_idx = queries[4].long(), queries[5].long()
+        df = torch.bincount(corpus[5].long(), minlength=S.VOCAB)
+        cnt = qb_off[1:] - qb_off[:-1]
+        rows = torch.repeat_interleave(torch.arange(args.queries, device=dev), cnt)
+        f = df[qb_idx].float()
+        f[f == 0] = float("inf")
+        best = torch.full((args.queries,), float("inf"), device=dev).scatter_reduce(0, rows, f, "amin")
+        pos = torch.arange(qb_idx.numel(), device=dev)
+        first = torch.full((args.queries,), qb_idx.numel(), device=dev, dtype=torch.long).scatter_reduce(
+            0, rows, torch.where(f == best[rows], pos, torch.full_like(pos, qb_idx.numel())), "amin")
+        flagged = qb_idx.clone()
+        okq = first < qb_idx.numel()
+        flagged[first[okq]] |= 0x80000000
+        flagged32 = (flagged & 0xFFFFFFFF).to(torch.int64)
+        flagged32 = torch.where(flagged32 >= 2 ** 31, flagged32 - 2 ** 32, flagged32).to(torch.int32)
+        gqk = apoe.Queries(ctx, *(tuple(queries[:5]) + (flagged32,) + tuple(queries[6:])))
+        apoe.search(ctx, gc, gqk, graph, w3, ec, keyword_filter=True)
+        ids_k, _, sw = apoe.search(ctx, gc, gqk, graph, w3, ec, keyword_filter=True)
+        extras["keyword filter, rarest BM25 term"] = dict(kernel_ms=sw.kernel_ms, qps=args.queries / (sw.kernel_ms / 1e3), evaluations=int(sw.evaluations),
+                                                          mean_hits_per_row=float((ids_k != 0x7FFFFFFF).sum(1).mean()),
+                                                          algo_gbs=sw.algo_bytes / (sw.kernel_ms / 1e3) / 1e9)
+        log(f"[bench] extras: keyword-filter search cands {ec}: {sw.kernel_ms:.2f} ms, {extras['keyword filter, rarest BM25 term']['mean_hits_per_row']:.1f} hits per row")
+
     if args.copy_calib:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
@@ -262,6 +307,7 @@ def main():
             "nnd_algo_gbs": nnd_bytes / (nnd_ms / 1e3) / 1e9,
             "cands_sweep": sweep,
             "kernel_ms": avg_kernel_ms,
+            **({"extras": extras} if extras else {}),
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC.get((args.docs, args.degree, args.queries, cands, args.variant)) if not args.calibrate else None,
