@@ -388,9 +388,14 @@ __device__ __forceinline__ void eval_issue_desc(PendingEval& p, const CorpusView
     const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
     const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
     p.kv0 = p.kv1 = p.kv2 = make_uint2(0, 0);
-    if (j0 < p.end) p.kv0 = sp[j0];
-    if (j1 < p.end) p.kv1 = sp[j1];
-    if (j2 < p.end) p.kv2 = sp[j2];
+    // no per-lane branches: a lane past the end of the row loads the row's last pair again and the
+    // consumer masks it (it tests j < end anyway)
+    if (p.begin < p.end) {
+        const uint32_t last = p.end - 1;
+        p.kv0 = sp[min(j0, last)];
+        p.kv1 = sp[min(j1, last)];
+        p.kv2 = sp[min(j2, last)];
+    }
 }
 
 __device__ __forceinline__ void eval_issue(PendingEval& p, const CorpusView& C, uint32_t id, float pv_norm, uint32_t paths, float dense_mul) {

@@ -13,25 +13,34 @@ constexpr int RING = 32;      // keyword-filter search: evicted keyword hits kep
 // What the kernel does on top of the plain beam search.
 enum SearchMode { MODE_PLAIN = 0, MODE_KG = 1, MODE_KEYWORD = 2 };
 
-struct SearchArgs {
-    CorpusView C;
+// Arguments that a query needs once (when it starts or ends) stay in device memory and are read
+// where they are used; the rest travels by value. Scalar registers are the scarce resource of this
+// kernel: every argument held in one for the whole launch pushes loop state into vector registers.
+struct SearchCold {
     SetView Q;
-    const uint32_t* graph;
-    uint32_t W, degree;
     const uint32_t* entry;
     uint32_t n_entry;
     float w_d, w_s, w_b;
-    uint32_t paths;
-    uint32_t cands, max_iter, q_begin, q_count;
+    uint32_t q_begin;
     uint32_t* out_ids;
     float* out_dist;
+    const uint32_t *q2e_off, *q2e_idx;
+};
+
+struct SearchArgs {
+    CorpusView C;
+    const SearchCold* cold;
+    const uint32_t* graph;
+    uint32_t W, degree;
+    uint32_t paths;
+    uint32_t cands, max_iter, q_count;
     uint32_t* bitmaps;     // one visited bitmap per workgroup
     uint32_t bitmap_words; // multiple of 4
     unsigned long long* work; // [0] next query, [1] expansions, [2] evaluations, [3] nnz splade, [4] nnz bm25, [5] dense rows read
     uint32_t full_eval;       // 1: read the dense row of every candidate (no bound test)
     uint32_t slots;
     // knowledge graph (KG kernels only)
-    const uint32_t *e2e_off, *e2e_idx, *e2d_off, *e2d_idx, *q2e_off, *q2e_idx;
+    const uint32_t *e2e_off, *e2e_idx, *e2d_off, *e2d_idx;
     uint32_t n_entities;
     float kg_weight;
     uint32_t kw_slots; // keyword-filter kernels only: slots of the per-query keyword term set
@@ -170,7 +179,7 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
         R.n += cnt;
         wave_fence();
     }
-    const uint32_t lo0 = P.lb[0];
+    const uint32_t lo0 = uniform(P.lb[0]);
     for (int base = (int)((cands - 1) & ~(uint32_t)(WAVE - 1)); base >= 0 && (uint32_t)base + WAVE > lo0; base -= WAVE) {
         const uint32_t p = base + lane;
         const bool act = p >= lo0 && p < cands;
@@ -241,9 +250,9 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
         __syncthreads();
         if (tid == 0) ctl[CTL_QUERY] = (uint32_t)atomicAdd(a.work, 1ull);
         __syncthreads();
-        const uint32_t qi = ctl[CTL_QUERY];
+        const uint32_t qi = uniform(ctl[CTL_QUERY]);
         if (qi >= a.q_count) break;
-        const uint32_t q = a.q_begin + qi;
+        const uint32_t q = a.cold->q_begin + qi;
 
         // ---- reset per-query state ----
         {
@@ -261,19 +270,19 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             if (KG) { P.ent[i] = EMPTY; P.hop[i] = 0; }
         }
         {
-            const float4* src = reinterpret_cast<const float4*>(a.Q.dense + (size_t)q * DIM);
+            const float4* src = reinterpret_cast<const float4*>(a.cold->Q.dense + (size_t)q * DIM);
             for (uint32_t i = tid; i < DIM / 4; i += NW * WAVE) {
                 const float4 x = src[i];
-                qd[i] = make_float4(x.x * a.w_d, x.y * a.w_d, x.z * a.w_d, x.w * a.w_d);
+                qd[i] = make_float4(x.x * a.cold->w_d, x.y * a.cold->w_d, x.z * a.cold->w_d, x.w * a.cold->w_d);
             }
         }
         __threadfence();
         __syncthreads();
-        bucket_terms_from_query(T, a.Q, q, a.w_s, a.w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
+        bucket_terms_from_query(T, a.cold->Q, q, a.cold->w_s, a.cold->w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
         if (KWD) {
             // required keywords: BM25 query terms whose id arrives with bit 31 set (query.cu:1828-1843)
-            for (uint32_t j = a.Q.b_off[q] + tid; j < a.Q.b_off[q + 1]; j += NW * WAVE) {
-                const uint32_t t = a.Q.b_idx[j];
+            for (uint32_t j = a.cold->Q.b_off[q] + tid; j < a.cold->Q.b_off[q + 1]; j += NW * WAVE) {
+                const uint32_t t = a.cold->Q.b_idx[j];
                 if (t & BM25_BIT) id_set_insert(kwset, a.kw_slots - 1, t);
             }
         }
@@ -287,7 +296,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
         if (!KG) {
             // entry points (query.cu:440-485)
             if (wave == 0) {
-                uint32_t c = lane < (int)a.n_entry ? a.entry[lane] : EMPTY;
+                uint32_t c = lane < (int)a.cold->n_entry ? a.cold->entry[lane] : EMPTY;
                 bool fresh = false;
                 if (c < a.C.n) {
                     const uint32_t bit = 1u << (c & 31);
@@ -304,9 +313,9 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             if (wave == 0) {
                 const uint32_t seed_cap = cands + a.degree;
                 uint32_t n_seed = 0;
-                const uint32_t qe0 = uniform(a.q2e_off[q]), qe1 = uniform(a.q2e_off[q + 1]);
+                const uint32_t qe0 = uniform(a.cold->q2e_off[q]), qe1 = uniform(a.cold->q2e_off[q + 1]);
                 for (uint32_t i = qe0; i < qe1; i++) {
-                    const uint32_t e = uniform(a.q2e_idx[i]);
+                    const uint32_t e = uniform(a.cold->q2e_idx[i]);
                     if (e >= a.n_entities) continue;
                     const uint32_t d0 = uniform(a.e2d_off[e]), d1 = uniform(a.e2d_off[e + 1]);
                     for (uint32_t b0 = d0; b0 < d1; b0 += WAVE) {
@@ -323,7 +332,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                     }
                 }
                 if (n_seed < cands) {
-                    const uint32_t c = lane < (int)a.n_entry ? a.entry[lane] : EMPTY;
+                    const uint32_t c = lane < (int)a.cold->n_entry ? a.cold->entry[lane] : EMPTY;
                     bool fresh = false;
                     if (c < a.C.n) {
                         const uint32_t bit = 1u << (c & 31);
@@ -337,7 +346,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                 if (lane == 0) ctl[CTL_NSEED] = n_seed;
             }
             __syncthreads();
-            const uint32_t n_seed = ctl[CTL_NSEED];
+            const uint32_t n_seed = uniform(ctl[CTL_NSEED]);
             const uint32_t n_ovf_seed = uniform(ctl[CTL_NOVF]);
             for (uint32_t j = wave; j < n_seed; j += NW) {
                 const uint32_t id = uniform(seed_id[j]);
@@ -379,8 +388,8 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
 
         for (uint32_t it = 0; it <= a.max_iter; it++) {
             // ---- evaluate the fresh candidates: one wave per candidate ----
-            const uint32_t n_new = ctl[CTL_NNEW];
-            if (ctl[CTL_PARENT] == EMPTY) break;
+            const uint32_t n_new = uniform(ctl[CTL_NNEW]);
+            if (uniform(ctl[CTL_PARENT]) == EMPTY) break;
             // a candidate that provably cannot enter the (full) pool is dropped after its sparse part:
             // it is reported as INF_DIS and falls off the end of the merge like any other loser
             const float thr = a.full_eval ? __builtin_inff() : P.dist[cands - 1];
@@ -598,14 +607,14 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
         // ---- results (query.cu:566-569) ----
         if (!KWD) {
             for (uint32_t i = tid; i < cands; i += NW * WAVE) {
-                a.out_ids[(size_t)qi * cands + i] = P.id[i] & ~FLAG;
-                a.out_dist[(size_t)qi * cands + i] = P.dist[i];
+                a.cold->out_ids[(size_t)qi * cands + i] = P.id[i] & ~FLAG;
+                a.cold->out_dist[(size_t)qi * cands + i] = P.dist[i];
             }
         } else if (wave == 0) {
             // pool entries that hold a required keyword, in pool order, then the evicted hits by
             // (distance, id); the rest of the row is empty (query.cu:1464-1481)
-            uint32_t* oid = a.out_ids + (size_t)qi * cands;
-            float* od = a.out_dist + (size_t)qi * cands;
+            uint32_t* oid = a.cold->out_ids + (size_t)qi * cands;
+            float* od = a.cold->out_dist + (size_t)qi * cands;
             uint32_t kn = 0;
             for (uint32_t base = 0; base < cands; base += WAVE) {
                 const uint32_t id = base + lane < cands ? P.id[base + lane] : EMPTY;
@@ -685,23 +694,24 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     if (q_count == 0) return APOE_OK;
 
     SearchArgs a{};
+    SearchCold cold{};
     a.C = c->view();
-    a.Q = q->view();
+    cold.Q = q->view();
     a.graph = g->rows.p;
     a.W = g->width;
     a.degree = g->width - APOE_KW_SLOTS;
-    a.entry = g->entry.p;
-    a.n_entry = std::min<uint32_t>(g->n_entry, MAX_NEW);
-    a.w_d = p->w_dense;
-    a.w_s = p->w_sparse;
-    a.w_b = p->w_bm25;
+    cold.entry = g->entry.p;
+    cold.n_entry = std::min<uint32_t>(g->n_entry, MAX_NEW);
+    cold.w_d = p->w_dense;
+    cold.w_s = p->w_sparse;
+    cold.w_b = p->w_bm25;
     a.paths = (!(p->w_dense < 1e-5f) ? PATH_DENSE : 0) | (!(p->w_sparse < 1e-5f) ? PATH_SPARSE : 0) | (!(p->w_bm25 < 1e-5f) ? PATH_BM25 : 0);
     a.cands = p->cands;
     a.max_iter = p->max_iter ? p->max_iter : 1000;
-    a.q_begin = p->q_begin;
+    cold.q_begin = p->q_begin;
     a.q_count = q_count;
-    a.out_ids = out_ids_dev;
-    a.out_dist = out_dist_dev;
+    cold.out_ids = out_ids_dev;
+    cold.out_dist = out_dist_dev;
     a.slots = next_pow2(std::max(64u, 2 * q->max_nnz));
     a.kg_weight = p->kg_weight;
     a.full_eval = (p->variant & 0x100u) ? 1u : 0u;
@@ -721,8 +731,8 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
         a.e2e_idx = kg->e2e_idx.p;
         a.e2d_off = kg->e2d_off.p;
         a.e2d_idx = kg->e2d_idx.p;
-        a.q2e_off = kg->q2e_off.p;
-        a.q2e_idx = kg->q2e_idx.p;
+        cold.q2e_off = kg->q2e_off.p;
+        cold.q2e_idx = kg->q2e_idx.p;
         a.n_entities = kg->n_entities;
     }
     const SearchLds L(a.slots, a.cands, mode, a.kw_slots);
@@ -743,8 +753,12 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;
     DevBuf<uint32_t> bitmaps;
     DevBuf<unsigned long long> work;
+    DevBuf<SearchCold> cold_dev;
     APOE_TRY(bitmaps.alloc((size_t)grid * a.bitmap_words));
     APOE_TRY(work.alloc(8));
+    APOE_TRY(cold_dev.alloc(1));
+    APOE_HIP(hipMemcpy(cold_dev.p, &cold, sizeof(cold), hipMemcpyHostToDevice));
+    a.cold = cold_dev.p;
     APOE_HIP(hipMemsetAsync(work.p, 0, 8 * sizeof(unsigned long long), ctx->stream));
     a.bitmaps = bitmaps.p;
     a.work = work.p;
