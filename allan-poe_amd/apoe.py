@@ -6,6 +6,7 @@ call fails, an exception is raised.
 """
 import ctypes as C
 import os
+import sys
 
 import numpy as np
 
@@ -50,6 +51,14 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise ApoeError(f"{LIB_PATH} is not built; run `make -C {os.path.join(_HERE, 'csrc')}`")
+        # PyTorch wheels bring their own copy of the HIP runtime. A process that loads this library
+        # first and PyTorch second ends up with two runtimes, and the second one finds no device:
+        # let PyTorch (if it is installed) load its copy first, libapoe.so then binds to the same one.
+        if "torch" not in sys.modules:
+            try:
+                import torch  # noqa: F401
+            except ImportError:
+                pass
         _lib = C.CDLL(LIB_PATH)
         _lib.apoe_last_error_string.restype = C.c_char_p
         _lib.apoe_corpus_bytes.restype = C.c_uint64

@@ -1,0 +1,114 @@
+"""The whole path at 100 000 docs (degree 32, K = 64, 10 NN-Descent steps, cands 128): the oracle checks a
+sample, the rest is checked through properties that do not depend on the size."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))  # bench.py's torch ground truth
+
+from parity import assert_dist_close, assert_topk_match, recall_at_k
+
+pytestmark = pytest.mark.gpu
+
+N_DOCS, N_QUERIES, DEGREE, CANDS = 100_000, 2_000, 32, 128
+EMPTY_ID = 0x7FFFFFFF
+
+
+@pytest.fixture(scope="module")
+def world(gpu_ctx):
+    import torch
+    import apoe
+    import apoe_synth as S
+    corpus = S.corpus(N_DOCS, seed=101, device="cuda:0")
+    queries = S.queries(N_QUERIES, seed=102, device="cuda:0")
+    torch.cuda.synchronize()
+    gc = apoe.Corpus(gpu_ctx, *corpus)
+    gq = apoe.Queries(gpu_ctx, *queries)
+    graph, ms = apoe.build_graph(gpu_ctx, gc, K=64, iters=10, degree=DEGREE, seed=3)
+    rows, entry = graph.download()
+    yield dict(ctx=gpu_ctx, corpus=corpus, queries=queries, gc=gc, gq=gq, graph=graph, rows=rows, entry=entry, build_ms=ms)
+    graph.close()
+    gq.close()
+    gc.close()
+
+
+def test_graph_rows_are_well_formed(world):
+    rows, entry = world["rows"], world["entry"]
+    assert rows.shape == (N_DOCS, DEGREE + 8) and len(entry) == DEGREE
+    nb = rows[:, :DEGREE]
+    assert nb.max() < N_DOCS
+    assert not (nb == np.arange(N_DOCS, dtype=np.uint32)[:, None]).all(axis=1).any()
+    # the forward half of a row holds distinct documents
+    half = np.sort(nb[:, :DEGREE // 2], axis=1)
+    assert (np.diff(half.astype(np.int64), axis=1) != 0).mean() > 0.999
+    cnt = rows[:, DEGREE]
+    assert cnt.max() <= 7
+    kw = rows[:, DEGREE + 1:]
+    assert np.all(kw[np.arange(7)[None, :] >= cnt[:, None]] == 0)
+    assert kw.max() < N_DOCS
+    assert len(set(entry.tolist())) == DEGREE
+
+
+def test_search_rows_sorted_unique_and_distances_are_the_metric(world):
+    import apoe
+    w = world
+    ids, dist, st = apoe.search(w["ctx"], w["gc"], w["gq"], w["graph"], (1, 1, 1), CANDS)
+    assert np.all(np.diff(dist, axis=1) >= 0)
+    real = ids != EMPTY_ID
+    assert real[:, :10].all()
+    for q in range(0, N_QUERIES, 97):
+        r = ids[q][real[q]]
+        assert len(set(r.tolist())) == len(r)
+    # every reported distance is the fused metric of that pair (an independent kernel computes it)
+    safe = np.where(real, ids, 0).astype(np.uint32)
+    again = apoe.distance_batch(w["ctx"], w["gc"], w["gq"], (1, 1, 1), safe)
+    assert_dist_close(dist[real], again[real], "search distances vs distance_batch")
+    # the bound never changes a result: reading every dense row gives the same rows
+    ids2, dist2, st2 = apoe.search(w["ctx"], w["gc"], w["gq"], w["graph"], (1, 1, 1), CANDS, variant=0x100)
+    assert np.array_equal(ids, ids2) and np.array_equal(dist, dist2)
+    assert st.evaluations == st2.evaluations and st.dense_rows < st2.dense_rows == st2.evaluations
+    # launch shapes agree
+    ids3, dist3, _ = apoe.search(w["ctx"], w["gc"], w["gq"], w["graph"], (1, 1, 1), CANDS, variant=2)
+    assert assert_topk_match(ids, dist, ids3, dist3, 10, "launch shapes") > 0.99
+
+
+def test_sample_matches_oracle_on_the_gpu_built_graph(world):
+    import apoe_synth as S
+    import oracle as O
+    import apoe
+    w = world
+    C = O.HybridSet(*S.to_numpy(w["corpus"]))
+    nq = 200
+    Q = O.HybridSet(*S.to_numpy(w["queries"])).head(nq)
+    for w3 in ((1.0, 1.0, 1.0), (1.0, 0.5, 2.0)):
+        ids, dist, _ = apoe.search(w["ctx"], w["gc"], w["gq"], w["graph"], w3, CANDS, q_count=nq)
+        oid, odist, _ = O.search(C, Q, w["rows"], w["entry"], w3, CANDS)
+        assert assert_topk_match(ids, dist, oid, odist, 10, f"100k docs, weights {w3}") > 0.97
+        same = ids == oid
+        assert same.mean() > 0.95
+        assert_dist_close(dist[same], odist[same], "pool distances")
+    # entry points and norms as the oracle derives them from the same corpus
+    assert np.array_equal(w["entry"], O.entry_points(O.norms(C, 7.0), DEGREE))
+
+
+def test_recall_grows_with_the_pool_and_beats_a_random_graph(world):
+    import torch
+    import apoe
+    from bench import ground_truth
+    w = world
+    nq = 500
+    truth, _ = ground_truth(torch, w["corpus"], w["queries"], (1.0, 1.0, 1.0), 10, nq)
+    rec = []
+    for cands in (32, 128, 512):
+        ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], w["graph"], (1, 1, 1), cands, q_count=nq)
+        rec.append(recall_at_k(ids, truth, 10))
+    assert rec == sorted(rec) and rec[-1] > rec[0] + 0.05, rec
+    rng = np.random.default_rng(0)
+    rnd_rows = w["rows"].copy()
+    rnd_rows[:, :DEGREE] = rng.integers(0, N_DOCS, (N_DOCS, DEGREE))
+    g2 = apoe.Graph(w["ctx"], rnd_rows, w["entry"])
+    ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], g2, (1, 1, 1), 128, q_count=nq)
+    assert recall_at_k(ids, truth, 10) < rec[1]
+    g2.close()
