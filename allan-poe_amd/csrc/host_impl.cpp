@@ -161,6 +161,32 @@ void load_graph(const std::string& path, std::vector<unsigned>& rows, std::vecto
     }
 }
 
+// K-NN graph between NN-Descent and the prune: "APKN", n, K, ids [n][K], distances [n][K].
+void write_knn(const std::string& path, unsigned n, unsigned K, const std::vector<unsigned>& ids, const std::vector<float>& dist) {
+    std::ofstream out(path, std::ios::binary | std::ios::out);
+    if (!out.is_open()) fail("cannot write " + path);
+    const unsigned head[3] = {0x4E4B5041u, n, K}; // "APKN"
+    out.write(reinterpret_cast<const char*>(head), sizeof(head));
+    out.write(reinterpret_cast<const char*>(ids.data()), (std::streamsize)ids.size() * 4);
+    out.write(reinterpret_cast<const char*>(dist.data()), (std::streamsize)dist.size() * 4);
+    if (!out.good()) fail("write error on " + path);
+}
+
+void load_knn(const std::string& path, unsigned n, unsigned K, std::vector<unsigned>& ids, std::vector<float>& dist) {
+    std::ifstream in(path, std::ios::binary);
+    if (!in.is_open()) fail("open file error: " + path);
+    unsigned head[3] = {0, 0, 0};
+    read_exact(in, head, 3, path);
+    if (head[0] != 0x4E4B5041u) fail(path + " is not a K-NN graph file");
+    if (head[1] != n || head[2] != K) fail("K-NN graph in " + path + " is for " + std::to_string(head[1]) + " points, K = " + std::to_string(head[2]));
+    ids.resize((size_t)n * K);
+    dist.resize((size_t)n * K);
+    read_exact(in, ids.data(), ids.size(), path);
+    read_exact(in, dist.data(), dist.size(), path);
+    for (unsigned v : ids)
+        if (v >= n && v != 0xFFFFFFFFu) fail("K-NN graph in " + path + " names a point beyond the corpus");
+}
+
 // query.cu:111-145: IDCG over all ground-truth ids, DCG by position in the result
 double ndcg_at_k(const std::vector<std::vector<unsigned>>& res, std::vector<std::vector<unsigned>> gt, double* recall) {
     float all = 0.f, ndcg = 0.f;
@@ -208,9 +234,22 @@ void build_index_impl(const std::string& dense_data_path, const std::string& spa
           "apoe_corpus_create");
     // index.cu:889-903; the x7 dense scale of index.cu:836-840 is applied inside the metric
     check(apoe_knn_create(h.ctx, h.corpus, opt.nnd_k, opt.dense_build_scale, &h.knn), "apoe_knn_create");
-    check(apoe_nnd_init(h.knn, opt.seed), "apoe_nnd_init");
-    for (unsigned it = 0; it < opt.nnd_iters; it++) check(apoe_nnd_iterate(h.knn, it + 1 == opt.nnd_iters, nullptr), "apoe_nnd_iterate");
-    check(apoe_nnd_merge_reverse(h.knn), "apoe_nnd_merge_reverse");
+    if (!opt.knn_load_path.empty()) {
+        std::vector<unsigned> ids;
+        std::vector<float> dist;
+        load_knn(opt.knn_load_path, points_num, opt.nnd_k, ids, dist);
+        check(apoe_knn_upload(h.knn, ids.data(), dist.data()), "apoe_knn_upload");
+    } else {
+        check(apoe_nnd_init(h.knn, opt.seed), "apoe_nnd_init");
+        for (unsigned it = 0; it < opt.nnd_iters; it++) check(apoe_nnd_iterate(h.knn, it + 1 == opt.nnd_iters, nullptr), "apoe_nnd_iterate");
+        check(apoe_nnd_merge_reverse(h.knn), "apoe_nnd_merge_reverse");
+    }
+    if (!opt.knn_save_path.empty()) {
+        std::vector<unsigned> ids((size_t)points_num * opt.nnd_k);
+        std::vector<float> dist((size_t)points_num * opt.nnd_k);
+        check(apoe_knn_download(h.knn, ids.data(), dist.data()), "apoe_knn_download");
+        write_knn(opt.knn_save_path, points_num, opt.nnd_k, ids, dist);
+    }
     check(apoe_prune(h.knn, opt.degree), "apoe_prune");
     check(apoe_finalize_graph(h.knn, &h.graph), "apoe_finalize_graph");
     std::cout << "Indexing time: " << apoe_knn_elapsed_ms(h.knn) / 1000.0f << "s" << std::endl;

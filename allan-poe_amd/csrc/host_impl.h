@@ -20,6 +20,12 @@ struct BuildOptions {
     float dense_build_scale = 7.0f; // index.cu:836-840
     uint64_t seed = 20251125;       // the reference seeds from clock(), index.cu:102
     int device = 0;
+    // Intermediate artefact, no counterpart in the reference: the K-NN graph between NN-Descent
+    // (after the reverse merge) and the prune. Saving it allows a re-prune to another degree
+    // without repeating NN-Descent; loading it skips NN-Descent.
+    // File: "APKN", n, K (u32 each), then ids [n][K] u32, then distances [n][K] f32.
+    std::string knn_save_path;
+    std::string knn_load_path;
 };
 
 struct SearchOptions {
@@ -44,6 +50,8 @@ void load_kg(const std::string& path, std::vector<unsigned>& off, std::vector<un
 void load_txt(const std::string& path, std::vector<std::vector<unsigned>>& results, unsigned query_num);
 void write_graph(const std::string& path, const std::vector<unsigned>& rows, unsigned n, unsigned width, const std::vector<unsigned>& entry);
 void load_graph(const std::string& path, std::vector<unsigned>& rows, std::vector<unsigned>& entry, unsigned& width, unsigned& num);
+void write_knn(const std::string& path, unsigned n, unsigned K, const std::vector<unsigned>& ids, const std::vector<float>& dist);
+void load_knn(const std::string& path, unsigned n, unsigned K, std::vector<unsigned>& ids, std::vector<float>& dist);
 double ndcg_at_k(const std::vector<std::vector<unsigned>>& res, std::vector<std::vector<unsigned>> gt, double* recall);
 
 void build_index_impl(const std::string& dense_data_path, const std::string& sparse_data_path, const std::string& bm25_data_path,

@@ -125,6 +125,40 @@ def test_keyword_file_search(files, capfd):
     assert (oid != 0x7FFFFFFF).any()
 
 
+def test_knn_graph_save_and_reprune(files, capfd):
+    """The K-NN graph saved between NN-Descent and the prune rebuilds the same index without NN-Descent,
+    and re-prunes to another degree."""
+    import hybrid_search
+    import oracle as O
+    p = files["paths"]
+    d = os.path.dirname(p["index.poe"])
+    knn_path, a_path, b_path, c_path = (os.path.join(d, x) for x in ("graph.knn", "a.poe", "b.poe", "c.poe"))
+    common = dict(dense_data_path=p["dense.fvecs"], sparse_data_path=p["sparse.bin"], bm25_data_path=p["bm25.bin"])
+    hybrid_search.build_index(output_graph_path=a_path, nnd_iters=6, knn_save_path=knn_path, **common)
+    n = files["n"]
+    assert os.path.getsize(knn_path) == 12 + n * 64 * 8
+    head = np.fromfile(knn_path, np.uint32, 3)
+    assert head.tolist() == [0x4E4B5041, n, 64]
+    ids = np.fromfile(knn_path, np.uint32, n * 64, offset=12).reshape(n, 64)
+    dist = np.fromfile(knn_path, np.float32, n * 64, offset=12 + n * 64 * 4).reshape(n, 64)
+    assert ids.max() < n and np.all(np.diff(dist, axis=1) >= 0)
+    hybrid_search.build_index(output_graph_path=b_path, nnd_iters=0, knn_load_path=knn_path, **common)
+    ra, ea = O.read_poe(a_path)
+    rb, eb = O.read_poe(b_path)
+    assert np.array_equal(ra, rb) and np.array_equal(ea, eb)
+    hybrid_search.build_index(output_graph_path=c_path, degree=16, knn_load_path=knn_path, **common)
+    rc, ec = O.read_poe(c_path)
+    assert rc.shape == (n, 24) and len(ec) == 16
+    # the oracle prunes the saved graph to the same rows
+    C = files["C"]
+    fwd, det, cnt, kw = O.prune(C, 7.0, O.norms(C, 7.0), ids, dist, 16)
+    want = O.final_graph(fwd, det, cnt, kw)
+    assert (rc == want).all(axis=1).mean() > 0.995
+    capfd.readouterr()
+    with pytest.raises(RuntimeError, match="K-NN graph"):
+        hybrid_search.build_index(output_graph_path=c_path, nnd_k=128, knn_load_path=knn_path, **common)
+
+
 def test_errors_raise(files):
     import hybrid_search
     p = files["paths"]
