@@ -218,6 +218,16 @@ def main():
             extras[f"weights {wx}"] = dict(kernel_ms=sx.kernel_ms, qps=args.queries / (sx.kernel_ms / 1e3), recall_at_10=recall_at_k(ids_x[:nq_truth], tx, 10),
                                            algo_gbs=sx.algo_bytes / (sx.kernel_ms / 1e3) / 1e9)
             log(f"[bench] extras: weights {wx} cands {ec}: {sx.kernel_ms:.2f} ms, recall {extras[f'weights {wx}']['recall_at_10']:.4f}")
+        # the host boundary: the same corpus handed over as host (pageable) buffers, H2D included
+        host = S.to_numpy(corpus)
+        th = time.perf_counter()
+        gch = apoe.Corpus(ctx, *host)
+        ctx.synchronize()
+        h2d_s = time.perf_counter() - th
+        gch.close()
+        del host
+        extras["corpus handed over as host buffers"] = dict(seconds=h2d_s, gb=gc.bytes() / 1e9, gbs=gc.bytes() / 1e9 / h2d_s)
+        log(f"[bench] extras: corpus from host buffers: {h2d_s:.2f}s for {gc.bytes() / 1e9:.2f} GB")
         kg = S.knowledge_graph(200_000, args.docs, args.queries, device=dev)
         gkg = apoe.KnowledgeGraph(ctx, *kg)
         apoe.search(ctx, gc, gq, graph, w3, ec, kg=gkg, kg_weight=40.0)
