@@ -223,6 +223,222 @@ __device__ __forceinline__ void gram_sparse_64(const CorpusView& C, const uint32
     __syncthreads();
 }
 
+// ---- sparse part, union-table form ----
+// The terms of GU_T pivot rows go into ONE table: a term's slot holds GU_T values, one per pivot
+// (zero where the pivot lacks the term). A pair of a later row is then looked up once per group
+// instead of once per pivot, and most lookups end at the key compare because most terms of a row
+// are in none of the pivots. Keys sit in buckets of 8 (two ds_read_b128), values in float4 slots
+// (one ds_read_b128, read with the hit masked into the multiplier, so there is no branch); a term
+// whose bucket is full goes to a short overflow list. When the pivots of a group hold more distinct
+// terms than the table takes, the group is retried with half as many pivots; one row always fits
+// (the host sizes the table for the longest row), else *fail is raised and G must be discarded.
+constexpr int GU_T = 4;      // pivots per union table
+constexpr int GU_BUCKET = 8; // keys per bucket
+constexpr int GU_OVF = 32;   // overflow terms per group
+
+struct GramUnionLds { // byte offsets inside the table region
+    uint32_t keys, vals, ovf_key, ovf_val, total;
+    __host__ __device__ explicit GramUnionLds(uint32_t slots) {
+        uint32_t o = 0;
+        keys = o; o += slots * 4;
+        vals = o; o += slots * GU_T * 4;
+        ovf_key = o; o += GU_OVF * 4;
+        ovf_val = o; o += GU_OVF * GU_T * 4;
+        total = o;
+    }
+};
+
+__device__ __forceinline__ uint32_t gu_hash(uint32_t key, uint32_t bucket_mask) {
+    const uint32_t k = key ^ (key >> 15); // the BM25 bit must reach the multiplied bits
+    return ((k * 0x9E3779B1u) >> 14) & bucket_mask;
+}
+
+// ctl2: two LDS words (overflow count, spare). slots: power of two, >= 2 x the longest row.
+__device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uint32_t* ids, uint32_t m, float* G, char* table, uint32_t slots,
+                                                  uint32_t* ctl2, unsigned long long* rowptr, uint32_t* rownnz, uint32_t* fail, int tid,
+                                                  int nthreads) {
+    const GramUnionLds L(slots);
+    uint32_t* keys = reinterpret_cast<uint32_t*>(table + L.keys);
+    float* vals = reinterpret_cast<float*>(table + L.vals);
+    uint32_t* ovf_key = reinterpret_cast<uint32_t*>(table + L.ovf_key);
+    float* ovf_val = reinterpret_cast<float*>(table + L.ovf_val);
+    const uint4* keys4 = reinterpret_cast<const uint4*>(keys);
+    const float4* vals4 = reinterpret_cast<const float4*>(vals);
+    const float4* ovf_val4 = reinterpret_cast<const float4*>(ovf_val);
+    const uint32_t bmask = slots / GU_BUCKET - 1;
+    const int wave = (int)uniform(tid / WAVE), lane = tid & (WAVE - 1), nwaves = nthreads / WAVE;
+    for (uint32_t i = tid; i < m; i += nthreads) {
+        const uint64_t d = C.desc[ids[i]];
+        rowptr[i] = (unsigned long long)(C.recs + desc_off(d) * 16 + DENSE_BYTES);
+        rownnz[i] = desc_nnz_s(d) + desc_nnz_b(d);
+    }
+    __syncthreads();
+    uint32_t a0 = 0;
+    while (a0 + 1 < m) { // the last row is never a pivot
+        uint32_t nt = min((uint32_t)GU_T, m - 1 - a0);
+        while (true) {
+            for (uint32_t i = tid; i < slots; i += nthreads) keys[i] = EMPTY;
+            for (uint32_t i = tid; i < slots * GU_T / 4; i += nthreads) reinterpret_cast<float4*>(vals)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (uint32_t i = tid; i < GU_OVF; i += nthreads) ovf_key[i] = EMPTY;
+            for (uint32_t i = tid; i < GU_OVF * GU_T; i += nthreads) ovf_val[i] = 0.f;
+            if (tid == 0) ctl2[0] = 0;
+            __syncthreads();
+            // wave w scatters pivot (w % GU_T); waves w and w + GU_T share a pivot
+            const uint32_t t = (uint32_t)wave % GU_T;
+            if (t < nt) {
+                const uint2* sp = reinterpret_cast<const uint2*>(rowptr[a0 + t]);
+                const uint32_t nnz = rownnz[a0 + t];
+                const uint32_t step = (uint32_t)(nwaves / GU_T > 0 ? nwaves / GU_T : 1) * WAVE;
+                for (uint32_t j = (uint32_t)(wave / GU_T) * WAVE + lane; j < nnz; j += step) {
+                    const uint2 kv = sp[j];
+                    const uint32_t b0 = gu_hash(kv.x, bmask) * GU_BUCKET;
+                    uint32_t slot = EMPTY;
+                    for (uint32_t s = 0; s < GU_BUCKET; s++) {
+                        const uint32_t old = atomicCAS(&keys[b0 + s], EMPTY, kv.x);
+                        if (old == EMPTY || old == kv.x) { slot = b0 + s; break; }
+                    }
+                    if (slot != EMPTY) {
+                        vals[slot * GU_T + t] = __uint_as_float(kv.y);
+                    } else {
+                        uint32_t at = EMPTY;
+                        for (uint32_t s = 0; s < GU_OVF; s++) {
+                            const uint32_t old = atomicCAS(&ovf_key[s], EMPTY, kv.x);
+                            if (old == EMPTY) atomicAdd(&ctl2[0], 1u);
+                            if (old == EMPTY || old == kv.x) { at = s; break; }
+                        }
+                        if (at != EMPTY) ovf_val[at * GU_T + t] = __uint_as_float(kv.y);
+                        else atomicAdd(&ctl2[0], GU_OVF + 1u); // the list is full too
+                    }
+                }
+            }
+            __syncthreads();
+            const uint32_t filled = ctl2[0];
+            if (filled <= GU_OVF) break;
+            if (nt == 1) { // one row does not fit: the caller falls back
+                if (tid == 0) *fail = 1;
+                break;
+            }
+            nt = (nt + 1) / 2;
+            __syncthreads();
+        }
+        const uint32_t novf = uniform(min(ctl2[0], (uint32_t)GU_OVF));
+        uint32_t b = a0 + 1 + wave;
+        RowPairs cur;
+        if (b < m) row_pairs_load(cur, reinterpret_cast<const uint2*>(rowptr[b]), rownnz[b], lane);
+        while (b < m) {
+            const uint32_t bn = b + nwaves;
+            RowPairs nxt;
+            if (bn < m) row_pairs_load(nxt, reinterpret_cast<const uint2*>(rowptr[bn]), rownnz[bn], lane);
+            const uint32_t nnz = uniform(rownnz[b]);
+            const uint32_t np = min(nt, b - a0); // pivots a0 .. a0+np-1 precede row b
+            float acc[GU_T];
+#pragma unroll
+            for (int t = 0; t < GU_T; t++) acc[t] = 0.f;
+            // one pair against the union table: keys of its bucket, then the value slot of the key that matched
+            auto match = [&](const uint4 k0, const uint4 k1, uint32_t bucket, uint2 kv, uint32_t& slot) -> float {
+                const uint32_t off = k0.x == kv.x ? 0u : k0.y == kv.x ? 1u : k0.z == kv.x ? 2u : k0.w == kv.x ? 3u : k1.x == kv.x ? 4u
+                                     : k1.y == kv.x ? 5u : k1.z == kv.x ? 6u : k1.w == kv.x ? 7u : 8u;
+                slot = bucket * GU_BUCKET + (off & 7u);
+                return off < 8u ? __uint_as_float(kv.y) : 0.f; // a miss multiplies whatever the slot holds by zero
+            };
+            auto overflow = [&](uint2 kv) {
+                for (uint32_t o = 0; o < novf; o++) { // uniform, almost always zero trips
+                    if (ovf_key[o] == kv.x) {
+                        const float4 v = ovf_val4[o];
+                        const float val = __uint_as_float(kv.y);
+                        acc[0] = fmaf(val, v.x, acc[0]);
+                        acc[1] = fmaf(val, v.y, acc[1]);
+                        acc[2] = fmaf(val, v.z, acc[2]);
+                        acc[3] = fmaf(val, v.w, acc[3]);
+                    }
+                }
+            };
+            // the first three chunks (192 pairs) as one batch: six key reads, then three value reads
+            {
+                uint2 kv[3];
+                uint32_t bk[3], slot[3];
+                uint4 k0[3], k1[3];
+#pragma unroll
+                for (int c = 0; c < 3; c++) {
+                    kv[c] = cur.kv[c];
+                    if (kv[c].x == EMPTY) kv[c].y = 0u; // padding lane: matches an empty key at most, and adds 0 * value
+                    bk[c] = gu_hash(kv[c].x, bmask);
+                    k0[c] = keys4[bk[c] * 2];
+                    k1[c] = keys4[bk[c] * 2 + 1];
+                }
+                asm volatile("" : "+v"(k0[0].x), "+v"(k1[0].x), "+v"(k0[1].x), "+v"(k1[1].x), "+v"(k0[2].x), "+v"(k1[2].x));
+                float val[3];
+                float4 v[3];
+#pragma unroll
+                for (int c = 0; c < 3; c++) {
+                    val[c] = match(k0[c], k1[c], bk[c], kv[c], slot[c]);
+                    v[c] = vals4[slot[c]];
+                }
+                asm volatile("" : "+v"(v[0].x), "+v"(v[1].x), "+v"(v[2].x));
+#pragma unroll
+                for (int c = 0; c < 3; c++) {
+                    acc[0] = fmaf(val[c], v[c].x, acc[0]);
+                    acc[1] = fmaf(val[c], v[c].y, acc[1]);
+                    acc[2] = fmaf(val[c], v[c].z, acc[2]);
+                    acc[3] = fmaf(val[c], v[c].w, acc[3]);
+                }
+                if (novf) {
+#pragma unroll
+                    for (int c = 0; c < 3; c++) overflow(kv[c]);
+                }
+            }
+            auto lookup = [&](uint2 kv) {
+                if (kv.x == EMPTY) kv.y = 0u;
+                const uint32_t bk = gu_hash(kv.x, bmask);
+                uint32_t slot;
+                const float val = match(keys4[bk * 2], keys4[bk * 2 + 1], bk, kv, slot);
+                const float4 v = vals4[slot];
+                acc[0] = fmaf(val, v.x, acc[0]);
+                acc[1] = fmaf(val, v.y, acc[1]);
+                acc[2] = fmaf(val, v.z, acc[2]);
+                acc[3] = fmaf(val, v.w, acc[3]);
+                if (novf) overflow(kv);
+            };
+#pragma unroll
+            for (int c = 3; c < GRAM_CHUNKS; c++)
+                if (c * WAVE < (int)nnz) lookup(cur.kv[c]); // wave-uniform
+            if (nnz > GRAM_CHUNKS * WAVE) { // rows longer than the register window
+                const uint2* sp = reinterpret_cast<const uint2*>(rowptr[b]);
+                for (uint32_t j0 = GRAM_CHUNKS * WAVE; j0 < nnz; j0 += WAVE) {
+                    const uint32_t j = j0 + lane;
+                    lookup(j < nnz ? sp[j] : make_uint2(EMPTY, 0u));
+                }
+            }
+            // four sums over the wave at once: after two exchange-and-add steps inside each quad, lane l
+            // holds pivot t(l) = 2 * (l & 1) + ((l >> 1) & 1) summed over its quad; the rest is one sum per lane
+            {
+                const bool odd = lane & 1, hi = lane & 2;
+                const float keep0 = odd ? acc[2] : acc[0], keep1 = odd ? acc[3] : acc[1];
+                const float give0 = odd ? acc[0] : acc[2], give1 = odd ? acc[1] : acc[3];
+                const float x0 = keep0 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give0), 0xB1, 0xF, 0xF, false));
+                const float x1 = keep1 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give1), 0xB1, 0xF, 0xF, false));
+                const float keep = hi ? x1 : x0, give = hi ? x0 : x1;
+                float z = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give), 0x4E, 0xF, 0xF, false));
+                z += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, z), 0x124, 0xF, 0xF, false)); // row_ror:4
+                z += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, z), 0x128, 0xF, 0xF, false)); // row_ror:8
+                z += __shfl_xor(z, 16, WAVE);
+                z += __shfl_xor(z, 32, WAVE);
+                const uint32_t t = 2u * (lane & 1) + ((lane >> 1) & 1);
+                if (lane < GU_T && t < np) G[(a0 + t) * GRAM_STRIDE + b] += z;
+            }
+            cur = nxt;
+            b = bn;
+        }
+        __syncthreads();
+        a0 += nt;
+    }
+    for (uint32_t t = tid; t < m * m; t += nthreads) {
+        const uint32_t i = t / m, j = t % m;
+        if (i > j) G[i * GRAM_STRIDE + j] = G[j * GRAM_STRIDE + i];
+    }
+    __syncthreads();
+}
+
 #endif // __HIPCC__
 
 } // namespace apoe

@@ -7,6 +7,8 @@
 #include <memory>
 
 #include "apoe_gram.h"
+#include <cmath>
+
 #include "apoe_internal.h"
 
 namespace apoe {
@@ -239,15 +241,17 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
 // ---- gather-once form of the prune (K = 64) ----
 
 constexpr int GRAM_THREADS = 512; // 8 waves share one node's tables: more lookups in flight per byte of LDS
-constexpr int GRAM_T = 8; // upper bound on the pivot rows whose term tables are live at once
 
 struct GramPruneLds {
     uint32_t G, tabs, ovf_cnt, rowptr, rownnz, umap, R, idmap, nb_id, nb_dist, nrm, det, order, sel_gi, sel_live, sel_kw, o_fwd, o_det, o_kw, ctl, total;
-    __host__ __device__ GramPruneLds(uint32_t term_slots, uint32_t tgroup, uint32_t umap_slots, uint32_t map_slots, uint32_t words) {
+    // union_slots != 0: the table region holds one union table (apoe_gram.h) instead of tgroup pivot tables
+    __host__ __device__ GramPruneLds(uint32_t term_slots, uint32_t tgroup, uint32_t umap_slots, uint32_t map_slots, uint32_t words,
+                                     uint32_t union_slots) {
         uint32_t o = 0;
         G = o; o += GRAM_ROWS * GRAM_STRIDE * 4;
         o = (o + 15) & ~15u;
-        tabs = o; o += tgroup * (term_slots + GRAM_OVF) * 8;
+        tabs = o; o += union_slots ? GramUnionLds(union_slots).total : tgroup * (term_slots + GRAM_OVF) * 8;
+        o = (o + 15) & ~15u;
         ovf_cnt = o; o += 8 * 4;
         rowptr = o; o += GRAM_ROWS * 8;
         rownnz = o; o += GRAM_ROWS * 4;
@@ -281,10 +285,10 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
                                                                 uint32_t d, uint32_t* fwd, uint32_t* det_out, uint32_t* cnt_out,
                                                                 uint32_t* kw_out, uint32_t term_slots, uint32_t tgroup,
                                                                 uint32_t umap_slots, uint32_t map_slots, uint32_t words,
-                                                                unsigned long long* gfail) {
+                                                                uint32_t union_slots, unsigned long long* gfail) {
     constexpr uint32_t K = GRAM_ROWS;
     extern __shared__ __align__(16) char smem[];
-    const GramPruneLds L(term_slots, tgroup, umap_slots, map_slots, words);
+    const GramPruneLds L(term_slots, tgroup, umap_slots, map_slots, words, union_slots);
     float* G = reinterpret_cast<float*>(smem + L.G);
     uint2* tabs = reinterpret_cast<uint2*>(smem + L.tabs);
     uint32_t* ovf_cnt = reinterpret_cast<uint32_t*>(smem + L.ovf_cnt);
@@ -396,7 +400,8 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     // hybrid Gram matrix of the m rows
     if (m > 0 && wave < 4) gram_dense_64(C, nb_id, m, dense_mul, G, wave, lane);
     __syncthreads();
-    if (tgroup == 8) gram_sparse_64<8>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
+    if (union_slots) gram_sparse_union(C, nb_id, m, G, reinterpret_cast<char*>(tabs), union_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
+    else if (tgroup == 8) gram_sparse_64<8>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else gram_sparse_64<4>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     // (b) stable order by detour count
     for (uint32_t i = tid; i < m; i += NT) {
@@ -594,14 +599,18 @@ int launch_prune(apoe_knn* g, uint32_t degree) {
     const uint32_t gram_slots = next_pow2(std::max(64u, 2 * (g->corpus->max_nnz_s + g->corpus->max_nnz_b)));
     // 8 live pivot tables if two workgroups then still share a CU's LDS, else 4
     const uint32_t lds_budget = (uint32_t)std::min<size_t>(ctx->lds_per_block, 80 * 1024);
-    uint32_t tgroup = GramPruneLds(gram_slots, 8, uset_slots, map_slots, words).total <= lds_budget ? 8 : 4;
-    const GramPruneLds GL(gram_slots, tgroup, uset_slots, map_slots, words);
+    uint32_t tgroup = GramPruneLds(gram_slots, 8, uset_slots, map_slots, words, 0).total <= lds_budget ? 8 : 4;
+    // one union table for GU_T pivots when it fits: 2.5 slots per term of an average group, and room for the longest row alone
+    const double mean_nnz = g->n ? ((double)g->corpus->rec_bytes / g->n - DENSE_BYTES) / 8.0 : 0.0;
+    uint32_t union_slots = std::max(next_pow2((uint32_t)std::ceil(2.5 * GU_T * mean_nnz)), std::max(512u, gram_slots));
+    if (GramPruneLds(gram_slots, tgroup, uset_slots, map_slots, words, union_slots).total > lds_budget) union_slots = 0;
+    const GramPruneLds GL(gram_slots, tgroup, uset_slots, map_slots, words, union_slots);
     if (g->K == GRAM_ROWS && GL.total <= lds_budget && !g->force_sequential_prune) {
         APOE_HIP(hipMemsetAsync(g->counter.p + 1, 0, sizeof(unsigned long long), ctx->stream));
         APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&prune_gram_kernel<GRAM_THREADS>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GL.total));
         prune_gram_kernel<GRAM_THREADS><<<g->n, GRAM_THREADS, GL.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->norms.p, g->ids.p,
                                                                       g->dist.p, degree, g->fwd.p, g->det.p, g->cnt.p, g->kw.p, gram_slots,
-                                                                      tgroup, uset_slots, map_slots, words, g->counter.p + 1);
+                                                                      tgroup, uset_slots, map_slots, words, union_slots, g->counter.p + 1);
         APOE_HIP(hipGetLastError());
         unsigned long long failed = 0;
         APOE_HIP(hipMemcpyAsync(&failed, g->counter.p + 1, sizeof(failed), hipMemcpyDeviceToHost, ctx->stream));
