@@ -1,0 +1,122 @@
+"""A corpus with a few very long sparse rows among ordinary ones: the table overflow lists, the loop over rows
+longer than the register window and the union-table retry of the prune all run, and must not change a result."""
+import numpy as np
+import pytest
+
+from parity import assert_dist_close, assert_topk_match
+
+pytestmark = pytest.mark.gpu
+
+N, HEAVY_EVERY = 2000, 50  # every 50th doc is heavy: 450 SPLADE + 260 BM25 terms more than the others
+
+
+@pytest.fixture(scope="module")
+def heavy_world(gpu_ctx):
+    import apoe
+    import apoe_synth as S
+    import oracle as O
+    dense, s_off, s_idx, s_val, b_off, b_idx, b_val = S.to_numpy(S.corpus(N, seed=61, device="cpu"))
+    rng = np.random.default_rng(7)
+
+    def inflate(off, idx, val, n_terms, lo, hi):
+        rows_i, rows_v = [], []
+        for v in range(N):
+            i, x = idx[off[v]:off[v + 1]], val[off[v]:off[v + 1]]
+            if v % HEAVY_EVERY == 0:
+                extra = np.setdiff1d(rng.choice(30000, n_terms, replace=False).astype(np.uint32), i)
+                i = np.concatenate([i, extra])
+                x = np.concatenate([x, rng.uniform(lo, hi, len(extra)).astype(np.float32)])
+                o = np.argsort(i)
+                i, x = i[o], x[o]
+            rows_i.append(i)
+            rows_v.append(x)
+        new_off = np.zeros(N + 1, np.uint32)
+        new_off[1:] = np.cumsum([len(r) for r in rows_i])
+        return new_off, np.concatenate(rows_i).astype(np.uint32), np.concatenate(rows_v).astype(np.float32)
+
+    s_off, s_idx, s_val = inflate(s_off, s_idx, s_val, 450, 0.2, 2.0)
+    b_off, b_idx, b_val = inflate(b_off, b_idx, b_val, 260, 0.5, 8.0)
+    corpus = (dense, s_off, s_idx, s_val, b_off, b_idx, b_val)
+    queries = S.to_numpy(S.queries(100, seed=62, device="cpu"))
+    C, Q = O.HybridSet(*corpus), O.HybridSet(*queries)
+    rows, entry, knn_ids, knn_dist = O.build_index(C, dense_scale=7.0, K=64, iters=6, d=32, seed=5, return_knn=True)
+    gc = apoe.Corpus(gpu_ctx, *corpus)
+    gq = apoe.Queries(gpu_ctx, *queries)
+    info = gc.info()
+    assert info[2] > 400 and info[3] > 250  # the heavy rows are there
+    return dict(ctx=gpu_ctx, C=C, Q=Q, gc=gc, gq=gq, rows=rows, entry=entry, knn_ids=knn_ids, knn_dist=knn_dist)
+
+
+def test_pair_distances_with_heavy_pivots_and_candidates(heavy_world):
+    import apoe
+    import oracle as O
+    w = heavy_world
+    rng = np.random.default_rng(3)
+    heavy = np.arange(0, N, HEAVY_EVERY, dtype=np.uint32)
+    a = np.concatenate([rng.choice(heavy, 300), rng.integers(0, N, 300).astype(np.uint32), rng.choice(heavy, 300)]).astype(np.uint32)
+    b = np.concatenate([rng.integers(0, N, 300).astype(np.uint32), rng.choice(heavy, 300), rng.choice(heavy, 300)]).astype(np.uint32)
+    got = apoe.distance_pairs(w["ctx"], w["gc"], 7.0, a, b)
+    assert_dist_close(got, O.distance_pairs(w["C"], 7.0, a, b), "pairs with heavy rows")
+
+
+def test_nn_descent_stores_the_metric(heavy_world):
+    """Every stored distance is the metric of that pair: heavy pivots go through the overflow list of the
+    four-entry bucket table, heavy candidates through the loop over more than 192 pairs."""
+    import apoe
+    import oracle as O
+    w = heavy_world
+    knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+    knn.init(9)
+    for it in range(4):
+        knn.iterate(last=(it == 3))
+    knn.merge_reverse()
+    ids, dist = knn.download()
+    knn.close()
+    assert np.all(np.diff(dist, axis=1) >= 0) and ids.max() < N
+    heavy = np.arange(0, N, HEAVY_EVERY)
+    rows_ = np.concatenate([np.repeat(heavy, 64), np.random.default_rng(1).integers(0, N, 3000)])
+    cols_ = np.concatenate([np.tile(np.arange(64), len(heavy)), np.random.default_rng(2).integers(0, 64, 3000)])
+    want = O.distance_pairs(w["C"], 7.0, rows_.astype(np.uint32), ids[rows_, cols_])
+    assert_dist_close(dist[rows_, cols_], want, "stored distance == recomputed distance")
+    # ... and where a heavy row is the stored neighbour (a candidate with more than 192 pairs)
+    hr, hc = np.nonzero(np.isin(ids, heavy))
+    assert len(hr) > 1000
+    want = O.distance_pairs(w["C"], 7.0, hr[:4000].astype(np.uint32), ids[hr[:4000], hc[:4000]])
+    assert_dist_close(dist[hr[:4000], hc[:4000]], want, "stored distance of a heavy neighbour")
+
+
+def test_prune_matches_oracle_on_the_same_knn_graph(heavy_world):
+    import apoe
+    import oracle as O
+    w = heavy_world
+    knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+    knn.upload(w["knn_ids"], w["knn_dist"])
+    knn.prune(32)
+    g_fwd, g_det, g_cnt, g_kw = knn.prune_download()
+    graph = knn.finalize()
+    rows, entry = graph.download()
+    graph.close()
+    knn.close()
+    c_fwd, c_det, c_cnt, c_kw = O.prune(w["C"], 7.0, O.norms(w["C"], 7.0), w["knn_ids"], w["knn_dist"], 32)
+    same = np.all(g_fwd == c_fwd, axis=1)
+    assert same.mean() >= 0.995, same.mean()
+    assert np.array_equal(g_det[same], c_det[same]) and np.array_equal(g_cnt[same], c_cnt[same])
+    assert np.all(g_kw == c_kw, axis=1)[same].mean() >= 0.995
+    assert (rows == w["rows"]).all(axis=1).mean() >= 0.99
+    assert np.array_equal(entry, w["entry"])
+
+
+@pytest.mark.parametrize("w3", [(1.0, 1.0, 1.0), (0.0, 1.0, 1.0)])
+def test_search_matches_oracle(heavy_world, w3):
+    import apoe
+    import oracle as O
+    w = heavy_world
+    g = apoe.Graph(w["ctx"], w["rows"], w["entry"])
+    ids, dist, st = apoe.search(w["ctx"], w["gc"], w["gq"], g, w3, 64)
+    oid, odist, cnt = O.search(w["C"], w["Q"], w["rows"], w["entry"], w3, 64)
+    assert assert_topk_match(ids, dist, oid, odist, 10, f"heavy rows, weights {w3}") > 0.97
+    same = ids == oid
+    assert_dist_close(dist[same], odist[same], "pool distances")
+    ids2, dist2, _ = apoe.search(w["ctx"], w["gc"], w["gq"], g, w3, 64, variant=0x100)
+    assert np.array_equal(ids, ids2) and np.array_equal(dist, dist2)
+    g.close()
