@@ -15,24 +15,27 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int GRAM_ROWS = 64;
 constexpr int GRAM_STRIDE = GRAM_ROWS + 1; // odd stride: column reads do not collide on LDS banks
 
-// G[i][j] = dense_mul * <dense_i, dense_j> for i, j < 64; rows >= m repeat row m-1 (their
-// entries are never read). Called by 4 waves; wave w owns tile (w >> 1, w & 1).
+// G[i][j] (+)= dense_mul * <dense_i, dense_j> over the 8-float blocks [b_begin, b_end) of the rows, for
+// i, j < 64; rows >= m repeat row m-1 (their entries are never read). One call computes the 32x32
+// tile (tile >> 1, tile & 1); `add` says whether the tile's partial sum is stored or added (two
+// groups of four waves split the 1024 dimensions between them, the second group adds after a barrier).
 // MFMA 32x32x2 operand layout: lane l feeds A[l % 32][l / 32] and B[l / 32][l % 32];
 // accumulator register v of lane l is C[8 * (v / 4) + 4 * (l / 32) + v % 4][l % 32].
 // A lane therefore streams ITS row: float4 number (2 * block + l / 32) of every 8-float block,
 // and the four components go into four consecutive MFMAs (the k order inside the sum is free).
-__device__ __forceinline__ void gram_dense_64(const CorpusView& C, const uint32_t* ids, uint32_t m, float dense_mul, float* G, int wave,
-                                              int lane) {
-    const int ti = wave >> 1, tj = wave & 1;
-    if ((uint32_t)(ti * 32) >= m || (uint32_t)(tj * 32) >= m) return;
-    const uint32_t ra = min((uint32_t)(ti * 32 + (lane & 31)), m - 1), rb = min((uint32_t)(tj * 32 + (lane & 31)), m - 1);
-    const float4* pa = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[ra]]) * 16) + (lane >> 5);
-    const float4* pb = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[rb]]) * 16) + (lane >> 5);
+__device__ __forceinline__ floatx16 gram_dense_tile(const CorpusView& C, const uint32_t* ids, uint32_t m, int tile, int lane, int b_begin,
+                                                    int b_end, bool& active) {
+    const int ti = tile >> 1, tj = tile & 1;
     floatx16 acc;
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[v] = 0.f;
+    active = !((uint32_t)(ti * 32) >= m || (uint32_t)(tj * 32) >= m);
+    if (!active) return acc;
+    const uint32_t ra = min((uint32_t)(ti * 32 + (lane & 31)), m - 1), rb = min((uint32_t)(tj * 32 + (lane & 31)), m - 1);
+    const float4* pa = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[ra]]) * 16) + (lane >> 5);
+    const float4* pb = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[rb]]) * 16) + (lane >> 5);
     if (ti == tj) {
-        for (int b = 0; b < DIM / 8; b += 4) {
+        for (int b = b_begin; b < b_end; b += 4) {
             float4 a[4];
 #pragma unroll
             for (int u = 0; u < 4; u++) a[u] = pa[2 * (b + u)];
@@ -45,7 +48,7 @@ __device__ __forceinline__ void gram_dense_64(const CorpusView& C, const uint32_
             }
         }
     } else {
-        for (int b = 0; b < DIM / 8; b += 4) {
+        for (int b = b_begin; b < b_end; b += 4) {
             float4 a[4], bb[4];
 #pragma unroll
             for (int u = 0; u < 4; u++) { a[u] = pa[2 * (b + u)]; bb[u] = pb[2 * (b + u)]; }
@@ -58,10 +61,16 @@ __device__ __forceinline__ void gram_dense_64(const CorpusView& C, const uint32_
             }
         }
     }
+    return acc;
+}
+
+__device__ __forceinline__ void gram_dense_store(float* G, int tile, int lane, const floatx16& acc, float dense_mul, bool add) {
+    const int ti = tile >> 1, tj = tile & 1;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
         const int i = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4), j = lane & 31;
-        G[(ti * 32 + i) * GRAM_STRIDE + tj * 32 + j] = dense_mul * acc[v];
+        float* at = &G[(ti * 32 + i) * GRAM_STRIDE + tj * 32 + j];
+        *at = add ? *at + dense_mul * acc[v] : dense_mul * acc[v];
     }
 }
 

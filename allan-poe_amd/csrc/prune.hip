@@ -398,7 +398,17 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
         }
     }
     // hybrid Gram matrix of the m rows
-    if (m > 0 && wave < 4) gram_dense_64(C, nb_id, m, dense_mul, G, wave, lane);
+    // waves 0-3 take the first half of the dimensions of the four tiles, waves 4-7 (if there) the second half
+    {
+        constexpr int NWAVES = NT / WAVE, PARTS = NWAVES >= 8 ? 2 : 1, BLOCKS = DIM / 8;
+        const int part = wave >> 2;
+        bool active = false;
+        floatx16 acc;
+        if (m > 0 && part < PARTS) acc = gram_dense_tile(C, nb_id, m, wave & 3, lane, part * (BLOCKS / PARTS), (part + 1) * (BLOCKS / PARTS), active);
+        if (active && part == 0) gram_dense_store(G, wave & 3, lane, acc, dense_mul, false);
+        __syncthreads();
+        if (active && part == 1) gram_dense_store(G, wave & 3, lane, acc, dense_mul, true);
+    }
     __syncthreads();
     if (union_slots) gram_sparse_union(C, nb_id, m, G, reinterpret_cast<char*>(tabs), union_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else if (tgroup == 8) gram_sparse_64<8>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
