@@ -243,7 +243,7 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
 constexpr int GRAM_THREADS = 512; // 8 waves share one node's tables: more lookups in flight per byte of LDS
 
 struct GramPruneLds {
-    uint32_t G, tabs, ovf_cnt, rowptr, rownnz, umap, R, idmap, nb_id, nb_dist, nrm, det, order, sel_gi, sel_live, sel_kw, o_fwd, o_det, o_kw, ctl, total;
+    uint32_t G, tabs, ovf_cnt, rowptr, rownnz, umap, R, F, idmap, nb_id, nb_dist, nrm, det, order, sel_gi, sel_live, sel_kw, o_fwd, o_det, o_kw, ctl, total;
     // union_slots != 0: the table region holds one union table (apoe_gram.h) instead of tgroup pivot tables
     __host__ __device__ GramPruneLds(uint32_t term_slots, uint32_t tgroup, uint32_t umap_slots, uint32_t map_slots, uint32_t words,
                                      uint32_t union_slots) {
@@ -258,6 +258,7 @@ struct GramPruneLds {
         umap = o; o += umap_slots * 8;
         idmap = o; o += map_slots * 8;
         R = o; o += GRAM_ROWS * words * 4;
+        F = o; o += GRAM_ROWS * 2 * 4; // keyword-flag matrix: bit s of row c = "s holds a term of u that c lacks"
         nb_id = o; o += GRAM_ROWS * 4;
         nb_dist = o; o += GRAM_ROWS * 4;
         nrm = o; o += GRAM_ROWS * 4;
@@ -297,6 +298,7 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     uint2* umap = reinterpret_cast<uint2*>(smem + L.umap);
     uint2* idmap = reinterpret_cast<uint2*>(smem + L.idmap);
     uint32_t* R = reinterpret_cast<uint32_t*>(smem + L.R);
+    uint32_t* F = reinterpret_cast<uint32_t*>(smem + L.F);
     uint32_t* nb_id = reinterpret_cast<uint32_t*>(smem + L.nb_id);
     float* nb_dist = reinterpret_cast<float*>(smem + L.nb_dist);
     float* nrm = reinterpret_cast<float*>(smem + L.nrm);
@@ -319,6 +321,7 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     for (uint32_t i = tid; i < umap_slots; i += NT) umap[i] = make_uint2(EMPTY, 0u);
     for (uint32_t i = tid; i < K * words; i += NT) R[i] = 0;
     for (uint32_t i = tid; i < K; i += NT) det[i] = 0;
+    for (uint32_t i = tid; i < K * 2; i += NT) F[i] = 0;
     if (tid < 16) ctl[tid] = 0;
     __syncthreads();
 
@@ -422,33 +425,42 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     }
     __syncthreads();
 
-    // (c)+(d) sequential selection on the Gram matrix: wave 0, one lane per selected member
+    // keyword flags of all pairs at once (index.cu:637,651-654): flag(c, s) = (R[s] & ~R[c]) != 0
+    for (uint32_t p = tid; p < m * m; p += NT) {
+        const uint32_t c = p / m, sidx = p % m;
+        bool flag = false;
+        for (uint32_t w = 0; w < words; w++) flag |= (R[sidx * words + w] & ~R[c * words + w]) != 0;
+        if (flag) atomicOr(&F[c * 2 + (sidx >> 5)], 1u << (sidx & 31));
+    }
+    __syncthreads();
+
+    // (c)+(d) sequential selection on the Gram matrix: wave 0, lane i keeps selected member i in registers
     if (wave == 0 && m > 0) {
         uint32_t n_sel = 1;
-        if (lane == 0) { sel_gi[0] = order[0]; sel_live[0] = 1; sel_kw[0] = 0; }
-        wave_fence_lds();
+        uint32_t my_gi = order[0], my_kw = 0;
+        bool my_live = lane == 0;
+        float my_nrm = nrm[my_gi];
         for (uint32_t t = 1; t < m; t++) {
-            const uint32_t c = order[t];
+            const uint32_t c = uniform(order[t]);
             const float norm_c = nrm[c];
+            const uint64_t fc = ((uint64_t)F[c * 2 + 1] << 32) | F[c * 2];
             bool rej = false, noflag = false, tomb = false;
-            if ((uint32_t)lane < n_sel && sel_live[lane]) {
-                const uint32_t sgi = sel_gi[lane];
-                const float p = G[c * GRAM_STRIDE + sgi];
+            if ((uint32_t)lane < n_sel && my_live) {
+                const float p = G[c * GRAM_STRIDE + my_gi];
                 rej = norm_c < p;
-                tomb = nrm[sgi] < p;
-                bool flag = false;
-                for (uint32_t w = 0; w < words; w++) flag |= (R[sgi * words + w] & ~R[c * words + w]) != 0;
-                noflag = !flag;
+                tomb = my_nrm < p;
+                noflag = !((fc >> my_gi) & 1ull);
             }
             const bool reject = __ballot(rej) != 0;
             const bool allflag = __ballot(noflag) == 0;
-            if (tomb) sel_live[lane] = 0;
+            if (tomb) my_live = false;
             if (!reject) {
-                if (lane == 0) { sel_gi[n_sel] = c; sel_live[n_sel] = 1; sel_kw[n_sel] = allflag ? 1u : 0u; }
+                if ((uint32_t)lane == n_sel) { my_gi = c; my_live = true; my_nrm = norm_c; my_kw = allflag ? 1u : 0u; }
                 n_sel++;
             }
-            wave_fence_lds();
         }
+        if ((uint32_t)lane < n_sel) { sel_gi[lane] = my_gi; sel_live[lane] = my_live ? 1u : 0u; sel_kw[lane] = my_kw; }
+        wave_fence_lds();
         // (e) emit
         if (lane == 0) {
             uint32_t cnt = 0, nkw = 0;
