@@ -8,6 +8,7 @@ namespace apoe {
 constexpr int MAX_NEW = 64;   // fresh candidates per step: one lane each in wave 0
 constexpr int EVAL_BATCH = 3;  // candidates whose sparse parts a wave keeps in flight together
 constexpr int DENSE_BATCH = 1; // dense rows a wave keeps in flight together
+constexpr int MERGE_ROUNDS = 4; // 64-element rounds of the pool that the merge moves per LDS round trip
 constexpr int RING = 32;      // keyword-filter search: evicted keyword hits kept beside the pool (query.cu:18)
 
 // What the kernel does on top of the plain beam search.
@@ -180,22 +181,36 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
         wave_fence();
     }
     const uint32_t lo0 = uniform(P.lb[0]);
-    for (int base = (int)((cands - 1) & ~(uint32_t)(WAVE - 1)); base >= 0 && (uint32_t)base + WAVE > lo0; base -= WAVE) {
-        const uint32_t p = base + lane;
-        const bool act = p >= lo0 && p < cands;
-        float v = 0.f;
-        uint32_t pid = 0, pent = 0, phop = 0, shift = 0;
-        if (act) {
-            v = P.dist[p];
-            pid = P.id[p];
-            if (KG) { pent = P.ent[p]; phop = P.hop[p]; }
-            for (uint32_t i = 0; i < n_in; i++) shift += P.lb[i] <= p;
+    // MERGE_ROUNDS rounds are read before any of them is written: one LDS round trip per group, and a
+    // group only writes at or above its own positions (into rounds that were moved before it)
+    for (int top = (int)((cands - 1) & ~(uint32_t)(WAVE - 1)); top >= 0 && (uint32_t)top + WAVE > lo0; top -= WAVE * MERGE_ROUNDS) {
+        float v[MERGE_ROUNDS];
+        uint32_t pid[MERGE_ROUNDS], pent[MERGE_ROUNDS], phop[MERGE_ROUNDS], dst[MERGE_ROUNDS];
+#pragma unroll
+        for (int r = 0; r < MERGE_ROUNDS; r++) {
+            const int base = top - r * WAVE;
+            const uint32_t p = (uint32_t)(base + lane);
+            const bool act = base >= 0 && (uint32_t)base + WAVE > lo0 && p >= lo0 && p < cands;
+            dst[r] = cands; // nothing to write
+            v[r] = 0.f;
+            pid[r] = pent[r] = phop[r] = 0;
+            if (act) {
+                v[r] = P.dist[p];
+                pid[r] = P.id[p];
+                if (KG) { pent[r] = P.ent[p]; phop[r] = P.hop[p]; }
+                uint32_t shift = 0;
+                for (uint32_t i = 0; i < n_in; i++) shift += (uint32_t)__builtin_amdgcn_readlane((int)lb, i) <= p;
+                dst[r] = p + shift;
+            }
         }
         wave_fence();
-        if (act && p + shift < cands) {
-            P.dist[p + shift] = v;
-            P.id[p + shift] = pid;
-            if (KG) { P.ent[p + shift] = pent; P.hop[p + shift] = phop; }
+#pragma unroll
+        for (int r = 0; r < MERGE_ROUNDS; r++) {
+            if (dst[r] < cands) {
+                P.dist[dst[r]] = v[r];
+                P.id[dst[r]] = pid[r];
+                if (KG) { P.ent[dst[r]] = pent[r]; P.hop[dst[r]] = phop[r]; }
+            }
         }
         wave_fence();
     }
