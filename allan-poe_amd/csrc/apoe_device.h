@@ -89,40 +89,6 @@ __device__ __forceinline__ uint64_t shfl_xor64(uint64_t v, int m) {
     return ((uint64_t)hi << 32) | lo;
 }
 
-// Bitonic sort of one 64-bit key per lane across the wave, ascending by lane.
-__device__ __forceinline__ uint64_t wave_sort64(uint64_t key) {
-    const int lane = lane_id();
-#pragma unroll
-    for (int k = 2; k <= WAVE; k <<= 1) {
-#pragma unroll
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            uint64_t other = shfl_xor64(key, j);
-            bool up = (lane & k) == 0;       // ascending block
-            bool lower = (lane & j) == 0;    // this lane keeps the smaller in an ascending block
-            bool take_min = up == lower;
-            key = take_min ? (key < other ? key : other) : (key < other ? other : key);
-        }
-    }
-    return key;
-}
-// Same with a 32-bit payload that travels with the key.
-__device__ __forceinline__ void wave_sort64_payload(uint64_t& key, uint32_t& pay0, uint32_t& pay1) {
-    const int lane = lane_id();
-#pragma unroll
-    for (int k = 2; k <= WAVE; k <<= 1) {
-#pragma unroll
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            uint64_t other = shfl_xor64(key, j);
-            uint32_t o0 = __shfl_xor(pay0, j, WAVE), o1 = __shfl_xor(pay1, j, WAVE);
-            bool up = (lane & k) == 0;
-            bool lower = (lane & j) == 0;
-            bool take_min = up == lower;
-            bool swap = take_min ? (other < key) : (key < other);
-            if (swap) { key = other; pay0 = o0; pay1 = o1; }
-        }
-    }
-}
-
 // ---- LDS term hash: (key, value-bits) slots, open addressing, linear probing ----
 
 __device__ __forceinline__ uint32_t term_hash(uint32_t key, uint32_t mask) {
@@ -281,93 +247,13 @@ __device__ __forceinline__ EvalOut eval_wave(const CorpusView& C, uint32_t id, c
     return o;
 }
 
-// Euclidean norm of the pivot's dense part as held in registers (weights included).
-__device__ __forceinline__ float pivot_dense_norm(const PivotDense& p) {
-    float a = 0.f;
-#pragma unroll
-    for (int i = 0; i < NV; i++) a += p.v[i].x * p.v[i].x + p.v[i].y * p.v[i].y + p.v[i].z * p.v[i].z + p.v[i].w * p.v[i].w;
-    return sqrtf(wave_sum_dpp(a));
-}
-
-struct BoundedOut {
-    float dist;      // 1 - ip - bonus, or INF_DIS when the dense part was skipped
-    uint32_t nnz_s;  // SPLADE pairs read
-    uint32_t nnz_b;  // BM25 pairs read
-    bool dense_read; // the 4 KB dense row was read
-    bool kw_hit;     // keyword-filter search only: a BM25 term of the document is one of the query's required keywords
-};
-
-// Two-stage hybrid distance between the pivot and document `id` (wave-uniform).
-// Stage 1 reads the descriptor, the dense norm and the pairs and forms the sparse sum.
-// |<pivot_d, doc_d>| <= |pivot_d| * |doc_d|, so 1 - (sparse + dense_mul*|p|*|d|) - bonus is a
-// lower bound of the distance: if even that is above `thr` (the value the caller would reject
-// anyway: the worst entry of a full pool / list), the dense row is not read and INF_DIS is
-// returned. Otherwise stage 2 reads the row. Pass thr = +inf to always get the exact distance.
-__device__ __forceinline__ BoundedOut eval_wave_bounded(const CorpusView& C, uint32_t id, const PivotDense& pv, float pv_norm, const uint2* tab,
-                                                        uint32_t mask, uint32_t paths, float dense_mul, float bonus, float thr) {
-    const int lane = lane_id();
-    const uint64_t desc = C.desc[id];
-    const char* rec = C.recs + desc_off(desc) * 16;
-    const uint32_t ns = desc_nnz_s(desc), nb = desc_nnz_b(desc);
-    const uint32_t begin = (paths & PATH_SPARSE) ? 0u : ns;
-    const uint32_t end = (paths & PATH_BM25) ? ns + nb : ns;
-    BoundedOut o;
-    o.nnz_s = (paths & PATH_SPARSE) ? ns : 0u;
-    o.nnz_b = (paths & PATH_BM25) ? nb : 0u;
-    o.dense_read = false;
-    o.kw_hit = false;
-    float ssum = 0.f;
-    const bool has_sparse = (paths & (PATH_SPARSE | PATH_BM25)) != 0;
-    if (has_sparse) {
-        const float dub = (paths & PATH_DENSE) ? dense_mul * pv_norm * C.dnorm[id] : 0.f;
-        const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
-        uint2 kv0 = make_uint2(0, 0), kv1 = kv0, kv2 = kv0;
-        const uint32_t j0 = begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
-        if (j0 < end) kv0 = sp[j0];
-        if (j1 < end) kv1 = sp[j1];
-        if (j2 < end) kv2 = sp[j2];
-        float acc = 0.f;
-        if (j0 < end) term_table_probe(tab, mask, kv0.x, __uint_as_float(kv0.y), acc);
-        if (j1 < end) term_table_probe(tab, mask, kv1.x, __uint_as_float(kv1.y), acc);
-        if (j2 < end) term_table_probe(tab, mask, kv2.x, __uint_as_float(kv2.y), acc);
-        for (uint32_t j = j2 + WAVE; j < end; j += WAVE) {
-            const uint2 kv = sp[j];
-            term_table_probe(tab, mask, kv.x, __uint_as_float(kv.y), acc);
-        }
-        ssum = wave_sum_dpp(acc);
-        if (!(paths & PATH_DENSE)) {
-            o.dist = 1.0f - ssum - bonus;
-            return o;
-        }
-        const float lb = 1.0f - (ssum + dub) - bonus;
-        if (lb > thr + 1e-5f * (fabsf(ssum) + dub + fabsf(bonus) + 1.0f)) {
-            o.dist = INF_DIS;
-            return o;
-        }
-    }
-    float dsum = 0.f;
-    if (paths & PATH_DENSE) {
-        const float4* r = reinterpret_cast<const float4*>(rec);
-        float4 x[NV];
-#pragma unroll
-        for (int i = 0; i < NV; i++) x[i] = r[lane + WAVE * i];
-        float acc = 0.f;
-#pragma unroll
-        for (int i = 0; i < NV; i++) {
-            acc = fmaf(x[i].x, pv.v[i].x, acc);
-            acc = fmaf(x[i].y, pv.v[i].y, acc);
-            acc = fmaf(x[i].z, pv.v[i].z, acc);
-            acc = fmaf(x[i].w, pv.v[i].w, acc);
-        }
-        dsum = dense_mul * wave_sum_dpp(acc);
-        o.dense_read = true;
-    }
-    o.dist = 1.0f - (dsum + ssum) - bonus;
-    return o;
-}
-
-// The same two-stage evaluation split in two calls, so that a wave can have the sparse
-// parts of several candidates in flight before it consumes the first one.
+// ---- two-stage evaluation ----
+// Stage 1 reads the candidate's descriptor, dense norm and pairs and forms the sparse sum.
+// |<pivot_d, doc_d>| <= |pivot_d| * |doc_d|, so 1 - (sparse + dense_mul*|p|*|d|) - bonus is a lower
+// bound of the distance: if even that is above `thr` (the value the caller would reject anyway: the
+// worst entry of a full pool / list), the dense row is not read and INF_DIS is reported. Otherwise
+// stage 2 reads the row. thr = +inf always gives the exact distance. The stages are separate calls
+// so that a wave can have the loads of several candidates in flight before it consumes the first.
 struct PendingEval {
     const char* rec;
     uint2 kv0, kv1, kv2;
@@ -409,71 +295,6 @@ __device__ __forceinline__ uint64_t readlane64(uint64_t v, uint32_t src) {
 }
 __device__ __forceinline__ float readlane_f32(float v, uint32_t src) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
-}
-
-// A pair of the candidate against the query's table. With KWD, a BM25 pair that hits the table and
-// whose term is in `kwset` (the query's required keywords, keys carry BM25_BIT) raises `hit`
-// (the test of the search-time cal_bm25_dist, utils.cuh:318-340).
-template <bool KWD>
-__device__ __forceinline__ void probe_query_pair(const uint2* tab, uint32_t mask, uint2 kv, float& acc, const uint32_t* kwset, uint32_t kwmask,
-                                                 bool& hit) {
-    const bool found = term_table_probe(tab, mask, kv.x, __uint_as_float(kv.y), acc);
-    if (KWD) {
-        if (found && (kv.x & BM25_BIT) && id_set_contains(kwset, kwmask, kv.x)) hit = true;
-    }
-}
-
-template <bool KWD = false>
-__device__ __forceinline__ BoundedOut eval_finish(const PendingEval& p, const PivotDense& pv, const uint2* tab, uint32_t mask, uint32_t paths,
-                                                  float dense_mul, float bonus, float thr, const uint32_t* kwset = nullptr,
-                                                  uint32_t kwmask = 0) {
-    const int lane = lane_id();
-    BoundedOut o;
-    o.nnz_s = (paths & PATH_SPARSE) ? p.ns : 0u;
-    o.nnz_b = (paths & PATH_BM25) ? p.nb : 0u;
-    o.dense_read = false;
-    o.kw_hit = false;
-    float ssum = 0.f;
-    if (paths & (PATH_SPARSE | PATH_BM25)) {
-        const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
-        const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
-        float acc = 0.f;
-        bool hit = false;
-        if (j0 < p.end) probe_query_pair<KWD>(tab, mask, p.kv0, acc, kwset, kwmask, hit);
-        if (j1 < p.end) probe_query_pair<KWD>(tab, mask, p.kv1, acc, kwset, kwmask, hit);
-        if (j2 < p.end) probe_query_pair<KWD>(tab, mask, p.kv2, acc, kwset, kwmask, hit);
-        for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) probe_query_pair<KWD>(tab, mask, sp[j], acc, kwset, kwmask, hit);
-        if (KWD) o.kw_hit = __ballot(hit) != 0;
-        ssum = wave_sum_dpp(acc);
-        if (!(paths & PATH_DENSE)) {
-            o.dist = 1.0f - ssum - bonus;
-            return o;
-        }
-        const float lb = 1.0f - (ssum + p.dub) - bonus;
-        if (lb > thr + 1e-5f * (fabsf(ssum) + p.dub + fabsf(bonus) + 1.0f)) {
-            o.dist = INF_DIS;
-            return o;
-        }
-    }
-    float dsum = 0.f;
-    if (paths & PATH_DENSE) {
-        const float4* r = reinterpret_cast<const float4*>(p.rec);
-        float4 x[NV];
-#pragma unroll
-        for (int i = 0; i < NV; i++) x[i] = r[lane + WAVE * i];
-        float acc = 0.f;
-#pragma unroll
-        for (int i = 0; i < NV; i++) {
-            acc = fmaf(x[i].x, pv.v[i].x, acc);
-            acc = fmaf(x[i].y, pv.v[i].y, acc);
-            acc = fmaf(x[i].z, pv.v[i].z, acc);
-            acc = fmaf(x[i].w, pv.v[i].w, acc);
-        }
-        dsum = dense_mul * wave_sum_dpp(acc);
-        o.dense_read = true;
-    }
-    o.dist = 1.0f - (dsum + ssum) - bonus;
-    return o;
 }
 
 // ---- bucket table: the query's terms for the search kernels ----
@@ -611,21 +432,8 @@ __device__ __forceinline__ void dense_issue(DenseRow& d, const char* rec) {
 #pragma unroll
     for (int i = 0; i < NV; i++) d.x[i] = r[lane + WAVE * i];
 }
-// dense_mul * <row, pivot>, the same FMA chain and reduction as eval_finish.
-__device__ __forceinline__ float dense_finish(const DenseRow& d, const PivotDense& pv, float dense_mul) {
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < NV; i++) {
-        acc = fmaf(d.x[i].x, pv.v[i].x, acc);
-        acc = fmaf(d.x[i].y, pv.v[i].y, acc);
-        acc = fmaf(d.x[i].z, pv.v[i].z, acc);
-        acc = fmaf(d.x[i].w, pv.v[i].w, acc);
-    }
-    return dense_mul * wave_sum_dpp(acc);
-}
-
-// The same with the pivot's dense row in LDS (float4 number l + 64*i belongs to lane l, as in
-// PivotDense): frees 64 registers per lane for kernels that need the occupancy more.
+// dense_mul * <row, pivot> with the pivot's dense row in LDS (float4 number l + 64*i belongs to lane l,
+// as in PivotDense): frees 64 registers per lane for kernels that need the occupancy more.
 __device__ __forceinline__ float dense_finish_lds(const DenseRow& d, const float4* pivot, float dense_mul) {
     const int lane = lane_id();
     float acc = 0.f;
