@@ -76,6 +76,15 @@ struct apoe_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     int num_cus = 0;
     size_t lds_per_block = 0;
+    // Search workspace (visited bitmaps, counters, once-per-query arguments): grows to the largest
+    // request and is kept until the context is destroyed, so that repeated searches do not pay for
+    // a device allocation each. One search at a time per context.
+    apoe::DevBuf<char> search_ws;
+    int search_workspace(size_t bytes, char** out) {
+        if (search_ws.n < bytes) APOE_TRY(search_ws.alloc(bytes));
+        *out = search_ws.p;
+        return APOE_OK;
+    }
 };
 
 struct apoe_corpus {

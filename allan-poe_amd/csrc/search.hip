@@ -766,24 +766,24 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     const uint32_t grid = std::min<uint32_t>(q_count, (uint32_t)per_cu * (uint32_t)ctx->num_cus);
 
     a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;
-    DevBuf<uint32_t> bitmaps;
-    DevBuf<unsigned long long> work;
-    DevBuf<SearchCold> cold_dev;
-    APOE_TRY(bitmaps.alloc((size_t)grid * a.bitmap_words));
-    APOE_TRY(work.alloc(8));
-    APOE_TRY(cold_dev.alloc(1));
-    APOE_HIP(hipMemcpy(cold_dev.p, &cold, sizeof(cold), hipMemcpyHostToDevice));
-    a.cold = cold_dev.p;
-    APOE_HIP(hipMemsetAsync(work.p, 0, 8 * sizeof(unsigned long long), ctx->stream));
-    a.bitmaps = bitmaps.p;
-    a.work = work.p;
+    // workspace: [counters: 8 x u64][once-per-query arguments][visited bitmaps]
+    const size_t cold_at = 8 * sizeof(unsigned long long), bitmaps_at = (cold_at + sizeof(SearchCold) + 255) & ~(size_t)255;
+    char* ws = nullptr;
+    APOE_TRY(ctx->search_workspace(bitmaps_at + (size_t)grid * a.bitmap_words * sizeof(uint32_t), &ws));
+    unsigned long long* work = reinterpret_cast<unsigned long long*>(ws);
+    APOE_HIP(hipMemcpyAsync(ws + cold_at, &cold, sizeof(cold), hipMemcpyHostToDevice, ctx->stream));
+    APOE_HIP(hipStreamSynchronize(ctx->stream)); // `cold` lives on this stack frame
+    a.cold = reinterpret_cast<const SearchCold*>(ws + cold_at);
+    APOE_HIP(hipMemsetAsync(work, 0, 8 * sizeof(unsigned long long), ctx->stream));
+    a.bitmaps = reinterpret_cast<uint32_t*>(ws + bitmaps_at);
+    a.work = work;
 
     float ms = 0.f;
     APOE_TRY(timed(ctx, &ms, [&]() { return launch_mode(ctx, mode, nw, a, grid, L.total, nullptr); }));
     APOE_HIP(hipStreamSynchronize(ctx->stream));
     if (stats) {
         unsigned long long h[8];
-        APOE_HIP(hipMemcpy(h, work.p, sizeof(h), hipMemcpyDeviceToHost));
+        APOE_HIP(hipMemcpy(h, work, sizeof(h), hipMemcpyDeviceToHost));
         stats->kernel_ms = ms;
         stats->expansions = h[1];
         stats->evaluations = h[2];
