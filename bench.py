@@ -98,7 +98,7 @@ def main():
     ap.add_argument("--nnd-iters", type=int, default=10)
     ap.add_argument("--cands", type=str, default="64,128,256,512")
     ap.add_argument("--truth-queries", type=int, default=1000)
-    ap.add_argument("--cpu-queries", type=int, default=2000)
+    ap.add_argument("--cpu-queries", type=int, default=10000)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--extras", action="store_true",
