@@ -37,7 +37,7 @@ class SearchStats(C.Structure):
 
 EXPORTS = [
     "apoe_last_error_string", "apoe_ctx_create", "apoe_ctx_destroy", "apoe_ctx_synchronize", "apoe_corpus_create",
-    "apoe_corpus_destroy", "apoe_corpus_info", "apoe_corpus_bytes", "apoe_queries_create", "apoe_queries_destroy",
+    "apoe_corpus_destroy", "apoe_corpus_info", "apoe_corpus_bytes", "apoe_corpus_pair_bytes", "apoe_queries_create", "apoe_queries_destroy",
     "apoe_kg_create", "apoe_kg_destroy", "apoe_calibrate_weights", "apoe_hybrid_distance_batch", "apoe_hybrid_distance_pairs", "apoe_norms",
     "apoe_knn_create", "apoe_knn_destroy", "apoe_nnd_init", "apoe_nnd_iterate", "apoe_nnd_merge_reverse",
     "apoe_knn_download", "apoe_knn_upload", "apoe_prune", "apoe_prune_download", "apoe_finalize_graph",
@@ -63,6 +63,8 @@ def lib():
         _lib.apoe_last_error_string.restype = C.c_char_p
         _lib.apoe_corpus_bytes.restype = C.c_uint64
         _lib.apoe_corpus_bytes.argtypes = [C.c_void_p]
+        _lib.apoe_corpus_pair_bytes.restype = C.c_uint32
+        _lib.apoe_corpus_pair_bytes.argtypes = [C.c_void_p]
         _lib.apoe_knn_elapsed_ms.restype = C.c_float
         _lib.apoe_knn_elapsed_ms.argtypes = [C.c_void_p]
         for name in ("apoe_ctx_destroy", "apoe_corpus_destroy", "apoe_queries_destroy", "apoe_kg_destroy",
@@ -133,6 +135,9 @@ class Corpus:
 
     def bytes(self):
         return int(lib().apoe_corpus_bytes(self.h))
+
+    def pair_bytes(self):
+        return int(lib().apoe_corpus_pair_bytes(self.h))
 
     def close(self):
         if self.h:

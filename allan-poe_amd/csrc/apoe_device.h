@@ -32,13 +32,21 @@ __host__ __device__ inline uint64_t desc_off(uint64_t d) { return d & DESC_OFF_M
 __host__ __device__ inline uint32_t desc_nnz_s(uint64_t d) { return (uint32_t)(d >> DESC_OFF_BITS) & DESC_NNZ_MAX; }
 __host__ __device__ inline uint32_t desc_nnz_b(uint64_t d) { return (uint32_t)(d >> (DESC_OFF_BITS + DESC_NNZ_BITS)) & DESC_NNZ_MAX; }
 
-// Record = [DIM floats][nnz_s x (term, value)][nnz_b x (term | BM25_BIT, value)], 16-byte aligned.
+// Record = [DIM floats][pairs], 16-byte aligned, pairs = nnz_s SPLADE terms then nnz_b BM25 terms.
+// Wide pairs:   nnz x (term | path bit, value), two 32-bit words each.
+// Narrow pairs: nnz x value (f32), then nnz x term (u16); the path of pair j follows from j >= nnz_s.
+// A corpus is narrow when every term id of both paths is below 65536 (6 instead of 8 bytes a pair).
 struct CorpusView {
     const uint64_t* desc;
     const char* recs;
     const float* dnorm; // Euclidean norm of each dense row (bounds the dense inner product)
     uint32_t n;
+    uint32_t narrow;
 };
+
+__host__ __device__ inline uint64_t record_units(uint32_t nnz, bool narrow) { // 16-byte units of one record
+    return ((uint64_t)DENSE_BYTES + (uint64_t)(narrow ? 6 : 8) * nnz + 15) / 16;
+}
 
 struct SetView { // a set kept in CSR form on the device (queries)
     const float* dense;
@@ -54,6 +62,44 @@ struct SetView { // a set kept in CSR form on the device (queries)
 #ifdef __HIPCC__
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+// The path bit of pair j of a record with ns SPLADE pairs: narrow records do not store it.
+__device__ __forceinline__ uint32_t pair_flag(uint32_t narrow, uint32_t ns, uint32_t j) { return narrow && j >= ns ? 0x80000000u : 0u; }
+
+// The pair array of one record; [j] gives (term | path bit, value bits) whatever the format.
+// `narrow` is the same for every record of a corpus, so the branch on it is uniform (the hot
+// kernels make it a compile-time constant). raw(j) is the load alone: a kernel that wants the loads
+// of several rows in flight takes raw pairs and ORs pair_flag() in where it consumes them, because
+// an OR next to the load makes the wave wait for the load there.
+struct Pairs {
+    const char* base; // first byte after the dense row
+    uint32_t ns, nnz; // SPLADE pairs, all pairs
+    uint32_t narrow;
+    __device__ __forceinline__ uint2 raw(uint32_t j) const {
+        if (narrow) return make_uint2(reinterpret_cast<const uint16_t*>(base + 4 * (size_t)nnz)[j], reinterpret_cast<const uint32_t*>(base)[j]);
+        return reinterpret_cast<const uint2*>(base)[j];
+    }
+    __device__ __forceinline__ uint32_t key(uint32_t j) const {
+        if (narrow) return (uint32_t) reinterpret_cast<const uint16_t*>(base + 4 * (size_t)nnz)[j] | pair_flag(1, ns, j);
+        return reinterpret_cast<const uint2*>(base)[j].x;
+    }
+    __device__ __forceinline__ uint2 operator[](uint32_t j) const {
+        uint2 kv = raw(j);
+        kv.x |= pair_flag(narrow, ns, j);
+        return kv;
+    }
+};
+__device__ __forceinline__ Pairs record_pairs(const CorpusView& C, const char* rec, uint32_t ns, uint32_t nb) {
+    Pairs p;
+    p.base = rec + DENSE_BYTES;
+    p.ns = ns;
+    p.nnz = ns + nb;
+    p.narrow = C.narrow;
+    return p;
+}
+__device__ __forceinline__ Pairs record_pairs(const CorpusView& C, uint64_t desc) {
+    return record_pairs(C, C.recs + desc_off(desc) * 16, desc_nnz_s(desc), desc_nnz_b(desc));
+}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -138,9 +184,8 @@ __device__ __forceinline__ void pivot_dense_load(PivotDense& p, const float* row
 }
 
 // Insert the sparse part of a packed document record (all pairs, both paths).
-__device__ __forceinline__ void pivot_terms_from_record(uint2* tab, uint32_t mask, const char* rec, uint32_t nnz, int tid, int nthreads) {
-    const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
-    for (uint32_t j = tid; j < nnz; j += nthreads) {
+__device__ __forceinline__ void pivot_terms_from_record(uint2* tab, uint32_t mask, const Pairs& sp, int tid, int nthreads) {
+    for (uint32_t j = tid; j < sp.nnz; j += nthreads) {
         uint2 kv = sp[j];
         term_table_insert(tab, mask, kv.x, __uint_as_float(kv.y));
     }
@@ -210,7 +255,7 @@ __device__ __forceinline__ EvalOut eval_wave(const CorpusView& C, uint32_t id, c
     const uint32_t ns = desc_nnz_s(desc), nb = desc_nnz_b(desc);
     const uint32_t begin = (paths & PATH_SPARSE) ? 0u : ns;
     const uint32_t end = (paths & PATH_BM25) ? ns + nb : ns;
-    const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
+    const Pairs sp = record_pairs(C, rec, ns, nb);
     float4 x[NV];
     if (paths & PATH_DENSE) {
         const float4* r = reinterpret_cast<const float4*>(rec);
@@ -256,7 +301,7 @@ __device__ __forceinline__ EvalOut eval_wave(const CorpusView& C, uint32_t id, c
 // so that a wave can have the loads of several candidates in flight before it consumes the first.
 struct PendingEval {
     const char* rec;
-    uint2 kv0, kv1, kv2;
+    uint2 kv0, kv1, kv2; // raw pairs: the consumer adds pair_flag()
     uint32_t ns, nb, begin, end;
     float dub;
 };
@@ -271,16 +316,16 @@ __device__ __forceinline__ void eval_issue_desc(PendingEval& p, const CorpusView
     p.begin = (paths & PATH_SPARSE) ? 0u : p.ns;
     p.end = (paths & PATH_BM25) ? p.ns + p.nb : p.ns;
     p.dub = (paths & PATH_DENSE) ? dense_mul * pv_norm * dnorm : 0.f;
-    const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
+    const Pairs sp = record_pairs(C, p.rec, p.ns, p.nb);
     const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
     p.kv0 = p.kv1 = p.kv2 = make_uint2(0, 0);
     // no per-lane branches: a lane past the end of the row loads the row's last pair again and the
     // consumer masks it (it tests j < end anyway)
     if (p.begin < p.end) {
         const uint32_t last = p.end - 1;
-        p.kv0 = sp[min(j0, last)];
-        p.kv1 = sp[min(j1, last)];
-        p.kv2 = sp[min(j2, last)];
+        p.kv0 = sp.raw(min(j0, last));
+        p.kv1 = sp.raw(min(j1, last));
+        p.kv2 = sp.raw(min(j2, last));
     }
 }
 
@@ -364,28 +409,31 @@ __device__ __forceinline__ void overflow_match(const BucketTab& T, uint32_t n_ov
 
 // n_ovf is the (wave-uniform) overflow count read after the table was built.
 template <bool KWD>
-__device__ __forceinline__ float sparse_probe(const PendingEval& p, const BucketTab& T, uint32_t n_ovf, uint32_t paths, const uint32_t* kwset,
-                                              uint32_t kwmask, bool& hit) {
+__device__ __forceinline__ float sparse_probe(const CorpusView& C, const PendingEval& p, const BucketTab& T, uint32_t n_ovf, uint32_t paths,
+                                              const uint32_t* kwset, uint32_t kwmask, bool& hit) {
     const int lane = lane_id();
     float acc = 0.f;
     if (!(paths & (PATH_SPARSE | PATH_BM25))) return acc;
     const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
     const bool in0 = j0 < p.end, in1 = j1 < p.end, in2 = j2 < p.end;
-    uint4 e0 = T.b[term_hash(p.kv0.x, T.mask)];
-    uint4 e1 = T.b[term_hash(p.kv1.x, T.mask)];
-    uint4 e2 = T.b[term_hash(p.kv2.x, T.mask)];
+    const uint2 kv0 = make_uint2(p.kv0.x | pair_flag(C.narrow, p.ns, j0), p.kv0.y);
+    const uint2 kv1 = make_uint2(p.kv1.x | pair_flag(C.narrow, p.ns, j1), p.kv1.y);
+    const uint2 kv2 = make_uint2(p.kv2.x | pair_flag(C.narrow, p.ns, j2), p.kv2.y);
+    uint4 e0 = T.b[term_hash(kv0.x, T.mask)];
+    uint4 e1 = T.b[term_hash(kv1.x, T.mask)];
+    uint4 e2 = T.b[term_hash(kv2.x, T.mask)];
     // keep the three reads together: nothing below may be scheduled between them
     asm volatile("" : "+v"(e0.x), "+v"(e1.x), "+v"(e2.x));
-    bucket_match<KWD>(e0, p.kv0, in0, acc, kwset, kwmask, hit);
-    bucket_match<KWD>(e1, p.kv1, in1, acc, kwset, kwmask, hit);
-    bucket_match<KWD>(e2, p.kv2, in2, acc, kwset, kwmask, hit);
+    bucket_match<KWD>(e0, kv0, in0, acc, kwset, kwmask, hit);
+    bucket_match<KWD>(e1, kv1, in1, acc, kwset, kwmask, hit);
+    bucket_match<KWD>(e2, kv2, in2, acc, kwset, kwmask, hit);
     if (n_ovf) {
-        overflow_match<KWD>(T, n_ovf, p.kv0, in0, acc, kwset, kwmask, hit);
-        overflow_match<KWD>(T, n_ovf, p.kv1, in1, acc, kwset, kwmask, hit);
-        overflow_match<KWD>(T, n_ovf, p.kv2, in2, acc, kwset, kwmask, hit);
+        overflow_match<KWD>(T, n_ovf, kv0, in0, acc, kwset, kwmask, hit);
+        overflow_match<KWD>(T, n_ovf, kv1, in1, acc, kwset, kwmask, hit);
+        overflow_match<KWD>(T, n_ovf, kv2, in2, acc, kwset, kwmask, hit);
     }
     if (p.begin + 3 * WAVE < p.end) { // rows with more than 192 pairs
-        const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
+        const Pairs sp = record_pairs(C, p.rec, p.ns, p.nb);
         for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) {
             const uint2 kv = sp[j];
             bucket_match<KWD>(T.b[term_hash(kv.x, T.mask)], kv, true, acc, kwset, kwmask, hit);
@@ -486,9 +534,8 @@ __device__ __forceinline__ void bucket4_insert(const Bucket4Tab& T, uint32_t key
     if (at < T.ovf_cap) T.ovf[at] = make_uint2(key, val_bits);
 }
 
-__device__ __forceinline__ void bucket4_terms_from_record(const Bucket4Tab& T, const char* rec, uint32_t nnz, int tid, int nthreads) {
-    const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
-    for (uint32_t j = tid; j < nnz; j += nthreads) {
+__device__ __forceinline__ void bucket4_terms_from_record(const Bucket4Tab& T, const Pairs& sp, int tid, int nthreads) {
+    for (uint32_t j = tid; j < sp.nnz; j += nthreads) {
         const uint2 kv = sp[j];
         bucket4_insert(T, kv.x, kv.y);
     }
@@ -504,15 +551,14 @@ __device__ __forceinline__ bool bucket4_match(const uint4 e0, const uint4 e1, ui
 }
 
 // Terms that are not in their bucket: the overflow list, or the pivot's pair array if the list overflowed.
-__device__ __forceinline__ void bucket4_overflow(const Bucket4Tab& T, uint32_t n_ovf, const uint2* pivot_pairs, uint32_t pivot_nnz, uint2 kv,
-                                                 bool pending, float& acc) {
+__device__ __forceinline__ void bucket4_overflow(const Bucket4Tab& T, uint32_t n_ovf, const Pairs& pivot_pairs, uint2 kv, bool pending, float& acc) {
     if (n_ovf <= T.ovf_cap) {
         for (uint32_t i = 0; i < n_ovf; i++) {
             const uint2 o = T.ovf[i];
             if (pending && o.x == kv.x) acc = fmaf(__uint_as_float(kv.y), __uint_as_float(o.y), acc);
         }
     } else {
-        for (uint32_t i = 0; i < pivot_nnz; i++) {
+        for (uint32_t i = 0; i < pivot_pairs.nnz; i++) {
             const uint2 o = pivot_pairs[i];
             if (pending && o.x == kv.x) acc = fmaf(__uint_as_float(kv.y), __uint_as_float(o.y), acc);
         }
@@ -520,33 +566,36 @@ __device__ __forceinline__ void bucket4_overflow(const Bucket4Tab& T, uint32_t n
 }
 
 // Per-lane part of stage 1 against a document pivot (all paths on).
-__device__ __forceinline__ float doc_sparse_probe(const PendingEval& p, const Bucket4Tab& T, uint32_t n_ovf, const uint2* pivot_pairs,
-                                                  uint32_t pivot_nnz) {
+__device__ __forceinline__ float doc_sparse_probe(const CorpusView& C, const PendingEval& p, const Bucket4Tab& T, uint32_t n_ovf,
+                                                  const Pairs& pivot_pairs) {
     const int lane = lane_id();
     float acc = 0.f;
     const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
     const bool in0 = j0 < p.end, in1 = j1 < p.end, in2 = j2 < p.end;
-    const uint4* b0 = T.b + 2 * term_hash(p.kv0.x, T.mask);
-    const uint4* b1 = T.b + 2 * term_hash(p.kv1.x, T.mask);
-    const uint4* b2 = T.b + 2 * term_hash(p.kv2.x, T.mask);
+    const uint2 kv0 = make_uint2(p.kv0.x | pair_flag(C.narrow, p.ns, j0), p.kv0.y);
+    const uint2 kv1 = make_uint2(p.kv1.x | pair_flag(C.narrow, p.ns, j1), p.kv1.y);
+    const uint2 kv2 = make_uint2(p.kv2.x | pair_flag(C.narrow, p.ns, j2), p.kv2.y);
+    const uint4* b0 = T.b + 2 * term_hash(kv0.x, T.mask);
+    const uint4* b1 = T.b + 2 * term_hash(kv1.x, T.mask);
+    const uint4* b2 = T.b + 2 * term_hash(kv2.x, T.mask);
     uint4 e00 = b0[0], e01 = b0[1], e10 = b1[0], e11 = b1[1], e20 = b2[0], e21 = b2[1];
     // keep the six reads together: nothing below may be scheduled between them
     asm volatile("" : "+v"(e00.x), "+v"(e01.x), "+v"(e10.x), "+v"(e11.x), "+v"(e20.x), "+v"(e21.x));
-    const bool f0 = bucket4_match(e00, e01, p.kv0, in0, acc);
-    const bool f1 = bucket4_match(e10, e11, p.kv1, in1, acc);
-    const bool f2 = bucket4_match(e20, e21, p.kv2, in2, acc);
+    const bool f0 = bucket4_match(e00, e01, kv0, in0, acc);
+    const bool f1 = bucket4_match(e10, e11, kv1, in1, acc);
+    const bool f2 = bucket4_match(e20, e21, kv2, in2, acc);
     if (n_ovf) {
-        bucket4_overflow(T, n_ovf, pivot_pairs, pivot_nnz, p.kv0, in0 && !f0, acc);
-        bucket4_overflow(T, n_ovf, pivot_pairs, pivot_nnz, p.kv1, in1 && !f1, acc);
-        bucket4_overflow(T, n_ovf, pivot_pairs, pivot_nnz, p.kv2, in2 && !f2, acc);
+        bucket4_overflow(T, n_ovf, pivot_pairs, kv0, in0 && !f0, acc);
+        bucket4_overflow(T, n_ovf, pivot_pairs, kv1, in1 && !f1, acc);
+        bucket4_overflow(T, n_ovf, pivot_pairs, kv2, in2 && !f2, acc);
     }
     if (p.begin + 3 * WAVE < p.end) { // rows with more than 192 pairs
-        const uint2* sp = reinterpret_cast<const uint2*>(p.rec + DENSE_BYTES);
+        const Pairs sp = record_pairs(C, p.rec, p.ns, p.nb);
         for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) {
             const uint2 kv = sp[j];
             const uint4* bb = T.b + 2 * term_hash(kv.x, T.mask);
             const bool f = bucket4_match(bb[0], bb[1], kv, true, acc);
-            if (n_ovf) bucket4_overflow(T, n_ovf, pivot_pairs, pivot_nnz, kv, !f, acc);
+            if (n_ovf) bucket4_overflow(T, n_ovf, pivot_pairs, kv, !f, acc);
         }
     }
     return acc;

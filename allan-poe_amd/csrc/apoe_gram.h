@@ -86,16 +86,44 @@ __device__ __forceinline__ void gram_dense_store(float* G, int tile, int lane, c
 constexpr int GRAM_CHUNKS = 5;  // 64-pair chunks of a row kept in registers (320 pairs)
 constexpr int GRAM_OVF = 32;    // overflow entries per pivot table
 
-struct RowPairs {
+struct RowPairs { // raw pairs: the consumer adds pair_flag()
     uint2 kv[GRAM_CHUNKS];
 };
 
-__device__ __forceinline__ void row_pairs_load(RowPairs& r, const uint2* sp, uint32_t nnz, int lane) {
+__device__ __forceinline__ void row_pairs_load(RowPairs& r, const Pairs& sp, int lane) {
 #pragma unroll
     for (int c = 0; c < GRAM_CHUNKS; c++) {
         const uint32_t j = c * WAVE + lane;
-        r.kv[c] = j < nnz ? sp[j] : make_uint2(EMPTY, 0u);
+        r.kv[c] = j < sp.nnz ? sp.raw(j) : make_uint2(EMPTY, 0u);
     }
+}
+// Chunk c of a prefetched row as (term | path bit, value); a padding lane gives (EMPTY, 0): value 0
+// adds nothing, and key EMPTY matches only empty slots, whose value is 0.
+__device__ __forceinline__ uint2 row_pairs_get(const RowPairs& r, int c, uint32_t narrow, uint32_t ns, int lane) {
+    uint2 kv = r.kv[c];
+    if (kv.x == EMPTY) kv.y = 0u;
+    else kv.x |= pair_flag(narrow, ns, c * WAVE + lane);
+    return kv;
+}
+
+// The 64 gathered rows are kept in LDS as the address of the pair array and one word with
+// nnz (low half) and nnz_s (high half); nnz <= 2 * DESC_NNZ_MAX fits 16 bits.
+__device__ __forceinline__ void gram_rows_gather(const CorpusView& C, const uint32_t* ids, uint32_t m, unsigned long long* rowptr, uint32_t* rownnz,
+                                                 int tid, int nthreads) {
+    for (uint32_t i = tid; i < m; i += nthreads) {
+        const uint64_t d = C.desc[ids[i]];
+        rowptr[i] = (unsigned long long)(C.recs + desc_off(d) * 16 + DENSE_BYTES);
+        rownnz[i] = (desc_nnz_s(d) + desc_nnz_b(d)) | (desc_nnz_s(d) << 16);
+    }
+}
+__device__ __forceinline__ Pairs gram_row(const CorpusView& C, const unsigned long long* rowptr, const uint32_t* rownnz, uint32_t i) {
+    Pairs p;
+    p.base = reinterpret_cast<const char*>(rowptr[i]);
+    const uint32_t w = rownnz[i];
+    p.nnz = w & 0xFFFFu;
+    p.ns = w >> 16;
+    p.narrow = C.narrow;
+    return p;
 }
 
 struct Slots3 {
@@ -121,11 +149,7 @@ __device__ __forceinline__ void gram_sparse_64(const CorpusView& C, const uint32
     const uint32_t mask = slots - 1;
     const int wave = tid / WAVE, lane = tid & (WAVE - 1), nwaves = nthreads / WAVE;
     uint2* ovf = tabs + (size_t)T * slots;
-    for (uint32_t i = tid; i < m; i += nthreads) {
-        const uint64_t d = C.desc[ids[i]];
-        rowptr[i] = (unsigned long long)(C.recs + desc_off(d) * 16 + DENSE_BYTES);
-        rownnz[i] = desc_nnz_s(d) + desc_nnz_b(d);
-    }
+    gram_rows_gather(C, ids, m, rowptr, rownnz, tid, nthreads);
     __syncthreads();
     for (uint32_t a0 = 0; a0 + 1 < m; a0 += T) {
         const uint32_t nt = min((uint32_t)T, m - 1 - a0); // the last row is never a pivot
@@ -133,8 +157,8 @@ __device__ __forceinline__ void gram_sparse_64(const CorpusView& C, const uint32
         if (tid < T) ovf_cnt[tid] = 0;
         __syncthreads();
         for (uint32_t t = 0; t < nt; t++) {
-            const uint2* sp = reinterpret_cast<const uint2*>(rowptr[a0 + t]);
-            const uint32_t nnz = rownnz[a0 + t];
+            const Pairs sp = gram_row(C, rowptr, rownnz, a0 + t);
+            const uint32_t nnz = sp.nnz;
             uint2* tab = tabs + (size_t)t * slots;
             for (uint32_t j = tid; j < nnz; j += nthreads) {
                 const uint2 kv = sp[j];
@@ -159,12 +183,12 @@ __device__ __forceinline__ void gram_sparse_64(const CorpusView& C, const uint32
         for (int t = 0; t < T; t++) novf[t] = uniform(min(ovf_cnt[t], (uint32_t)GRAM_OVF));
         uint32_t b = a0 + 1 + wave;
         RowPairs cur;
-        if (b < m) row_pairs_load(cur, reinterpret_cast<const uint2*>(rowptr[b]), rownnz[b], lane);
+        if (b < m) row_pairs_load(cur, gram_row(C, rowptr, rownnz, b), lane);
         while (b < m) {
             const uint32_t bn = b + nwaves;
             RowPairs nxt;
-            if (bn < m) row_pairs_load(nxt, reinterpret_cast<const uint2*>(rowptr[bn]), rownnz[bn], lane);
-            const uint32_t nnz = rownnz[b];
+            if (bn < m) row_pairs_load(nxt, gram_row(C, rowptr, rownnz, bn), lane);
+            const uint32_t nnz = rownnz[b] & 0xFFFFu, ns_b = rownnz[b] >> 16;
             const uint32_t np = min(nt, b - a0); // pivots a0 .. a0+np-1 precede row b
             float acc[T];
 #pragma unroll
@@ -201,13 +225,11 @@ __device__ __forceinline__ void gram_sparse_64(const CorpusView& C, const uint32
 #pragma unroll
             for (int c = 0; c < GRAM_CHUNKS; c++) {
                 if (c * WAVE < (int)nnz) { // wave-uniform
-                    uint2 kv = cur.kv[c];
-                    if (kv.x == EMPTY) kv.y = 0u; // padding lane: value 0 adds nothing, key EMPTY matches only empty slots whose value is 0
-                    lookup(kv);
+                    lookup(row_pairs_get(cur, c, C.narrow, ns_b, lane));
                 }
             }
             if (nnz > GRAM_CHUNKS * WAVE) { // rows longer than the register window
-                const uint2* sp = reinterpret_cast<const uint2*>(rowptr[b]);
+                const Pairs sp = gram_row(C, rowptr, rownnz, b);
                 for (uint32_t j0 = GRAM_CHUNKS * WAVE; j0 < nnz; j0 += WAVE) {
                     const uint32_t j = j0 + lane;
                     lookup(j < nnz ? sp[j] : make_uint2(EMPTY, 0u));
@@ -276,11 +298,7 @@ __device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uin
     const float4* ovf_val4 = reinterpret_cast<const float4*>(ovf_val);
     const uint32_t bmask = slots / GU_BUCKET - 1;
     const int wave = (int)uniform(tid / WAVE), lane = tid & (WAVE - 1), nwaves = nthreads / WAVE;
-    for (uint32_t i = tid; i < m; i += nthreads) {
-        const uint64_t d = C.desc[ids[i]];
-        rowptr[i] = (unsigned long long)(C.recs + desc_off(d) * 16 + DENSE_BYTES);
-        rownnz[i] = desc_nnz_s(d) + desc_nnz_b(d);
-    }
+    gram_rows_gather(C, ids, m, rowptr, rownnz, tid, nthreads);
     __syncthreads();
     uint32_t a0 = 0;
     while (a0 + 1 < m) { // the last row is never a pivot
@@ -295,8 +313,8 @@ __device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uin
             // wave w scatters pivot (w % GU_T); waves w and w + GU_T share a pivot
             const uint32_t t = (uint32_t)wave % GU_T;
             if (t < nt) {
-                const uint2* sp = reinterpret_cast<const uint2*>(rowptr[a0 + t]);
-                const uint32_t nnz = rownnz[a0 + t];
+                const Pairs sp = gram_row(C, rowptr, rownnz, a0 + t);
+                const uint32_t nnz = sp.nnz;
                 const uint32_t step = (uint32_t)(nwaves / GU_T > 0 ? nwaves / GU_T : 1) * WAVE;
                 for (uint32_t j = (uint32_t)(wave / GU_T) * WAVE + lane; j < nnz; j += step) {
                     const uint2 kv = sp[j];
@@ -333,12 +351,12 @@ __device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uin
         const uint32_t novf = uniform(min(ctl2[0], (uint32_t)GU_OVF));
         uint32_t b = a0 + 1 + wave;
         RowPairs cur;
-        if (b < m) row_pairs_load(cur, reinterpret_cast<const uint2*>(rowptr[b]), rownnz[b], lane);
+        if (b < m) row_pairs_load(cur, gram_row(C, rowptr, rownnz, b), lane);
         while (b < m) {
             const uint32_t bn = b + nwaves;
             RowPairs nxt;
-            if (bn < m) row_pairs_load(nxt, reinterpret_cast<const uint2*>(rowptr[bn]), rownnz[bn], lane);
-            const uint32_t nnz = uniform(rownnz[b]);
+            if (bn < m) row_pairs_load(nxt, gram_row(C, rowptr, rownnz, bn), lane);
+            const uint32_t nnz = uniform(rownnz[b] & 0xFFFFu), ns_b = uniform(rownnz[b] >> 16);
             const uint32_t np = min(nt, b - a0); // pivots a0 .. a0+np-1 precede row b
             float acc[GU_T];
 #pragma unroll
@@ -369,8 +387,7 @@ __device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uin
                 uint4 k0[3], k1[3];
 #pragma unroll
                 for (int c = 0; c < 3; c++) {
-                    kv[c] = cur.kv[c];
-                    if (kv[c].x == EMPTY) kv[c].y = 0u; // padding lane: matches an empty key at most, and adds 0 * value
+                    kv[c] = row_pairs_get(cur, c, C.narrow, ns_b, lane);
                     bk[c] = gu_hash(kv[c].x, bmask);
                     k0[c] = keys4[bk[c] * 2];
                     k1[c] = keys4[bk[c] * 2 + 1];
@@ -410,9 +427,9 @@ __device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uin
             };
 #pragma unroll
             for (int c = 3; c < GRAM_CHUNKS; c++)
-                if (c * WAVE < (int)nnz) lookup(cur.kv[c]); // wave-uniform
+                if (c * WAVE < (int)nnz) lookup(row_pairs_get(cur, c, C.narrow, ns_b, lane)); // wave-uniform
             if (nnz > GRAM_CHUNKS * WAVE) { // rows longer than the register window
-                const uint2* sp = reinterpret_cast<const uint2*>(rowptr[b]);
+                const Pairs sp = gram_row(C, rowptr, rownnz, b);
                 for (uint32_t j0 = GRAM_CHUNKS * WAVE; j0 < nnz; j0 += WAVE) {
                     const uint32_t j = j0 + lane;
                     lookup(j < nnz ? sp[j] : make_uint2(EMPTY, 0u));

@@ -91,10 +91,11 @@ struct apoe_corpus {
     apoe_ctx* ctx = nullptr;
     uint32_t n = 0, dim = 0, max_nnz_s = 0, max_nnz_b = 0;
     uint64_t rec_bytes = 0;
+    bool narrow = false; // pair format of the records (6 instead of 8 bytes a pair when every term id is below 65536)
     apoe::DevBuf<uint64_t> desc;
     apoe::DevBuf<char> recs;
     apoe::DevBuf<float> dnorm;
-    apoe::CorpusView view() const { return apoe::CorpusView{desc.p, recs.p, dnorm.p, n}; }
+    apoe::CorpusView view() const { return apoe::CorpusView{desc.p, recs.p, dnorm.p, n, narrow ? 1u : 0u}; }
 };
 
 struct apoe_queries {
@@ -144,7 +145,9 @@ int copy_out(apoe_ctx* ctx, void* dst_any, const void* src_dev, size_t bytes);
 
 // Kernel launchers (one per .hip file).
 int launch_pack(apoe_ctx* ctx, uint32_t n, const float* dense, const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,
-                const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs, float* dnorm);
+                const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs, float* dnorm,
+                bool narrow);
+int launch_max_u32(apoe_ctx* ctx, const uint32_t* a_dev, size_t n, uint32_t* out_dev);
 int launch_distance_batch(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const float* w3, const uint32_t* ids_dev,
                           uint32_t M, float* out_dev);
 int launch_distance_pairs(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale, const uint32_t* a_dev, const uint32_t* b_dev,

@@ -151,34 +151,48 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
     c->ctx = ctx;
     c->n = n;
     c->dim = dim;
-    std::vector<uint64_t> desc(n);
-    uint64_t off16 = 0;
     for (uint32_t i = 0; i < n; i++) {
         const uint32_t ns = hs[i + 1] - hs[i], nb = hb[i + 1] - hb[i];
         APOE_REQUIRE(ns <= DESC_NNZ_MAX && nb <= DESC_NNZ_MAX, "row %u has %u/%u sparse/bm25 terms; at most %u each are supported", i, ns, nb,
                      DESC_NNZ_MAX);
         c->max_nnz_s = std::max(c->max_nnz_s, ns);
         c->max_nnz_b = std::max(c->max_nnz_b, nb);
-        desc[i] = make_desc(off16, ns, nb);
-        off16 += (DENSE_BYTES + 8ull * (ns + nb) + 15) / 16;
     }
-    APOE_REQUIRE(off16 < (1ull << DESC_OFF_BITS), "corpus of %llu bytes exceeds the record address range", (unsigned long long)off16 * 16);
-    c->rec_bytes = off16 * 16;
-    APOE_TRY(c->desc.alloc(n));
-    APOE_TRY(c->recs.alloc(c->rec_bytes));
-    APOE_TRY(c->dnorm.alloc(n));
-    APOE_TRY(copy_in(ctx, c->desc.p, desc.data(), n * sizeof(uint64_t)));
     {
         DevInput<float> d_dense, d_sval, d_bval;
         DevInput<uint32_t> d_soff, d_sidx, d_boff, d_bidx;
+        APOE_TRY(d_sidx.init(ctx, s_idx, hs[n]));
+        APOE_TRY(d_bidx.init(ctx, b_idx, hb[n]));
+        // the pair format follows from the largest term id of either path
+        DevBuf<uint32_t> d_max;
+        uint32_t max_term = 0;
+        APOE_TRY(d_max.alloc(1));
+        APOE_TRY(copy_in(ctx, d_max.p, &max_term, sizeof(uint32_t)));
+        APOE_TRY(launch_max_u32(ctx, d_sidx.p, hs[n], d_max.p));
+        APOE_TRY(launch_max_u32(ctx, d_bidx.p, hb[n], d_max.p));
+        APOE_TRY(copy_out(ctx, &max_term, d_max.p, sizeof(uint32_t)));
+        APOE_REQUIRE(max_term < BM25_BIT, "term id %u does not fit 31 bits", max_term);
+        c->narrow = max_term < 65536u;
+        std::vector<uint64_t> desc(n);
+        uint64_t off16 = 0;
+        for (uint32_t i = 0; i < n; i++) {
+            const uint32_t ns = hs[i + 1] - hs[i], nb = hb[i + 1] - hb[i];
+            desc[i] = make_desc(off16, ns, nb);
+            off16 += record_units(ns + nb, c->narrow);
+        }
+        APOE_REQUIRE(off16 < (1ull << DESC_OFF_BITS), "corpus of %llu bytes exceeds the record address range", (unsigned long long)off16 * 16);
+        c->rec_bytes = off16 * 16;
+        APOE_TRY(c->desc.alloc(n));
+        APOE_TRY(c->recs.alloc(c->rec_bytes));
+        APOE_TRY(c->dnorm.alloc(n));
+        APOE_TRY(copy_in(ctx, c->desc.p, desc.data(), n * sizeof(uint64_t)));
         APOE_TRY(d_dense.init(ctx, dense, (size_t)n * dim));
         APOE_TRY(d_soff.init(ctx, s_off, n + 1));
-        APOE_TRY(d_sidx.init(ctx, s_idx, hs[n]));
         APOE_TRY(d_sval.init(ctx, s_val, hs[n]));
         APOE_TRY(d_boff.init(ctx, b_off, n + 1));
-        APOE_TRY(d_bidx.init(ctx, b_idx, hb[n]));
         APOE_TRY(d_bval.init(ctx, b_val, hb[n]));
-        APOE_TRY(launch_pack(ctx, n, d_dense.p, d_soff.p, d_sidx.p, d_sval.p, d_boff.p, d_bidx.p, d_bval.p, c->desc.p, c->recs.p, c->dnorm.p));
+        APOE_TRY(launch_pack(ctx, n, d_dense.p, d_soff.p, d_sidx.p, d_sval.p, d_boff.p, d_bidx.p, d_bval.p, c->desc.p, c->recs.p, c->dnorm.p,
+                             c->narrow));
         APOE_HIP(hipStreamSynchronize(ctx->stream));
     }
     *out = c.release();
@@ -195,6 +209,8 @@ int apoe_corpus_info(const apoe_corpus* c, uint32_t* info4) {
     info4[3] = c->max_nnz_b;
     return APOE_OK;
 }
+
+uint32_t apoe_corpus_pair_bytes(const apoe_corpus* c) { return c ? (c->narrow ? 6u : 8u) : 0u; }
 
 uint64_t apoe_corpus_bytes(const apoe_corpus* c) { return c ? c->rec_bytes + (uint64_t)c->n * 12 : 0; }
 

@@ -3,12 +3,30 @@
 
 namespace apoe {
 
-// One workgroup per document: dense row, then SPLADE pairs, then BM25 pairs with
-// the path bit set in the term key, written as one contiguous record.
+// Largest value of an index array (decides whether the corpus can use narrow pairs).
+__global__ __launch_bounds__(256) void max_u32_kernel(const uint32_t* __restrict__ a, size_t n, uint32_t* out) {
+    uint32_t m = 0;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) m = max(m, a[i]);
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) m = max(m, (uint32_t)__shfl_xor(m, o, WAVE));
+    if (lane_id() == 0 && m) atomicMax(out, m);
+}
+
+int launch_max_u32(apoe_ctx* ctx, const uint32_t* a_dev, size_t n, uint32_t* out_dev) { // *out_dev must hold 0 (or a running maximum)
+    if (n == 0) return APOE_OK;
+    const uint32_t grid = (uint32_t)std::min<size_t>((n + 255) / 256, 4096);
+    max_u32_kernel<<<grid, 256, 0, ctx->stream>>>(a_dev, n, out_dev);
+    APOE_HIP(hipGetLastError());
+    return APOE_OK;
+}
+
+// One workgroup per document: dense row, then SPLADE pairs, then BM25 pairs, written as one
+// contiguous record in the wide (path bit in the term key) or the narrow pair format.
 __global__ __launch_bounds__(256) void pack_kernel(uint32_t n, const float* __restrict__ dense, const uint32_t* __restrict__ s_off,
                                                    const uint32_t* __restrict__ s_idx, const float* __restrict__ s_val,
                                                    const uint32_t* __restrict__ b_off, const uint32_t* __restrict__ b_idx,
-                                                   const float* __restrict__ b_val, const uint64_t* __restrict__ desc, char* recs, float* dnorm) {
+                                                   const float* __restrict__ b_val, const uint64_t* __restrict__ desc, char* recs, float* dnorm,
+                                                   uint32_t narrow) {
     __shared__ float part[4];
     for (uint32_t doc = blockIdx.x; doc < n; doc += gridDim.x) {
         const uint64_t d = desc[doc];
@@ -26,21 +44,37 @@ __global__ __launch_bounds__(256) void pack_kernel(uint32_t n, const float* __re
         if (lane_id() == 0) part[threadIdx.x / WAVE] = sq;
         __syncthreads();
         if (threadIdx.x == 0) dnorm[doc] = sqrtf(part[0] + part[1] + part[2] + part[3]);
-        uint2* sp = reinterpret_cast<uint2*>(rec + DENSE_BYTES);
-        const uint32_t s0 = s_off[doc], ns = desc_nnz_s(d), b0 = b_off[doc], nb = desc_nnz_b(d);
-        for (uint32_t j = threadIdx.x; j < ns; j += blockDim.x) sp[j] = make_uint2(s_idx[s0 + j], __float_as_uint(s_val[s0 + j]));
-        for (uint32_t j = threadIdx.x; j < nb; j += blockDim.x)
-            sp[ns + j] = make_uint2(b_idx[b0 + j] | BM25_BIT, __float_as_uint(b_val[b0 + j]));
-        // zero the alignment tail so that a record never holds stale bytes
-        if (((ns + nb) & 1u) && threadIdx.x == 0) sp[ns + nb] = make_uint2(EMPTY, 0u);
+        const uint32_t s0 = s_off[doc], ns = desc_nnz_s(d), b0 = b_off[doc], nb = desc_nnz_b(d), nnz = ns + nb;
+        if (narrow) {
+            float* vals = reinterpret_cast<float*>(rec + DENSE_BYTES);
+            uint16_t* keys = reinterpret_cast<uint16_t*>(rec + DENSE_BYTES + 4 * (size_t)nnz);
+            for (uint32_t j = threadIdx.x; j < ns; j += blockDim.x) {
+                vals[j] = s_val[s0 + j];
+                keys[j] = (uint16_t)s_idx[s0 + j];
+            }
+            for (uint32_t j = threadIdx.x; j < nb; j += blockDim.x) {
+                vals[ns + j] = b_val[b0 + j];
+                keys[ns + j] = (uint16_t)b_idx[b0 + j];
+            }
+            // fill the alignment tail so that a record never holds stale bytes
+            const uint32_t tail = (uint32_t)(record_units(nnz, true) * 16 - DENSE_BYTES - 6 * (size_t)nnz) / 2;
+            if (threadIdx.x < tail) keys[nnz + threadIdx.x] = 0xFFFFu;
+        } else {
+            uint2* sp = reinterpret_cast<uint2*>(rec + DENSE_BYTES);
+            for (uint32_t j = threadIdx.x; j < ns; j += blockDim.x) sp[j] = make_uint2(s_idx[s0 + j], __float_as_uint(s_val[s0 + j]));
+            for (uint32_t j = threadIdx.x; j < nb; j += blockDim.x)
+                sp[ns + j] = make_uint2(b_idx[b0 + j] | BM25_BIT, __float_as_uint(b_val[b0 + j]));
+            if ((nnz & 1u) && threadIdx.x == 0) sp[nnz] = make_uint2(EMPTY, 0u);
+        }
     }
 }
 
 int launch_pack(apoe_ctx* ctx, uint32_t n, const float* dense, const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,
-                const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs, float* dnorm) {
+                const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs, float* dnorm,
+                bool narrow) {
     uint32_t grid = n < 65536u * 16u ? n : 65536u * 16u;
     if (grid == 0) return APOE_OK;
-    pack_kernel<<<grid, 256, 0, ctx->stream>>>(n, dense, s_off, s_idx, s_val, b_off, b_idx, b_val, desc, recs, dnorm);
+    pack_kernel<<<grid, 256, 0, ctx->stream>>>(n, dense, s_off, s_idx, s_val, b_off, b_idx, b_val, desc, recs, dnorm, narrow ? 1u : 0u);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
 }
@@ -111,7 +145,7 @@ __global__ __launch_bounds__(64) void distance_pairs_kernel(CorpusView C, float 
             const char* rec = C.recs + desc_off(d) * 16;
             PivotDense pv;
             pivot_dense_load(pv, reinterpret_cast<const float*>(rec), 1.0f);
-            pivot_terms_from_record(tab, mask, rec, desc_nnz_s(d) + desc_nnz_b(d), lane, WAVE);
+            pivot_terms_from_record(tab, mask, record_pairs(C, d), lane, WAVE);
             __syncthreads();
             EvalOut e = eval_wave(C, ib, pv, tab, mask, PATH_DENSE | PATH_SPARSE | PATH_BM25, dense_mul);
             dist = 1.0f - e.ip;
@@ -148,9 +182,8 @@ __global__ __launch_bounds__(256) void norms_kernel(CorpusView C, float dense_mu
             acc += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
         }
         acc *= dense_mul;
-        const uint2* sp = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
-        const uint32_t nnz = desc_nnz_s(d) + desc_nnz_b(d);
-        for (uint32_t j = lane; j < nnz; j += WAVE) {
+        const Pairs sp = record_pairs(C, d);
+        for (uint32_t j = lane; j < sp.nnz; j += WAVE) {
             float v = __uint_as_float(sp[j].y);
             acc = fmaf(v, v, acc);
         }

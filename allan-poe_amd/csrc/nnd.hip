@@ -102,9 +102,11 @@ struct NndLds {
 // duplicates and ids already in u's list, evaluate the rest against u, merge those
 // closer than u's current worst into the list, and register u with every member of
 // the merged list when the list changed.
+template <bool NARROW> // the pair format of the corpus as a compile-time constant: no branch at the loads
 __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, float dense_mul, uint32_t K, uint32_t* ids, float* dist,
                                                                   unsigned long long* rev, uint32_t* rev_cnt, uint32_t term_slots,
                                                                   uint32_t seen_slots, unsigned long long* inserted) {
+    C.narrow = NARROW ? 1u : 0u;
     extern __shared__ __align__(16) char smem[];
     const NndLds L(term_slots, seen_slots, K);
     // the dedupe set is dead once the candidates are gathered: the pivot's dense row and the overflow
@@ -180,12 +182,12 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
     // pivot = u: dense row into LDS (float4 number l + 64*i belongs to lane l), terms into the bucket table
     const uint64_t du = C.desc[u];
     const char* rec = C.recs + desc_off(du) * 16;
-    const uint32_t u_nnz = desc_nnz_s(du) + desc_nnz_b(du);
+    const Pairs u_pairs = record_pairs(C, du);
     {
         const float4* src = reinterpret_cast<const float4*>(rec);
         for (uint32_t i = tid; i < DIM / 4; i += NND_THREADS) qd[i] = src[i];
     }
-    bucket4_terms_from_record(T, rec, u_nnz, tid, NND_THREADS);
+    bucket4_terms_from_record(T, u_pairs, tid, NND_THREADS);
     __syncthreads();
 
     // 4. distances; only those below the current worst matter (step 5), so a candidate whose
@@ -198,7 +200,6 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
     const float thr = worst < INF_DIS ? worst : __builtin_inff();
     const float pv_norm = pivot_dense_norm_lds(qd);
     const uint32_t n_ovf = uniform(ctl[8]);
-    const uint2* u_pairs = reinterpret_cast<const uint2*>(rec + DENSE_BYTES);
     for (uint32_t c0 = 0; c0 * NW < n_cand; c0 += WAVE) {
         // lane l fetches descriptor and dense norm of the wave's (c0 + l)-th candidate
         uint64_t my_desc = 0;
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
             for (int b = 0; b < NND_EVAL_BATCH; b++) {
                 const uint32_t jj = wave + (c0 + t + b) * NW;
                 acc[b] = 0.f;
-                if (t + b < WAVE && jj < n_cand) acc[b] = doc_sparse_probe(pe[b], T, n_ovf, u_pairs, u_nnz);
+                if (t + b < WAVE && jj < n_cand) acc[b] = doc_sparse_probe(C, pe[b], T, n_ovf, u_pairs);
             }
 #pragma unroll
             for (int b = 0; b < NND_EVAL_BATCH; b++) {
@@ -356,9 +357,10 @@ int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted) {
     APOE_REQUIRE(L.total <= 64 * 1024, "NN-Descent needs %u bytes of LDS (rows with up to %u sparse terms)", L.total,
                  g->corpus->max_nnz_s + g->corpus->max_nnz_b);
     APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), ctx->stream)); // [0] inserted; [2], [3] accumulate over the build
-    APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_iterate_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
-    nnd_iterate_kernel<<<g->n, NND_THREADS, L.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->K, g->ids.p, g->dist.p,
-                                                                    g->rev.p, g->rev_cnt.p, term_slots, seen_slots, g->counter.p);
+    auto kernel = g->corpus->narrow ? &nnd_iterate_kernel<true> : &nnd_iterate_kernel<false>;
+    APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
+    kernel<<<g->n, NND_THREADS, L.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->K, g->ids.p, g->dist.p, g->rev.p,
+                                                        g->rev_cnt.p, term_slots, seen_slots, g->counter.p);
     APOE_HIP(hipGetLastError());
     if (inserted) {
         unsigned long long h = 0;

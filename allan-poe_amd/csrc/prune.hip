@@ -107,10 +107,10 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
     }
     {   // u's BM25 terms
         const uint64_t du = C.desc[u];
-        const uint2* sp = reinterpret_cast<const uint2*>(C.recs + desc_off(du) * 16 + DENSE_BYTES);
+        const Pairs sp = record_pairs(C, du);
         const uint32_t ns = desc_nnz_s(du), nb = desc_nnz_b(du);
         for (uint32_t j = tid; j < nb; j += PR_THREADS) {
-            const uint32_t key = sp[ns + j].x;
+            const uint32_t key = sp.key(ns + j);
             uint32_t h = term_hash(key, umask);
             while (true) {
                 const uint32_t old = atomicCAS(&uset[h], EMPTY, key);
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
         const char* rec = C.recs + desc_off(dc) * 16;
         PivotDense pv;
         pivot_dense_load(pv, reinterpret_cast<const float*>(rec), 1.0f);
-        pivot_terms_from_record(tab, tmask, rec, desc_nnz_s(dc) + desc_nnz_b(dc), tid, PR_THREADS);
+        pivot_terms_from_record(tab, tmask, record_pairs(C, dc), tid, PR_THREADS);
         __syncthreads();
         const uint32_t n_sel = ctl[PC_NSEL];
         const float norm_c = norms[c];
@@ -280,7 +280,7 @@ struct GramPruneLds {
 // row's overlap with the centre node's BM25 terms becomes a bit mask, and the sequential
 // RNG-IP selection with its keyword flags then runs on LDS only:
 //   <c,s> = G[c][s];   flag(c,s) = (R[s] & ~R[c]) != 0   with R[x] = bm25(x) ∩ bm25(u).
-template <int NT>
+template <int NT, bool NARROW>
 __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dense_mul, const float* __restrict__ norms,
                                                                 const uint32_t* __restrict__ ids, const float* __restrict__ dist,
                                                                 uint32_t d, uint32_t* fwd, uint32_t* det_out, uint32_t* cnt_out,
@@ -288,6 +288,7 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
                                                                 uint32_t umap_slots, uint32_t map_slots, uint32_t words,
                                                                 uint32_t union_slots, unsigned long long* gfail) {
     constexpr uint32_t K = GRAM_ROWS;
+    C.narrow = NARROW ? 1u : 0u; // the pair format as a compile-time constant: no branch at the loads
     extern __shared__ __align__(16) char smem[];
     const GramPruneLds L(term_slots, tgroup, umap_slots, map_slots, words, union_slots);
     float* G = reinterpret_cast<float*>(smem + L.G);
@@ -340,10 +341,10 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     }
     {   // u's BM25 terms -> index
         const uint64_t du = C.desc[u];
-        const uint2* sp = reinterpret_cast<const uint2*>(C.recs + desc_off(du) * 16 + DENSE_BYTES);
+        const Pairs sp = record_pairs(C, du);
         const uint32_t ns = desc_nnz_s(du), nb = desc_nnz_b(du);
         for (uint32_t j = tid; j < nb; j += NT) {
-            const uint32_t key = sp[ns + j].x;
+            const uint32_t key = sp.key(ns + j);
             uint32_t h = term_hash(key, umask);
             while (true) {
                 const uint32_t old = atomicCAS(&umap[h].x, EMPTY, key);
@@ -370,10 +371,10 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     // R[r] = bits of u's BM25 terms that row r holds too: one wave per row, lanes over its BM25 pairs
     for (uint32_t r = wave; r < m; r += NT / WAVE) {
         const uint64_t dr = C.desc[nb_id[r]];
-        const uint2* sp = reinterpret_cast<const uint2*>(C.recs + desc_off(dr) * 16 + DENSE_BYTES);
+        const Pairs sp = record_pairs(C, dr);
         const uint32_t ns = desc_nnz_s(dr), nb = desc_nnz_b(dr);
         for (uint32_t j = lane; j < nb; j += WAVE) {
-            const uint32_t key = sp[ns + j].x;
+            const uint32_t key = sp.key(ns + j);
             uint32_t h = term_hash(key, umask);
             while (true) {
                 const uint2 e = umap[h];
@@ -623,16 +624,17 @@ int launch_prune(apoe_knn* g, uint32_t degree) {
     const uint32_t lds_budget = (uint32_t)std::min<size_t>(ctx->lds_per_block, 80 * 1024);
     uint32_t tgroup = GramPruneLds(gram_slots, 8, uset_slots, map_slots, words, 0).total <= lds_budget ? 8 : 4;
     // one union table for GU_T pivots when it fits: 2.5 slots per term of an average group, and room for the longest row alone
-    const double mean_nnz = g->n ? ((double)g->corpus->rec_bytes / g->n - DENSE_BYTES) / 8.0 : 0.0;
+    const double mean_nnz = g->n ? ((double)g->corpus->rec_bytes / g->n - DENSE_BYTES) / (g->corpus->narrow ? 6.0 : 8.0) : 0.0;
     uint32_t union_slots = std::max(next_pow2((uint32_t)std::ceil(2.5 * GU_T * mean_nnz)), std::max(512u, gram_slots));
     if (GramPruneLds(gram_slots, tgroup, uset_slots, map_slots, words, union_slots).total > lds_budget) union_slots = 0;
     const GramPruneLds GL(gram_slots, tgroup, uset_slots, map_slots, words, union_slots);
     if (g->K == GRAM_ROWS && GL.total <= lds_budget && !g->force_sequential_prune) {
         APOE_HIP(hipMemsetAsync(g->counter.p + 1, 0, sizeof(unsigned long long), ctx->stream));
-        APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&prune_gram_kernel<GRAM_THREADS>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GL.total));
-        prune_gram_kernel<GRAM_THREADS><<<g->n, GRAM_THREADS, GL.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->norms.p, g->ids.p,
-                                                                      g->dist.p, degree, g->fwd.p, g->det.p, g->cnt.p, g->kw.p, gram_slots,
-                                                                      tgroup, uset_slots, map_slots, words, union_slots, g->counter.p + 1);
+        auto kernel = g->corpus->narrow ? &prune_gram_kernel<GRAM_THREADS, true> : &prune_gram_kernel<GRAM_THREADS, false>;
+        APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GL.total));
+        kernel<<<g->n, GRAM_THREADS, GL.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->norms.p, g->ids.p, g->dist.p, degree,
+                                                              g->fwd.p, g->det.p, g->cnt.p, g->kw.p, gram_slots, tgroup, uset_slots, map_slots, words,
+                                                              union_slots, g->counter.p + 1);
         APOE_HIP(hipGetLastError());
         unsigned long long failed = 0;
         APOE_HIP(hipMemcpyAsync(&failed, g->counter.p + 1, sizeof(failed), hipMemcpyDeviceToHost, ctx->stream));

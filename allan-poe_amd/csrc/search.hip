@@ -223,9 +223,10 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
     return lo0;
 }
 
-template <int NW, int MODE>
+template <int NW, int MODE, bool NARROW>
 __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))) void search_kernel(SearchArgs a) {
     constexpr bool KG = MODE == MODE_KG, KWD = MODE == MODE_KEYWORD;
+    a.C.narrow = NARROW ? 1u : 0u; // the pair format as a compile-time constant: no branch at the loads
     extern __shared__ __align__(16) char smem[];
     const SearchLds L(a.slots, a.cands, MODE, a.kw_slots);
     volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
@@ -369,7 +370,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                 PendingEval pe;
                 eval_issue(pe, a.C, id, pv_norm, a.paths, 1.0f);
                 bool hit = false;
-                const float acc = sparse_probe<false>(pe, T, n_ovf_seed, a.paths, nullptr, 0, hit);
+                const float acc = sparse_probe<false>(a.C, pe, T, n_ovf_seed, a.paths, nullptr, 0, hit);
                 const SparseOut so = sparse_decide(pe, acc, a.paths, bonus, __builtin_inff());
                 float dist = so.v;
                 if (!so.decided) {
@@ -435,7 +436,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                     for (int b = 0; b < EVAL_BATCH; b++) {
                         hit[b] = false;
                         acc[b] = 0.f;
-                        if (j + b * NW < n_new) acc[b] = sparse_probe<KWD>(pe[b], T, n_ovf, a.paths, kwset, a.kw_slots - 1, hit[b]);
+                        if (j + b * NW < n_new) acc[b] = sparse_probe<KWD>(a.C, pe[b], T, n_ovf, a.paths, kwset, a.kw_slots - 1, hit[b]);
                     }
 #pragma unroll
                     for (int b = 0; b < EVAL_BATCH; b++) {
@@ -666,17 +667,22 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
     }
 }
 
-template <int NW, int MODE>
-static int launch_variant(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, size_t lds, int* per_cu) {
-    const void* fn = reinterpret_cast<const void*>(&search_kernel<NW, MODE>);
+template <int NW, int MODE, bool NARROW>
+static int launch_format(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, size_t lds, int* per_cu) {
+    const void* fn = reinterpret_cast<const void*>(&search_kernel<NW, MODE, NARROW>);
     APOE_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     if (per_cu) { // occupancy query only
         APOE_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, fn, NW * WAVE, lds));
         return APOE_OK;
     }
-    search_kernel<NW, MODE><<<grid, NW * WAVE, lds, ctx->stream>>>(a);
+    search_kernel<NW, MODE, NARROW><<<grid, NW * WAVE, lds, ctx->stream>>>(a);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
+}
+
+template <int NW, int MODE>
+static int launch_variant(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, size_t lds, int* per_cu) {
+    return a.C.narrow ? launch_format<NW, MODE, true>(ctx, a, grid, lds, per_cu) : launch_format<NW, MODE, false>(ctx, a, grid, lds, per_cu);
 }
 
 template <int MODE>
@@ -792,7 +798,7 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
         stats->dense_rows = h[5];
         // dense rows actually needed + pairs + descriptor and dense norm (12 B per evaluation)
         uint64_t bytes = h[5] * (uint64_t)DENSE_BYTES;
-        bytes += 8 * (h[3] + h[4]) + 12 * h[2];
+        bytes += (c->narrow ? 6 : 8) * (h[3] + h[4]) + 12 * h[2];
         bytes += h[1] * 4ull * a.W;
         uint64_t qbytes = (uint64_t)q_count * DENSE_BYTES + 8 * (q->h_s_off[p->q_begin + q_count] - q->h_s_off[p->q_begin]) +
                           8 * (q->h_b_off[p->q_begin + q_count] - q->h_b_off[p->q_begin]);

@@ -148,7 +148,7 @@ def main():
     knn.close()
     build_wall = time.time() - t0
     mean_pairs = (corpus[2].numel() + corpus[5].numel()) / args.docs
-    nnd_bytes = nnd_dense * 4096 + nnd_evals * (8 * mean_pairs + 12)
+    nnd_bytes = nnd_dense * 4096 + nnd_evals * (gc.pair_bytes() * mean_pairs + 12)
     log(f"[bench] build: {build_gpu_ms / 1e3:.2f}s GPU time ({build_wall:.2f}s wall); NN-Descent {nnd_ms / 1e3:.2f}s, "
         f"{nnd_evals / 1e9:.2f}G evaluations, {nnd_dense / 1e9:.2f}G dense rows, {nnd_bytes / (nnd_ms / 1e3) / 1e12:.2f} TB/s algorithmic")
 

@@ -56,6 +56,7 @@ int apoe_ctx_synchronize(apoe_ctx* ctx);
  * (index.cu:842-872) and search_index_impl (query.cu:1909-1934). The rows are
  * repacked on the device into one record per document (dense row followed by the
  * SPLADE and BM25 (id, value) pairs) so that one evaluation is one contiguous read.
+ * Term ids must be below 2^31.
  */
 int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* dense,
                        const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,
@@ -66,6 +67,10 @@ void apoe_corpus_destroy(apoe_corpus* c);
 int apoe_corpus_info(const apoe_corpus* c, uint32_t* info4);
 /* Bytes of the device records: the HBM footprint one full scan reads. */
 uint64_t apoe_corpus_bytes(const apoe_corpus* c);
+/* Bytes one (term, value) pair takes in the device records: 6 when every term id of the corpus
+ * (both paths) is below 65536 (values as f32, ids as u16, the path known from the position),
+ * else 8. Chosen by apoe_corpus_create from the data; results do not depend on it. */
+uint32_t apoe_corpus_pair_bytes(const apoe_corpus* c);
 
 /* Query upload (query.cu:1936-1961). Weights are NOT folded in here; they are
  * applied when a search or distance call loads the query (query.cu:1871-1881). */

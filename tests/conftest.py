@@ -35,12 +35,23 @@ def gpu_ctx():
     ctx.close()
 
 
-@pytest.fixture(scope="session")
-def gpu_world(small_world, gpu_ctx):
+@pytest.fixture(scope="session", params=["narrow_pairs", "wide_pairs"])
+def gpu_world(request, small_world, gpu_ctx):
+    """The small world on the GPU, once per pair format of the device records. The wide form is forced by
+    relabelling every BM25 term (corpus and queries alike) past 65535: distances, graphs and searches are
+    the same, term for term, so the oracle-built index of the small world serves both."""
     import apoe
+    import oracle as O
     w = dict(small_world)
+    if request.param == "wide_pairs":
+        shift = np.uint32(70000)
+        w["corpus"] = w["corpus"][:5] + (w["corpus"][5] + shift,) + w["corpus"][6:]
+        w["queries"] = w["queries"][:5] + (w["queries"][5] + shift,) + w["queries"][6:]
+        w["C"] = O.HybridSet(*w["corpus"])
+        w["Q"] = O.HybridSet(*w["queries"])
     w["ctx"] = gpu_ctx
-    w["gc"] = apoe.Corpus(gpu_ctx, *small_world["corpus"])
-    w["gq"] = apoe.Queries(gpu_ctx, *small_world["queries"])
+    w["gc"] = apoe.Corpus(gpu_ctx, *w["corpus"])
+    assert w["gc"].pair_bytes() == (8 if request.param == "wide_pairs" else 6)
+    w["gq"] = apoe.Queries(gpu_ctx, *w["queries"])
     w["gg"] = apoe.Graph(gpu_ctx, small_world["rows"], small_world["entry"])
     return w

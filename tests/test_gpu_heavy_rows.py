@@ -10,8 +10,8 @@ pytestmark = pytest.mark.gpu
 N, HEAVY_EVERY = 2000, 50  # every 50th doc is heavy: 450 SPLADE + 260 BM25 terms more than the others
 
 
-@pytest.fixture(scope="module")
-def heavy_world(gpu_ctx):
+@pytest.fixture(scope="module", params=[0, 70000], ids=["narrow_pairs", "wide_pairs"])
+def heavy_world(request, gpu_ctx):
     import apoe
     import apoe_synth as S
     import oracle as O
@@ -36,12 +36,15 @@ def heavy_world(gpu_ctx):
 
     s_off, s_idx, s_val = inflate(s_off, s_idx, s_val, 450, 0.2, 2.0)
     b_off, b_idx, b_val = inflate(b_off, b_idx, b_val, 260, 0.5, 8.0)
+    b_idx = b_idx + np.uint32(request.param)  # relabelled BM25 terms past 65535 force 8-byte pairs on the device
     corpus = (dense, s_off, s_idx, s_val, b_off, b_idx, b_val)
     queries = S.to_numpy(S.queries(100, seed=62, device="cpu"))
+    queries = queries[:5] + (queries[5] + np.uint32(request.param),) + queries[6:]
     C, Q = O.HybridSet(*corpus), O.HybridSet(*queries)
     rows, entry, knn_ids, knn_dist = O.build_index(C, dense_scale=7.0, K=64, iters=6, d=32, seed=5, return_knn=True)
     gc = apoe.Corpus(gpu_ctx, *corpus)
     gq = apoe.Queries(gpu_ctx, *queries)
+    assert gc.pair_bytes() == (8 if request.param else 6)
     info = gc.info()
     assert info[2] > 400 and info[3] > 250  # the heavy rows are there
     return dict(ctx=gpu_ctx, C=C, Q=Q, gc=gc, gq=gq, rows=rows, entry=entry, knn_ids=knn_ids, knn_dist=knn_dist)
