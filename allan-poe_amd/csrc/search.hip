@@ -121,27 +121,34 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
     const int lane = lane_id();
     const uint32_t cands = P.cands;
     if (n == 0) return cands;
-    // order by counting: rank = #{(d, id) pairs below mine}; ids are distinct
+    // a candidate beyond the pool's worst entry cannot enter (with a full pool that is most of them:
+    // everything the bound rejected, and more): only the others are ordered and merged
     float d = INF_DIS;
     uint32_t id = EMPTY, ent = EMPTY, hop = 0, rank = 0;
-    if (lane < (int)n) {
-        d = ndist[lane];
+    if (lane < (int)n) d = ndist[lane];
+    const bool keep = lane < (int)n && d <= P.dist[cands - 1];
+    const uint64_t kept = __ballot(keep);
+    if (kept == 0) return cands;
+    // order by counting: rank = #{kept (d, id) pairs below mine}; ids are distinct
+    if (keep) {
         id = nid[lane];
         if (KG) { ent = nent[lane]; hop = nhop[lane]; }
         if (KWD) ent = nent[lane];
-        for (uint32_t i = 0; i < n; i++) {
-            const float di = ndist[i];
-            const uint32_t ii = nid[i];
-            rank += (di < d) || (di == d && ii < id);
-        }
+    }
+    for (uint64_t rest = kept; rest; rest &= rest - 1) {
+        const uint32_t i = __builtin_ctzll(rest); // wave-uniform
+        const float di = ndist[i];
+        const uint32_t ii = nid[i];
+        rank += (di < d) || (di == d && ii < id);
     }
     wave_fence();
-    if (lane < (int)n) {
+    if (keep) {
         ndist[rank] = d;
         nid[rank] = id;
         if (KG) { nent[rank] = ent; nhop[rank] = hop; }
         if (KWD) nent[rank] = ent;
     }
+    n = __popcll(kept);
     wave_fence();
     // lane i now takes the i-th smallest
     uint32_t lb = cands;
