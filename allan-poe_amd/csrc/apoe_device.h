@@ -342,105 +342,175 @@ __device__ __forceinline__ float readlane_f32(float v, uint32_t src) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
 }
 
-// ---- bucket table: the query's terms for the search kernels ----
-// Two (key, value) entries per 16-byte bucket, so a lookup is ONE ds_read_b128 and no probe loop:
-// every lane can issue the reads for all its pairs (of several candidates) back to back instead of
-// walking a chain of dependent LDS reads whose length is set by the unluckiest lane. A term whose
-// bucket is already full goes to an overflow list that holds up to every term of the row (with
-// at least twice as many buckets as terms it is empty for most rows); its length is wave-uniform
-// and the list is only walked when it is not zero.
-struct BucketTab {
-    uint4* b;        // [mask + 1] buckets: (key0, value0, key1, value1)
-    uint2* ovf;      // overflow entries
+// ---- query term tables for the search kernels ----
+// One table per path (SPLADE first, BM25 second, the same number of buckets each), two (key, value)
+// entries per 16-byte bucket, so a lookup is ONE ds_read_b128 and no probe loop: every lane can issue
+// the reads for all its pairs (of several candidates) back to back instead of walking a chain of
+// dependent LDS reads whose length is set by the unluckiest lane. Keys are stored the way the record
+// loads deliver them ("raw": without the path bit for narrow records, with it for wide ones), so a
+// probe needs no operation on the loaded key besides the hash; the table is picked by the pair's
+// path. A term whose bucket is already full goes to an overflow list that holds up to every term of
+// the row (with at least twice as many buckets as terms it is empty for most rows); its length is
+// wave-uniform and the list is only walked when it is not zero.
+struct QueryTabs {
+    uint4* b;        // [2 * (mask + 1)] buckets: (key0, value0, key1, value1)
+    uint2* ovf;      // overflow entries: (term | path bit, value)
     uint32_t* n_ovf; // their number
-    uint32_t mask;
+    uint32_t mask;   // buckets per table - 1
 };
 
-__device__ __forceinline__ void bucket_tab_clear(const BucketTab& T, int tid, int nthreads) {
-    for (uint32_t i = tid; i <= T.mask; i += nthreads) T.b[i] = make_uint4(EMPTY, 0u, EMPTY, 0u);
+// Hash of a raw key. The 24-bit multiply is a full-rate instruction (the 32-bit one is not).
+template <bool NARROW>
+__device__ __forceinline__ uint32_t query_hash(uint32_t raw) {
+    if (NARROW) return __umul24(raw, 0x9E3779u) >> 10;
+    const uint32_t k = raw & 0x7FFFFFFFu;
+    return __umul24(k ^ (k >> 16), 0x9E3779u) >> 10;
+}
+
+__device__ __forceinline__ void query_tabs_clear(const QueryTabs& T, int tid, int nthreads) {
+    for (uint32_t i = tid; i < 2 * (T.mask + 1); i += nthreads) T.b[i] = make_uint4(EMPTY, 0u, EMPTY, 0u);
     if (tid == 0) *T.n_ovf = 0;
 }
 
-// Keys inserted into one table are distinct.
-__device__ __forceinline__ void bucket_tab_insert(const BucketTab& T, uint32_t key, float val) {
-    uint4* e = T.b + term_hash(key, T.mask);
-    if (atomicCAS(&e->x, EMPTY, key) == EMPTY) { e->y = __float_as_uint(val); return; }
-    if (atomicCAS(&e->z, EMPTY, key) == EMPTY) { e->w = __float_as_uint(val); return; }
+// key carries the path bit; keys inserted into one table are distinct.
+template <bool NARROW>
+__device__ __forceinline__ void query_tabs_insert(const QueryTabs& T, uint32_t key, float val) {
+    const uint32_t raw = NARROW ? key & ~BM25_BIT : key;
+    uint4* e = T.b + ((key & BM25_BIT) ? T.mask + 1 : 0u) + (query_hash<NARROW>(raw) & T.mask);
+    if (atomicCAS(&e->x, EMPTY, raw) == EMPTY) { e->y = __float_as_uint(val); return; }
+    if (atomicCAS(&e->z, EMPTY, raw) == EMPTY) { e->w = __float_as_uint(val); return; }
     T.ovf[atomicAdd(T.n_ovf, 1u)] = make_uint2(key, __float_as_uint(val));
 }
 
-__device__ __forceinline__ void bucket_terms_from_query(const BucketTab& T, const SetView& Q, uint32_t q, float w_s, float w_b, bool use_s,
-                                                        bool use_b, int tid, int nthreads) {
+template <bool NARROW>
+__device__ __forceinline__ void query_tabs_fill(const QueryTabs& T, const SetView& Q, uint32_t q, float w_s, float w_b, bool use_s, bool use_b,
+                                                int tid, int nthreads) {
     if (use_s)
-        for (uint32_t j = Q.s_off[q] + tid; j < Q.s_off[q + 1]; j += nthreads) bucket_tab_insert(T, Q.s_idx[j], Q.s_val[j] * w_s);
+        for (uint32_t j = Q.s_off[q] + tid; j < Q.s_off[q + 1]; j += nthreads) query_tabs_insert<NARROW>(T, Q.s_idx[j], Q.s_val[j] * w_s);
     if (use_b)
         for (uint32_t j = Q.b_off[q] + tid; j < Q.b_off[q + 1]; j += nthreads)
-            bucket_tab_insert(T, Q.b_idx[j] | BM25_BIT, Q.b_val[j] * w_b);
+            query_tabs_insert<NARROW>(T, Q.b_idx[j] | BM25_BIT, Q.b_val[j] * w_b);
 }
 
-// The per-lane part of stage 1: this lane's pairs of the candidate against the query's table.
-// Straight-line code on purpose: the three bucket reads of a candidate are issued back to back
-// and a lane without a pair at some position computes on a (0, 0) pair whose result is masked.
-template <bool KWD>
-__device__ __forceinline__ void bucket_match(const uint4 e, uint2 kv, bool valid, float& acc, const uint32_t* kwset, uint32_t kwmask, bool& hit) {
-    const bool m0 = e.x == kv.x, m1 = e.z == kv.x;
-    const float v = __uint_as_float(m0 ? e.y : e.w);
-    const bool found = valid && (m0 || m1);
-    const float next = fmaf(__uint_as_float(kv.y), v, acc);
-    acc = found ? next : acc;
-    if (KWD) {
-        if (found && (kv.x & BM25_BIT) && id_set_contains(kwset, kwmask, kv.x)) hit = true;
+// The pairs of one candidate row on their way to a probe: three chunks of 64, raw keys and value
+// bits per lane, and what the wave knows about the row. The loads are not clamped to the row (no
+// address arithmetic per lane beyond lane * size): a lane past the end reads whatever follows the
+// row (the record buffer ends with slack for that) and the probe masks it.
+struct RowLoad {
+    uint32_t k[3], v[3];
+};
+struct RowInfo { // wave-uniform
+    const char* rec;
+    uint32_t ns, nb;
+    uint32_t begin; // first pair of the paths in use
+    uint32_t n;     // pairs of the paths in use (0 for a candidate that is not there)
+    uint32_t nsr;   // SPLADE pairs among them
+};
+constexpr uint32_t ROW_LOAD_SLACK = 3 * WAVE * 8; // bytes a row load may read past the last record
+
+template <bool NARROW>
+__device__ __forceinline__ void row_issue(RowLoad& r, RowInfo& s, const CorpusView& C, uint64_t desc, bool live, uint32_t paths) {
+    const int lane = lane_id();
+    s.rec = C.recs + desc_off(desc) * 16;
+    s.ns = desc_nnz_s(desc);
+    s.nb = desc_nnz_b(desc);
+    s.begin = (paths & PATH_SPARSE) ? 0u : s.ns;
+    const uint32_t end = (paths & PATH_BM25) ? s.ns + s.nb : s.ns;
+    s.n = live ? end - s.begin : 0u;
+    s.nsr = s.ns - s.begin;
+    if (NARROW) {
+        const uint32_t* vals = reinterpret_cast<const uint32_t*>(s.rec + DENSE_BYTES) + s.begin;
+        const uint16_t* keys = reinterpret_cast<const uint16_t*>(s.rec + DENSE_BYTES + 4 * (size_t)(s.ns + s.nb)) + s.begin;
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            r.k[c] = keys[lane + WAVE * c];
+            r.v[c] = vals[lane + WAVE * c];
+        }
+    } else {
+        const uint2* pairs = reinterpret_cast<const uint2*>(s.rec + DENSE_BYTES) + s.begin;
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            const uint2 kv = pairs[lane + WAVE * c];
+            r.k[c] = kv.x;
+            r.v[c] = kv.y;
+        }
     }
 }
 
-template <bool KWD>
-__device__ __forceinline__ void overflow_match(const BucketTab& T, uint32_t n_ovf, uint2 kv, bool valid, float& acc, const uint32_t* kwset,
-                                               uint32_t kwmask, bool& hit) {
+template <bool NARROW, bool KWD>
+__device__ __forceinline__ void query_match(const uint4 e, uint32_t raw, uint32_t val_bits, bool valid, bool bm25, float& acc, const uint32_t* kwset,
+                                            uint32_t kwmask, bool& hit) {
+    const bool m0 = e.x == raw, m1 = e.z == raw;
+    const float v = __uint_as_float(m0 ? e.y : e.w);
+    const bool found = valid && (m0 || m1);
+    const float next = fmaf(__uint_as_float(val_bits), v, acc);
+    acc = found ? next : acc;
+    if (KWD) {
+        if (found && bm25 && id_set_contains(kwset, kwmask, raw | BM25_BIT)) hit = true;
+    }
+}
+
+template <bool NARROW, bool KWD>
+__device__ __forceinline__ void query_overflow(const QueryTabs& T, uint32_t n_ovf, uint32_t raw, uint32_t val_bits, bool valid, bool bm25, float& acc,
+                                               const uint32_t* kwset, uint32_t kwmask, bool& hit) {
+    const uint32_t key = NARROW ? raw | (bm25 ? BM25_BIT : 0u) : raw;
     for (uint32_t i = 0; i < n_ovf; i++) {
         const uint2 o = T.ovf[i];
-        if (valid && o.x == kv.x) {
-            acc = fmaf(__uint_as_float(kv.y), __uint_as_float(o.y), acc);
+        if (valid && o.x == key) {
+            acc = fmaf(__uint_as_float(val_bits), __uint_as_float(o.y), acc);
             if (KWD) {
-                if ((kv.x & BM25_BIT) && id_set_contains(kwset, kwmask, kv.x)) hit = true;
+                if (bm25 && id_set_contains(kwset, kwmask, key)) hit = true;
             }
         }
     }
 }
 
-// n_ovf is the (wave-uniform) overflow count read after the table was built.
-template <bool KWD>
-__device__ __forceinline__ float sparse_probe(const CorpusView& C, const PendingEval& p, const BucketTab& T, uint32_t n_ovf, uint32_t paths,
-                                              const uint32_t* kwset, uint32_t kwmask, bool& hit) {
+// The per-lane part of stage 1: this lane's pairs of the candidate against the query's tables.
+// Straight-line code on purpose: the three bucket reads of a candidate are issued back to back.
+// n_ovf is the (wave-uniform) overflow count read after the tables were built.
+template <bool NARROW, bool KWD>
+__device__ __forceinline__ float row_probe(const CorpusView& C, const RowLoad& r, const RowInfo& s, const QueryTabs& T, uint32_t n_ovf,
+                                           const uint32_t* kwset, uint32_t kwmask, bool& hit) {
     const int lane = lane_id();
     float acc = 0.f;
-    if (!(paths & (PATH_SPARSE | PATH_BM25))) return acc;
-    const uint32_t j0 = p.begin + lane, j1 = j0 + WAVE, j2 = j1 + WAVE;
-    const bool in0 = j0 < p.end, in1 = j1 < p.end, in2 = j2 < p.end;
-    const uint2 kv0 = make_uint2(p.kv0.x | pair_flag(C.narrow, p.ns, j0), p.kv0.y);
-    const uint2 kv1 = make_uint2(p.kv1.x | pair_flag(C.narrow, p.ns, j1), p.kv1.y);
-    const uint2 kv2 = make_uint2(p.kv2.x | pair_flag(C.narrow, p.ns, j2), p.kv2.y);
-    uint4 e0 = T.b[term_hash(kv0.x, T.mask)];
-    uint4 e1 = T.b[term_hash(kv1.x, T.mask)];
-    uint4 e2 = T.b[term_hash(kv2.x, T.mask)];
-    // keep the three reads together: nothing below may be scheduled between them
-    asm volatile("" : "+v"(e0.x), "+v"(e1.x), "+v"(e2.x));
-    bucket_match<KWD>(e0, kv0, in0, acc, kwset, kwmask, hit);
-    bucket_match<KWD>(e1, kv1, in1, acc, kwset, kwmask, hit);
-    bucket_match<KWD>(e2, kv2, in2, acc, kwset, kwmask, hit);
-    if (n_ovf) {
-        overflow_match<KWD>(T, n_ovf, kv0, in0, acc, kwset, kwmask, hit);
-        overflow_match<KWD>(T, n_ovf, kv1, in1, acc, kwset, kwmask, hit);
-        overflow_match<KWD>(T, n_ovf, kv2, in2, acc, kwset, kwmask, hit);
+    bool in[3], bm[3];
+    uint4 e[3];
+    const uint4* tab_s = T.b;
+    const uint4* tab_b = T.b + T.mask + 1;
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        in[c] = lane < (int)s.n - WAVE * c;
+        bm[c] = NARROW ? lane >= (int)s.nsr - WAVE * c : (int)r.k[c] < 0;
+        e[c] = (bm[c] ? tab_b : tab_s)[query_hash<NARROW>(r.k[c]) & T.mask];
     }
-    if (p.begin + 3 * WAVE < p.end) { // rows with more than 192 pairs
-        const Pairs sp = record_pairs(C, p.rec, p.ns, p.nb);
-        for (uint32_t j = j2 + WAVE; j < p.end; j += WAVE) {
-            const uint2 kv = sp[j];
-            bucket_match<KWD>(T.b[term_hash(kv.x, T.mask)], kv, true, acc, kwset, kwmask, hit);
-            overflow_match<KWD>(T, n_ovf, kv, true, acc, kwset, kwmask, hit);
+    // keep the three reads together: nothing below may be scheduled between them
+    asm volatile("" : "+v"(e[0].x), "+v"(e[1].x), "+v"(e[2].x));
+#pragma unroll
+    for (int c = 0; c < 3; c++) query_match<NARROW, KWD>(e[c], r.k[c], r.v[c], in[c], bm[c], acc, kwset, kwmask, hit);
+    if (n_ovf) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) query_overflow<NARROW, KWD>(T, n_ovf, r.k[c], r.v[c], in[c], bm[c], acc, kwset, kwmask, hit);
+    }
+    if (s.n > 3 * WAVE) { // rows with more than 192 pairs
+        Pairs sp = record_pairs(C, s.rec, s.ns, s.nb);
+        sp.narrow = NARROW ? 1u : 0u;
+        for (uint32_t j = s.begin + 3 * WAVE + lane; j < s.begin + s.n; j += WAVE) {
+            const uint2 kv = sp.raw(j);
+            const bool b = NARROW ? j >= s.ns : (int)kv.x < 0;
+            query_match<NARROW, KWD>((b ? tab_b : tab_s)[query_hash<NARROW>(kv.x) & T.mask], kv.x, kv.y, true, b, acc, kwset, kwmask, hit);
+            query_overflow<NARROW, KWD>(T, n_ovf, kv.x, kv.y, true, b, acc, kwset, kwmask, hit);
         }
     }
     return acc;
+}
+
+// Sum inside each row of 16 lanes (every lane of a row gets its row's sum): four DPP adds.
+__device__ __forceinline__ float row_sum_dpp(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));  // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));  // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)); // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)); // row_mirror
+    return v;
 }
 
 // The wave-level part of stage 1: reduce, then decide whether the dense row is needed at all.

@@ -101,6 +101,7 @@ struct apoe_corpus {
 struct apoe_queries {
     apoe_ctx* ctx = nullptr;
     uint32_t n = 0, dim = 0, max_nnz = 0; // max over queries of nnz_s + nnz_b
+    uint32_t max_nnz_s = 0, max_nnz_b = 0; // ... and of either alone
     uint32_t max_keywords = 0;            // max over queries of BM25 terms flagged as required keyword (bit 31)
     uint64_t total_nnz_s = 0, total_nnz_b = 0;
     std::vector<uint32_t> h_s_off, h_b_off;

@@ -183,7 +183,7 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
         APOE_REQUIRE(off16 < (1ull << DESC_OFF_BITS), "corpus of %llu bytes exceeds the record address range", (unsigned long long)off16 * 16);
         c->rec_bytes = off16 * 16;
         APOE_TRY(c->desc.alloc(n));
-        APOE_TRY(c->recs.alloc(c->rec_bytes));
+        APOE_TRY(c->recs.alloc(c->rec_bytes + ROW_LOAD_SLACK)); // unclamped row loads may read past the last record
         APOE_TRY(c->dnorm.alloc(n));
         APOE_TRY(copy_in(ctx, c->desc.p, desc.data(), n * sizeof(uint64_t)));
         APOE_TRY(d_dense.init(ctx, dense, (size_t)n * dim));
@@ -235,8 +235,11 @@ int apoe_queries_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* de
     const uint32_t nnz_s = q->h_s_off[n], nnz_b = q->h_b_off[n];
     APOE_REQUIRE(nnz_s == 0 || (s_idx && s_val), "sparse idx/val is null");
     APOE_REQUIRE(nnz_b == 0 || (b_idx && b_val), "bm25 idx/val is null");
-    for (uint32_t i = 0; i < n; i++)
+    for (uint32_t i = 0; i < n; i++) {
         q->max_nnz = std::max(q->max_nnz, (q->h_s_off[i + 1] - q->h_s_off[i]) + (q->h_b_off[i + 1] - q->h_b_off[i]));
+        q->max_nnz_s = std::max(q->max_nnz_s, q->h_s_off[i + 1] - q->h_s_off[i]);
+        q->max_nnz_b = std::max(q->max_nnz_b, q->h_b_off[i + 1] - q->h_b_off[i]);
+    }
     q->total_nnz_s = nnz_s;
     q->total_nnz_b = nnz_b;
     if (nnz_b) {

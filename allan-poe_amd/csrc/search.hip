@@ -6,8 +6,18 @@
 namespace apoe {
 
 constexpr int MAX_NEW = 64;   // fresh candidates per step: one lane each in wave 0
-constexpr int EVAL_BATCH = 3;  // candidates whose sparse parts a wave keeps in flight together
-constexpr int DENSE_BATCH = 1; // dense rows a wave keeps in flight together
+// Tuning constants (the defaults are the measured best on MI355X; -D overrides are for measuring others).
+#ifndef APOE_EVAL_BATCH
+#define APOE_EVAL_BATCH 3
+#endif
+#ifndef APOE_DENSE_BATCH
+#define APOE_DENSE_BATCH 1
+#endif
+#ifndef APOE_SEARCH_WAVES_PER_EU
+#define APOE_SEARCH_WAVES_PER_EU 5
+#endif
+constexpr int EVAL_BATCH = APOE_EVAL_BATCH;   // candidates whose sparse parts a wave keeps in flight together
+constexpr int DENSE_BATCH = APOE_DENSE_BATCH; // dense rows a wave keeps in flight together
 constexpr int MERGE_ROUNDS = 4; // 64-element rounds of the pool that the merge moves per LDS round trip
 constexpr int RING = 32;      // keyword-filter search: evicted keyword hits kept beside the pool (query.cu:18)
 
@@ -49,7 +59,7 @@ struct SearchArgs {
 
 // LDS carve-up shared by host (size) and device (pointers).
 struct SearchLds {
-    uint32_t qd, tab, ovf, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ring_id,
+    uint32_t qd, part, tab, ovf, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ring_id,
         ring_dist, kwset, ctl, total;
     __host__ __device__ SearchLds(uint32_t slots, uint32_t cands, int mode, uint32_t kw_slots) {
         const bool kg = mode == MODE_KG, kwd = mode == MODE_KEYWORD;
@@ -57,16 +67,18 @@ struct SearchLds {
         uint32_t o = 0;
         qd = o; o += DENSE_BYTES;       // the query's dense row, weight applied
         ctl = o; o += 16 * 4;
+        part = o; o += MAX_NEW * 16;    // sparse sum of a fresh candidate as four partial sums (one per 16 lanes)
         new_lb = o; o += MAX_NEW * 4;
         new_id = o; o += MAX_NEW * 4;
         new_dist = o; o += MAX_NEW * 4;
-        new_ent = o; o += MAX_NEW * 4;  // KG: linking entity; keyword search: the hit flag of a fresh candidate
-        new_hop = o; o += MAX_NEW * 4;
-        link = o; o += MAX_NEW * 4;
-        ring_id = o; o += RING * 4;
-        ring_dist = o; o += RING * 4;
-        tab = o; o += slots * 16;     // buckets of two (key, value) entries
-        ovf = o; o += slots / 2 * 8;  // overflow entries: up to every term of the longest query row
+        new_ent = o; o += kg || kwd ? MAX_NEW * 4 : 0; // KG: linking entity; keyword search: the hit flag of a fresh candidate
+        new_hop = o; o += kg ? MAX_NEW * 4 : 0;
+        link = o; o += kg ? MAX_NEW * 4 : 0;
+        ring_id = o; o += kwd ? RING * 4 : 0;
+        ring_dist = o; o += kwd ? RING * 4 : 0;
+        tab = o; o += 2 * slots * 16; // two tables (SPLADE, BM25) of `slots` buckets of two (key, value) entries; slots >= 2 x the
+                                      // longest row of either path keeps overflows rare
+        ovf = o; o += slots * 8;      // overflow entries: up to every term of the longest query row
         pool_id = o; o += cands * 4;
         pool_dist = o; o += cands * 4;
         pool_ent = o; o += kg ? cands * 4 : 0;
@@ -231,14 +243,15 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
 }
 
 template <int NW, int MODE, bool NARROW>
-__global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))) void search_kernel(SearchArgs a) {
+__global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(APOE_SEARCH_WAVES_PER_EU, 8))) void search_kernel(SearchArgs a) {
     constexpr bool KG = MODE == MODE_KG, KWD = MODE == MODE_KEYWORD;
     a.C.narrow = NARROW ? 1u : 0u; // the pair format as a compile-time constant: no branch at the loads
     extern __shared__ __align__(16) char smem[];
     const SearchLds L(a.slots, a.cands, MODE, a.kw_slots);
     volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
     float4* qd = reinterpret_cast<float4*>(smem + L.qd);
-    BucketTab T;
+    float* part = reinterpret_cast<float*>(smem + L.part);
+    QueryTabs T;
     T.b = reinterpret_cast<uint4*>(smem + L.tab);
     T.ovf = reinterpret_cast<uint2*>(smem + L.ovf);
     T.n_ovf = const_cast<uint32_t*>(&ctl[CTL_NOVF]);
@@ -282,7 +295,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             uint4* b4 = reinterpret_cast<uint4*>(bitmap);
             for (uint32_t i = tid; i < a.bitmap_words / 4; i += NW * WAVE) b4[i] = make_uint4(0, 0, 0, 0);
         }
-        bucket_tab_clear(T, tid, NW * WAVE);
+        query_tabs_clear(T, tid, NW * WAVE);
         if (KWD) {
             for (uint32_t i = tid; i < a.kw_slots; i += NW * WAVE) kwset[i] = EMPTY;
             R.n = 0;
@@ -301,7 +314,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
         }
         __threadfence();
         __syncthreads();
-        bucket_terms_from_query(T, a.cold->Q, q, a.cold->w_s, a.cold->w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
+        query_tabs_fill<NARROW>(T, a.cold->Q, q, a.cold->w_s, a.cold->w_b, a.paths & PATH_SPARSE, a.paths & PATH_BM25, tid, NW * WAVE);
         if (KWD) {
             // required keywords: BM25 query terms whose id arrives with bit 31 set (query.cu:1828-1843)
             for (uint32_t j = a.cold->Q.b_off[q] + tid; j < a.cold->Q.b_off[q + 1]; j += NW * WAVE) {
@@ -312,7 +325,8 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
 
         __syncthreads();
         const float pv_norm = pivot_dense_norm_lds(qd);
-        uint64_t st_exp = 0, st_eval = 0, st_ns = 0, st_nb = 0, st_dense = 0; // wave-uniform counters
+        uint64_t st_exp = 0, st_eval = 0, st_dense = 0; // wave-uniform counters
+        uint32_t ln_s = 0, ln_b = 0;                    // pairs read for the candidates this lane decided
         uint32_t hint = 0;                                       // wave 0: every pool slot below hint is explored
 
         // ---- seeds ----
@@ -374,22 +388,25 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             for (uint32_t j = wave; j < n_seed; j += NW) {
                 const uint32_t id = uniform(seed_id[j]);
                 const float bonus = seed_ent[j] != EMPTY ? a.kg_weight : 0.0f; // query.cu:1637-1638
-                PendingEval pe;
-                eval_issue(pe, a.C, id, pv_norm, a.paths, 1.0f);
+                RowLoad rl;
+                RowInfo ri;
+                row_issue<NARROW>(rl, ri, a.C, a.C.desc[id], true, a.paths);
                 bool hit = false;
-                const float acc = sparse_probe<false>(a.C, pe, T, n_ovf_seed, a.paths, nullptr, 0, hit);
-                const SparseOut so = sparse_decide(pe, acc, a.paths, bonus, __builtin_inff());
-                float dist = so.v;
-                if (!so.decided) {
+                const float acc = row_probe<NARROW, false>(a.C, rl, ri, T, n_ovf_seed, nullptr, 0, hit);
+                const float ssum = (a.paths & (PATH_SPARSE | PATH_BM25)) ? wave_sum_dpp(acc) : 0.f;
+                float dist = 1.0f - ssum - bonus;
+                if (a.paths & PATH_DENSE) { // seeds are never dropped by the bound
                     DenseRow row;
-                    dense_issue(row, pe.rec);
-                    dist = 1.0f - (dense_finish_lds(row, qd, 1.0f) + so.v) - bonus;
+                    dense_issue(row, ri.rec);
+                    dist = 1.0f - (dense_finish_lds(row, qd, 1.0f) + ssum) - bonus;
                     st_dense++;
                 }
                 st_eval++;
-                st_ns += (a.paths & PATH_SPARSE) ? pe.ns : 0u;
-                st_nb += (a.paths & PATH_BM25) ? pe.nb : 0u;
-                if (lane == 0) seed_dist[j] = dist;
+                if (lane == 0) {
+                    ln_s += (a.paths & PATH_SPARSE) ? ri.ns : 0u;
+                    ln_b += (a.paths & PATH_BM25) ? ri.nb : 0u;
+                    seed_dist[j] = dist;
+                }
             }
             __syncthreads();
             if (wave == 0) {
@@ -426,46 +443,73 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                 my_desc = a.C.desc[cid];
                 my_dn = a.C.dnorm[cid];
             }
-            // stage 1: the sparse parts of this wave's candidates, EVAL_BATCH of them in flight
-            uint64_t need = 0; // bit t: the wave's t-th candidate (id wave + t*NW) still needs its dense row
-            {
-                uint32_t t0 = 0;
-                for (uint32_t j = wave; j < n_new; j += NW * EVAL_BATCH, t0 += EVAL_BATCH) {
-                    PendingEval pe[EVAL_BATCH];
+            // stage 1: the sparse parts of this wave's candidates (wave + k * NW), EVAL_BATCH of them in flight.
+            // No branch on whether a candidate of the batch exists: one that does not is a row of no pairs,
+            // so the loads of the whole batch are issued back to back.
+            for (uint32_t j = wave; j < n_new; j += NW * EVAL_BATCH) {
+                RowLoad rl[EVAL_BATCH];
+                RowInfo ri[EVAL_BATCH];
 #pragma unroll
-                    for (int b = 0; b < EVAL_BATCH; b++) {
-                        const uint32_t jj = j + b * NW;
-                        if (jj < n_new) eval_issue_desc(pe[b], a.C, readlane64(my_desc, jj), readlane_f32(my_dn, jj), pv_norm, a.paths, 1.0f);
-                    }
-                    float acc[EVAL_BATCH];
-                    bool hit[EVAL_BATCH];
+                for (int b = 0; b < EVAL_BATCH; b++) {
+                    const uint32_t jj = j + b * NW;
+                    row_issue<NARROW>(rl[b], ri[b], a.C, readlane64(my_desc, jj & (WAVE - 1)), jj < n_new, a.paths);
+                }
+                float acc[EVAL_BATCH];
+                bool hit[EVAL_BATCH];
 #pragma unroll
-                    for (int b = 0; b < EVAL_BATCH; b++) {
-                        hit[b] = false;
-                        acc[b] = 0.f;
-                        if (j + b * NW < n_new) acc[b] = sparse_probe<KWD>(a.C, pe[b], T, n_ovf, a.paths, kwset, a.kw_slots - 1, hit[b]);
-                    }
+                for (int b = 0; b < EVAL_BATCH; b++) {
+                    hit[b] = false;
+                    acc[b] = row_probe<NARROW, KWD>(a.C, rl[b], ri[b], T, n_ovf, kwset, a.kw_slots - 1, hit[b]);
+                }
 #pragma unroll
-                    for (int b = 0; b < EVAL_BATCH; b++) {
-                        const uint32_t jj = j + b * NW;
-                        if (jj < n_new) {
-                            float bonus = 0.f;
-                            if (KG) {
-                                if (new_ent[jj] != EMPTY) bonus = a.kg_weight / (float)new_hop[jj]; // query.cu:1759-1760
-                            }
-                            const SparseOut so = sparse_decide(pe[b], acc[b], a.paths, bonus, thr_eff);
-                            const bool kw_hit = KWD ? __ballot(hit[b]) != 0 : false;
-                            st_eval++;
-                            st_ns += (a.paths & PATH_SPARSE) ? pe[b].ns : 0u;
-                            st_nb += (a.paths & PATH_BM25) ? pe[b].nb : 0u;
-                            if (lane == 0) {
-                                new_dist[jj] = so.v;
-                                if (KWD) new_ent[jj] = kw_hit ? 1u : 0u;
-                            }
-                            if (!so.decided) need |= 1ull << (t0 + b);
+                for (int b = 0; b < EVAL_BATCH; b++) {
+                    const uint32_t jj = j + b * NW;
+                    const float rs = row_sum_dpp(acc[b]);
+                    if (jj < n_new) {
+                        if ((lane & 15) == 0) part[jj * 4 + (lane >> 4)] = rs;
+                        if (KWD) {
+                            const bool kw_hit = __ballot(hit[b]) != 0;
+                            if (lane == 0) new_ent[jj] = kw_hit ? 1u : 0u;
                         }
                     }
                 }
+            }
+            wave_fence();
+            // the decision for all of the wave's candidates at once, lane l for candidate l: a candidate whose
+            // sparse part plus the bound of its dense part cannot reach the pool is reported as INF_DIS
+            uint64_t need; // bit l: candidate l still needs its dense row
+            {
+                const bool mine = (uint32_t)lane < n_new && (uint32_t)(lane & (NW - 1)) == (uint32_t)wave;
+                bool undecided = false;
+                if (mine) {
+                    float bonus = 0.f;
+                    if (KG) {
+                        if (new_ent[lane] != EMPTY) bonus = a.kg_weight / (float)new_hop[lane]; // query.cu:1759-1760
+                    }
+                    float ssum = 0.f, v = 0.f;
+                    undecided = true;
+                    if (a.paths & (PATH_SPARSE | PATH_BM25)) {
+                        const float4 p4 = reinterpret_cast<const float4*>(part)[lane];
+                        ssum = p4.x + p4.y + p4.z + p4.w; // the order wave_sum_dpp adds its four rows in
+                        v = ssum;
+                        if (!(a.paths & PATH_DENSE)) {
+                            v = 1.0f - ssum - bonus;
+                            undecided = false;
+                        } else {
+                            const float dub = pv_norm * my_dn; // |<query_d, doc_d>| <= |query_d| * |doc_d|
+                            const float lb = 1.0f - (ssum + dub) - bonus;
+                            if (lb > thr_eff + 1e-5f * (fabsf(ssum) + dub + fabsf(bonus) + 1.0f)) {
+                                v = INF_DIS;
+                                undecided = false;
+                            }
+                        }
+                    }
+                    new_dist[lane] = v;
+                    ln_s += (a.paths & PATH_SPARSE) ? desc_nnz_s(my_desc) : 0u;
+                    ln_b += (a.paths & PATH_BM25) ? desc_nnz_b(my_desc) : 0u;
+                }
+                st_eval += __popcll(__ballot(mine));
+                need = __ballot(undecided);
             }
             wave_fence();
             // stage 2: the dense rows of the survivors, DENSE_BATCH rows in flight
@@ -476,9 +520,8 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
                 for (int b = 0; b < DENSE_BATCH; b++) {
                     jj[b] = EMPTY;
                     if (need) {
-                        const uint32_t t = __builtin_ctzll(need);
+                        jj[b] = __builtin_ctzll(need);
                         need &= need - 1;
-                        jj[b] = wave + t * NW;
                         dense_issue(row[b], a.C.recs + desc_off(readlane64(my_desc, jj[b])) * 16);
                     }
                 }
@@ -664,11 +707,17 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(5, 8))
             }
             for (uint32_t i = kn + m + lane; i < cands; i += WAVE) { oid[i] = EMPTY & ~FLAG; od[i] = INF_DIS; }
         }
+        uint32_t st_ns = ln_s, st_nb = ln_b;
+#pragma unroll
+        for (int o = WAVE / 2; o > 0; o >>= 1) {
+            st_ns += __shfl_xor(st_ns, o, WAVE);
+            st_nb += __shfl_xor(st_nb, o, WAVE);
+        }
         if (lane == 0) {
             if (st_exp) atomicAdd(a.work + 1, st_exp);
             if (st_eval) atomicAdd(a.work + 2, st_eval);
-            if (st_ns) atomicAdd(a.work + 3, st_ns);
-            if (st_nb) atomicAdd(a.work + 4, st_nb);
+            if (st_ns) atomicAdd(a.work + 3, (unsigned long long)st_ns);
+            if (st_nb) atomicAdd(a.work + 4, (unsigned long long)st_nb);
             if (st_dense) atomicAdd(a.work + 5, st_dense);
         }
     }
@@ -740,7 +789,7 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     a.q_count = q_count;
     cold.out_ids = out_ids_dev;
     cold.out_dist = out_dist_dev;
-    a.slots = next_pow2(std::max(64u, 2 * q->max_nnz));
+    a.slots = next_pow2(std::max(32u, 2 * std::max(q->max_nnz_s, q->max_nnz_b)));
     a.kg_weight = p->kg_weight;
     a.full_eval = (p->variant & 0x100u) ? 1u : 0u;
 
