@@ -32,10 +32,13 @@ __host__ __device__ inline uint64_t desc_off(uint64_t d) { return d & DESC_OFF_M
 __host__ __device__ inline uint32_t desc_nnz_s(uint64_t d) { return (uint32_t)(d >> DESC_OFF_BITS) & DESC_NNZ_MAX; }
 __host__ __device__ inline uint32_t desc_nnz_b(uint64_t d) { return (uint32_t)(d >> (DESC_OFF_BITS + DESC_NNZ_BITS)) & DESC_NNZ_MAX; }
 
-// Record = [DIM floats][pairs], 16-byte aligned, pairs = nnz_s SPLADE terms then nnz_b BM25 terms.
+// Record = [DIM floats][pairs], pairs = nnz_s SPLADE terms then nnz_b BM25 terms.
 // Wide pairs:   nnz x (term | path bit, value), two 32-bit words each.
 // Narrow pairs: nnz x value (f32), then nnz x term (u16); the path of pair j follows from j >= nnz_s.
 // A corpus is narrow when every term id of both paths is below 65536 (6 instead of 8 bytes a pair).
+// Records start on a 128-byte boundary, and so does the term array of a narrow record: a read of
+// a row, of its values or of its terms then starts at a memory line and only its last line is partial.
+constexpr uint32_t REC_ALIGN = 128;
 struct CorpusView {
     const uint64_t* desc;
     const char* recs;
@@ -44,8 +47,12 @@ struct CorpusView {
     uint32_t narrow;
 };
 
+__host__ __device__ inline uint32_t narrow_keys_offset(uint32_t nnz) { // of the term array, from the first value
+    return (4u * nnz + REC_ALIGN - 1) & ~(REC_ALIGN - 1);
+}
 __host__ __device__ inline uint64_t record_units(uint32_t nnz, bool narrow) { // 16-byte units of one record
-    return ((uint64_t)DENSE_BYTES + (uint64_t)(narrow ? 6 : 8) * nnz + 15) / 16;
+    const uint64_t bytes = (uint64_t)DENSE_BYTES + (narrow ? (uint64_t)narrow_keys_offset(nnz) + 2ull * nnz : 8ull * nnz);
+    return (bytes + REC_ALIGN - 1) / REC_ALIGN * (REC_ALIGN / 16);
 }
 
 struct SetView { // a set kept in CSR form on the device (queries)
@@ -76,11 +83,11 @@ struct Pairs {
     uint32_t ns, nnz; // SPLADE pairs, all pairs
     uint32_t narrow;
     __device__ __forceinline__ uint2 raw(uint32_t j) const {
-        if (narrow) return make_uint2(reinterpret_cast<const uint16_t*>(base + 4 * (size_t)nnz)[j], reinterpret_cast<const uint32_t*>(base)[j]);
+        if (narrow) return make_uint2(reinterpret_cast<const uint16_t*>(base + narrow_keys_offset(nnz))[j], reinterpret_cast<const uint32_t*>(base)[j]);
         return reinterpret_cast<const uint2*>(base)[j];
     }
     __device__ __forceinline__ uint32_t key(uint32_t j) const {
-        if (narrow) return (uint32_t) reinterpret_cast<const uint16_t*>(base + 4 * (size_t)nnz)[j] | pair_flag(1, ns, j);
+        if (narrow) return (uint32_t) reinterpret_cast<const uint16_t*>(base + narrow_keys_offset(nnz))[j] | pair_flag(1, ns, j);
         return reinterpret_cast<const uint2*>(base)[j].x;
     }
     __device__ __forceinline__ uint2 operator[](uint32_t j) const {
@@ -420,7 +427,7 @@ __device__ __forceinline__ void row_issue(RowLoad& r, RowInfo& s, const CorpusVi
     s.nsr = s.ns - s.begin;
     if (NARROW) {
         const uint32_t* vals = reinterpret_cast<const uint32_t*>(s.rec + DENSE_BYTES) + s.begin;
-        const uint16_t* keys = reinterpret_cast<const uint16_t*>(s.rec + DENSE_BYTES + 4 * (size_t)(s.ns + s.nb)) + s.begin;
+        const uint16_t* keys = reinterpret_cast<const uint16_t*>(s.rec + DENSE_BYTES + narrow_keys_offset(s.ns + s.nb)) + s.begin;
 #pragma unroll
         for (int c = 0; c < 3; c++) {
             r.k[c] = keys[lane + WAVE * c];

@@ -90,7 +90,7 @@ struct apoe_ctx {
 struct apoe_corpus {
     apoe_ctx* ctx = nullptr;
     uint32_t n = 0, dim = 0, max_nnz_s = 0, max_nnz_b = 0;
-    uint64_t rec_bytes = 0;
+    uint64_t rec_bytes = 0, total_pairs = 0;
     bool narrow = false; // pair format of the records (6 instead of 8 bytes a pair when every term id is below 65536)
     apoe::DevBuf<uint64_t> desc;
     apoe::DevBuf<char> recs;

@@ -182,6 +182,7 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
         }
         APOE_REQUIRE(off16 < (1ull << DESC_OFF_BITS), "corpus of %llu bytes exceeds the record address range", (unsigned long long)off16 * 16);
         c->rec_bytes = off16 * 16;
+        c->total_pairs = (uint64_t)hs[n] + hb[n];
         APOE_TRY(c->desc.alloc(n));
         APOE_TRY(c->recs.alloc(c->rec_bytes + ROW_LOAD_SLACK)); // unclamped row loads may read past the last record
         APOE_TRY(c->dnorm.alloc(n));

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void pack_kernel(uint32_t n, const float* __re
         const uint32_t s0 = s_off[doc], ns = desc_nnz_s(d), b0 = b_off[doc], nb = desc_nnz_b(d), nnz = ns + nb;
         if (narrow) {
             float* vals = reinterpret_cast<float*>(rec + DENSE_BYTES);
-            uint16_t* keys = reinterpret_cast<uint16_t*>(rec + DENSE_BYTES + 4 * (size_t)nnz);
+            uint16_t* keys = reinterpret_cast<uint16_t*>(rec + DENSE_BYTES + narrow_keys_offset(nnz));
             for (uint32_t j = threadIdx.x; j < ns; j += blockDim.x) {
                 vals[j] = s_val[s0 + j];
                 keys[j] = (uint16_t)s_idx[s0 + j];
@@ -56,15 +56,17 @@ __global__ __launch_bounds__(256) void pack_kernel(uint32_t n, const float* __re
                 vals[ns + j] = b_val[b0 + j];
                 keys[ns + j] = (uint16_t)b_idx[b0 + j];
             }
-            // fill the alignment tail so that a record never holds stale bytes
-            const uint32_t tail = (uint32_t)(record_units(nnz, true) * 16 - DENSE_BYTES - 6 * (size_t)nnz) / 2;
-            if (threadIdx.x < tail) keys[nnz + threadIdx.x] = 0xFFFFu;
+            // fill the two alignment gaps so that a record never holds stale bytes
+            for (uint32_t j = nnz + threadIdx.x; j < narrow_keys_offset(nnz) / 4; j += blockDim.x) vals[j] = 0.f;
+            const uint32_t key_slots = (uint32_t)(record_units(nnz, true) * 16 - DENSE_BYTES - narrow_keys_offset(nnz)) / 2;
+            for (uint32_t j = nnz + threadIdx.x; j < key_slots; j += blockDim.x) keys[j] = 0xFFFFu;
         } else {
             uint2* sp = reinterpret_cast<uint2*>(rec + DENSE_BYTES);
             for (uint32_t j = threadIdx.x; j < ns; j += blockDim.x) sp[j] = make_uint2(s_idx[s0 + j], __float_as_uint(s_val[s0 + j]));
             for (uint32_t j = threadIdx.x; j < nb; j += blockDim.x)
                 sp[ns + j] = make_uint2(b_idx[b0 + j] | BM25_BIT, __float_as_uint(b_val[b0 + j]));
-            if ((nnz & 1u) && threadIdx.x == 0) sp[nnz] = make_uint2(EMPTY, 0u);
+            const uint32_t pair_slots = (uint32_t)(record_units(nnz, false) * 16 - DENSE_BYTES) / 8;
+            for (uint32_t j = nnz + threadIdx.x; j < pair_slots; j += blockDim.x) sp[j] = make_uint2(EMPTY, 0u);
         }
     }
 }

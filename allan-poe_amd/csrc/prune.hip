@@ -624,7 +624,7 @@ int launch_prune(apoe_knn* g, uint32_t degree) {
     const uint32_t lds_budget = (uint32_t)std::min<size_t>(ctx->lds_per_block, 80 * 1024);
     uint32_t tgroup = GramPruneLds(gram_slots, 8, uset_slots, map_slots, words, 0).total <= lds_budget ? 8 : 4;
     // one union table for GU_T pivots when it fits: 2.5 slots per term of an average group, and room for the longest row alone
-    const double mean_nnz = g->n ? ((double)g->corpus->rec_bytes / g->n - DENSE_BYTES) / (g->corpus->narrow ? 6.0 : 8.0) : 0.0;
+    const double mean_nnz = g->n ? (double)g->corpus->total_pairs / g->n : 0.0;
     uint32_t union_slots = std::max(next_pow2((uint32_t)std::ceil(2.5 * GU_T * mean_nnz)), std::max(512u, gram_slots));
     if (GramPruneLds(gram_slots, tgroup, uset_slots, map_slots, words, union_slots).total > lds_budget) union_slots = 0;
     const GramPruneLds GL(gram_slots, tgroup, uset_slots, map_slots, words, union_slots);
