@@ -425,16 +425,18 @@ __device__ __forceinline__ void row_issue(RowLoad& r, RowInfo& s, const CorpusVi
     const uint32_t end = (paths & PATH_BM25) ? s.ns + s.nb : s.ns;
     s.n = live ? end - s.begin : 0u;
     s.nsr = s.ns - s.begin;
+    // a dense-only search reads no pairs: its (masked) loads all go to the first record and stay in the cache
+    const char* from = (paths & (PATH_SPARSE | PATH_BM25)) ? s.rec : C.recs;
     if (NARROW) {
-        const uint32_t* vals = reinterpret_cast<const uint32_t*>(s.rec + DENSE_BYTES) + s.begin;
-        const uint16_t* keys = reinterpret_cast<const uint16_t*>(s.rec + DENSE_BYTES + narrow_keys_offset(s.ns + s.nb)) + s.begin;
+        const uint32_t* vals = reinterpret_cast<const uint32_t*>(from + DENSE_BYTES) + s.begin;
+        const uint16_t* keys = reinterpret_cast<const uint16_t*>(from + DENSE_BYTES + narrow_keys_offset(s.ns + s.nb)) + s.begin;
 #pragma unroll
         for (int c = 0; c < 3; c++) {
             r.k[c] = keys[lane + WAVE * c];
             r.v[c] = vals[lane + WAVE * c];
         }
     } else {
-        const uint2* pairs = reinterpret_cast<const uint2*>(s.rec + DENSE_BYTES) + s.begin;
+        const uint2* pairs = reinterpret_cast<const uint2*>(from + DENSE_BYTES) + s.begin;
 #pragma unroll
         for (int c = 0; c < 3; c++) {
             const uint2 kv = pairs[lane + WAVE * c];
