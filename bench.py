@@ -12,6 +12,8 @@ search run by the CPU oracle on the host cores (a reported baseline only).
 import argparse
 import json
 import os
+import re
+import subprocess
 import sys
 import time
 
@@ -24,11 +26,11 @@ HBM_PEAK_GBS = 8000.0
 # scaled by what the counters read for a 1 GiB copy), keyed by the workload they were taken on:
 # (docs, degree, queries, cands, variant). Other workloads report null.
 MEASURED_TRAFFIC = {
-    (1000000, 48, 10000, 512, 0): 393428145495,
+    (1000000, 48, 10000, 512, 0): 331855118633,
 }
 # The same for the launches that read every dense row (variant | 0x100).
 MEASURED_TRAFFIC_FULL = {
-    (1000000, 48, 10000, 512, 0): 987710363815,
+    (1000000, 48, 10000, 512, 0): 909885813748,
 }
 
 
@@ -101,6 +103,7 @@ def main():
     ap.add_argument("--cpu-queries", type=int, default=10000)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-membench", action="store_true", help="do not run allan-poe_amd/membench for roofline.random_read_ceiling")
     ap.add_argument("--extras", action="store_true",
                     help="also time the other search paths at cands=128: the query-time weight sweep, the knowledge-graph search "
                          "(200k entities, 1-3 entities per query, kg_weight 40) and the keyword-filter search (rarest BM25 term of each query)")
@@ -327,10 +330,34 @@ def main():
                      # default mode's time: what a kernel without the bound would have to sustain to be as fast
                      "equivalent_if_every_evaluation_read_its_dense_row": {"bytes_per_launch": full_bytes,
                                                                             "gbs": full_bytes / (avg_kernel_ms / 1e3) / 1e9},
-                     "every_dense_row_read": full_eval},
+                     "every_dense_row_read": full_eval,
+                     # what this GPU gives a kernel that does nothing but such loads (allan-poe_amd/membench, run now)
+                     "random_read_ceiling": None if args.no_membench else membench()},
         "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)
+
+
+def membench():
+    """GB/s of random 128-byte aligned chunk reads on this GPU, by chunk size, with nothing but the loads in the kernel:
+    the ceiling of a gather of records (the search reads about 1.1 KB per evaluation, 5.2 KB when it needs the dense row)."""
+    exe = os.path.join(ROOT, "allan-poe_amd", "membench")
+    if not os.path.exists(exe):
+        return None
+    try:
+        out = subprocess.run([exe], capture_output=True, text=True, timeout=120).stdout
+    except (OSError, subprocess.TimeoutExpired):
+        return None
+    res = {"unit": "GB/s", "what": "random chunk reads, 3 in flight per wave, 20 waves per CU"}
+    for line in out.splitlines():
+        m = re.match(r"random reads,\s+(\d+) B chunks, .*:\s+(\d+) GB/s", line)
+        if m:
+            res[f"{m.group(1)}B"] = float(m.group(2))
+        m = re.match(r"random reads,\s+(\d+) B chunks \+ ([\d.]+) returning atomics per chunk:\s+(\d+) GB/s", line)
+        if m:
+            res[f"{m.group(1)}B+{m.group(2)}atomics"] = float(m.group(3))
+        log("[bench] " + line)
+    return res
 
 
 if __name__ == "__main__":
