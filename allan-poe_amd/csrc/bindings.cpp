@@ -137,6 +137,30 @@ PYBIND11_MODULE(hybrid_search, m) {
         std::vector<unsigned> r(rows.data(), rows.data() + rows.size()), e(entry.data(), entry.data() + entry.size());
         hs::write_graph(path, r, (unsigned)rows.shape(0), (unsigned)rows.shape(1), e);
     });
+    m.def(
+        "validate_graph",
+        [](const std::string& path, unsigned num_docs) {
+            const hs::GraphReport r = hs::validate_graph(path, num_docs);
+            py::dict d;
+            d["ok"] = r.ok;
+            d["message"] = r.message;
+            d["width"] = r.width;
+            d["degree"] = r.degree;
+            d["num"] = r.num;
+            d["n_entry"] = r.n_entry;
+            d["file_bytes"] = r.file_bytes;
+            d["trailing_bytes"] = r.trailing_bytes;
+            d["bad_width_words"] = r.bad_width_words;
+            d["bad_neighbours"] = r.bad_neighbours;
+            d["bad_keyword_edges"] = r.bad_keyword_edges;
+            d["bad_entry_points"] = r.bad_entry_points;
+            d["self_loops"] = r.self_loops;
+            d["keyword_counts_over_7"] = r.keyword_counts_over_7;
+            d["keyword_edges"] = r.keyword_edges;
+            return d;
+        },
+        py::arg("graph_path"), py::arg("num_docs") = 0u,
+        "Check a .poe graph file (size formula, width words, id ranges, keyword counts) without a GPU; returns a dict with 'ok' and counts.");
     m.def("_ndcg", [](const std::vector<std::vector<unsigned>>& res, const std::vector<std::vector<unsigned>>& gt) {
         double recall = 0;
         double n = hs::ndcg_at_k(res, gt, &recall);

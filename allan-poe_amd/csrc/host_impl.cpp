@@ -161,6 +161,49 @@ void load_graph(const std::string& path, std::vector<unsigned>& rows, std::vecto
     }
 }
 
+GraphReport validate_graph(const std::string& path, unsigned num_docs) {
+    GraphReport r;
+    std::ifstream in(path, std::ios::binary);
+    if (!in.is_open()) fail("open file error: " + path);
+    r.file_bytes = file_size(in);
+    if (r.file_bytes < 8) fail("bad graph header in " + path);
+    read_exact(in, &r.width, 1, path);
+    read_exact(in, &r.n_entry, 1, path);
+    if (r.width <= 8 || r.file_bytes < ((uint64_t)r.n_entry + 2) * 4) fail("bad graph header in " + path);
+    r.degree = r.width - 8;
+    const uint64_t body = r.file_bytes - ((uint64_t)r.n_entry + 2) * 4, row_bytes = ((uint64_t)r.width + 1) * 4;
+    r.num = (unsigned)(body / row_bytes);
+    r.trailing_bytes = body % row_bytes;
+    std::vector<unsigned> entry(r.n_entry), row(r.width);
+    read_exact(in, entry.data(), r.n_entry, path);
+    for (unsigned e : entry) r.bad_entry_points += e >= r.num;
+    for (unsigned v = 0; v < r.num; v++) {
+        unsigned w = 0;
+        read_exact(in, &w, 1, path);
+        read_exact(in, row.data(), r.width, path);
+        r.bad_width_words += w != r.width;
+        for (unsigned j = 0; j < r.degree; j++) {
+            r.bad_neighbours += row[j] >= r.num;
+            r.self_loops += row[j] == v;
+        }
+        const unsigned cnt = row[r.degree];
+        r.keyword_counts_over_7 += cnt > 7;
+        for (unsigned j = 0; j < std::min(cnt, 7u); j++) r.bad_keyword_edges += row[r.degree + 1 + j] >= r.num;
+        r.keyword_edges += std::min(cnt, 7u);
+    }
+    std::ostringstream msg;
+    if (r.trailing_bytes) msg << r.trailing_bytes << " bytes after the last whole row; ";
+    if (num_docs && num_docs != r.num) msg << "holds " << r.num << " rows, expected " << num_docs << "; ";
+    if (r.bad_width_words) msg << r.bad_width_words << " rows with a wrong width word; ";
+    if (r.bad_neighbours) msg << r.bad_neighbours << " neighbour ids out of range; ";
+    if (r.bad_keyword_edges) msg << r.bad_keyword_edges << " keyword-edge ids out of range; ";
+    if (r.bad_entry_points) msg << r.bad_entry_points << " entry points out of range; ";
+    r.message = msg.str();
+    r.ok = r.message.empty();
+    if (r.ok) r.message = "ok";
+    return r;
+}
+
 // K-NN graph between NN-Descent and the prune: "APKN", n, K, ids [n][K], distances [n][K].
 void write_knn(const std::string& path, unsigned n, unsigned K, const std::vector<unsigned>& ids, const std::vector<float>& dist) {
     std::ofstream out(path, std::ios::binary | std::ios::out);

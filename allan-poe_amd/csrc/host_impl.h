@@ -50,6 +50,24 @@ void load_kg(const std::string& path, std::vector<unsigned>& off, std::vector<un
 void load_txt(const std::string& path, std::vector<std::vector<unsigned>>& results, unsigned query_num);
 void write_graph(const std::string& path, const std::vector<unsigned>& rows, unsigned n, unsigned width, const std::vector<unsigned>& entry);
 void load_graph(const std::string& path, std::vector<unsigned>& rows, std::vector<unsigned>& entry, unsigned& width, unsigned& num);
+
+// What a .poe file holds, and whether every row is usable by the search kernels: the size formula
+// 8 + 4*n_ep + N*(W+1)*4 (index.cu:927-939), the per-row width words, neighbour / keyword-edge /
+// entry-point ids below N, keyword counts at most 7 (a larger count is clamped by the search, so it
+// is reported, not an error). num_docs = 0 takes N from the file size, as the reader does
+// (query.cu:35-62). No counterpart in the reference, which trusts the file.
+struct GraphReport {
+    unsigned width = 0, degree = 0, num = 0, n_entry = 0;
+    uint64_t file_bytes = 0, trailing_bytes = 0; // bytes after the last whole row
+    uint64_t bad_width_words = 0;                // rows whose leading width word differs from the header's
+    uint64_t bad_neighbours = 0, bad_keyword_edges = 0, bad_entry_points = 0; // ids >= N
+    uint64_t self_loops = 0;                     // neighbour slots that hold the row's own id (legal padding)
+    uint64_t keyword_counts_over_7 = 0, keyword_edges = 0;
+    bool ok = false; // no trailing bytes, no bad width word, no id out of range, N as expected
+    std::string message;
+};
+GraphReport validate_graph(const std::string& path, unsigned num_docs = 0);
+
 void write_knn(const std::string& path, unsigned n, unsigned K, const std::vector<unsigned>& ids, const std::vector<float>& dist);
 void load_knn(const std::string& path, unsigned n, unsigned K, std::vector<unsigned>& ids, std::vector<float>& dist);
 double ndcg_at_k(const std::vector<std::vector<unsigned>>& res, std::vector<std::vector<unsigned>> gt, double* recall);

@@ -101,6 +101,65 @@ def test_poe_roundtrip_and_size(tmp_path):
 
 # ---- the C++ host loaders of the shipped module read the same bytes ----
 
+def test_validate_graph_reports_what_is_wrong(tmp_path):
+    """hybrid_search.validate_graph on a good file and on files broken one way each (host code only, no GPU)."""
+    import hybrid_search as hs
+    rng = np.random.default_rng(5)
+    n, d = 50, 6
+    rows = rng.integers(0, n, (n, d + 8)).astype(np.uint32)
+    rows[:, d] = rng.integers(0, 8, n)
+    rows[3, 2] = 3  # a self loop is legal padding
+    entry = np.arange(d, dtype=np.uint32)
+    good = str(tmp_path / "good.poe")
+    hs._write_poe(good, rows, entry)
+    r = hs.validate_graph(good, n)
+    assert r["ok"] and r["message"] == "ok"
+    assert (r["width"], r["degree"], r["num"], r["n_entry"]) == (d + 8, d, n, d)
+    assert r["file_bytes"] == 8 + 4 * d + n * (d + 9) * 4 and r["trailing_bytes"] == 0
+    assert r["keyword_edges"] == int(rows[:, d].sum()) and r["self_loops"] == int((rows[:, :d] == np.arange(n)[:, None]).sum()) >= 1
+    assert not hs.validate_graph(good, n + 1)["ok"]
+
+    def broken(name, change_rows=None, change_entry=None, tail=b""):
+        r2, e2 = rows.copy(), entry.copy()
+        if change_rows:
+            change_rows(r2)
+        if change_entry:
+            change_entry(e2)
+        path = str(tmp_path / name)
+        hs._write_poe(path, r2, e2)
+        if tail:
+            with open(path, "ab") as f:
+                f.write(tail)
+        return hs.validate_graph(path)
+
+    r = broken("nbr.poe", change_rows=lambda x: x.__setitem__((7, 1), n + 5))
+    assert not r["ok"] and r["bad_neighbours"] == 1 and "neighbour" in r["message"]
+
+    def bad_kw(x):
+        x[9, d] = 2
+        x[9, d + 2] = 1000
+        x[9, d + 3] = 1000  # beyond the count: not looked at
+
+    r = broken("kw.poe", change_rows=bad_kw)
+    assert not r["ok"] and r["bad_keyword_edges"] == 1
+    r = broken("cnt.poe", change_rows=lambda x: x.__setitem__((4, d), 40))
+    assert r["keyword_counts_over_7"] == 1 and r["ok"]  # the search clamps the count to the 7 slots
+    r = broken("ep.poe", change_entry=lambda e: e.__setitem__(0, n))
+    assert not r["ok"] and r["bad_entry_points"] == 1
+    r = broken("tail.poe", tail=b"\0" * 12)
+    assert not r["ok"] and r["trailing_bytes"] == 12
+    # a wrong width word inside the file
+    path = str(tmp_path / "width.poe")
+    hs._write_poe(path, rows, entry)
+    with open(path, "r+b") as f:
+        f.seek(8 + 4 * d + 5 * (d + 9) * 4)
+        f.write(np.uint32(d + 7).tobytes())
+    r = hs.validate_graph(path)
+    assert not r["ok"] and r["bad_width_words"] == 1
+    with pytest.raises(RuntimeError):
+        hs.validate_graph(str(tmp_path / "missing.poe"))
+
+
 def test_host_loaders_match(tmp_path, capfd):
     import hybrid_search as hs
     import oracle as O
