@@ -171,7 +171,8 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
         APOE_TRY(launch_max_u32(ctx, d_sidx.p, hs[n], d_max.p));
         APOE_TRY(launch_max_u32(ctx, d_bidx.p, hb[n], d_max.p));
         APOE_TRY(copy_out(ctx, &max_term, d_max.p, sizeof(uint32_t)));
-        APOE_REQUIRE(max_term < BM25_BIT, "term id %u does not fit 31 bits", max_term);
+        // bit 31 is the path bit of a stored key, and a BM25 key of all ones would read as an empty table slot
+        APOE_REQUIRE(max_term < BM25_BIT - 1, "term id %u does not fit 31 bits (the largest usable id is %u)", max_term, BM25_BIT - 2);
         c->narrow = max_term < 65536u;
         std::vector<uint64_t> desc(n);
         uint64_t off16 = 0;

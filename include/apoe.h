@@ -14,7 +14,7 @@
  *  - All work of a context runs on the context's own HIP stream. A context and
  *    its handles may be used from one thread at a time. There is no global state.
  *  - Sparse matrices are CSR in the reference's file layout: off[rows+1], idx[nnz]
- *    ascending inside a row, val[nnz] (utils.cuh:380-398). Term ids must be < 2^31.
+ *    ascending inside a row, val[nnz] (utils.cuh:380-398). Term ids must be < 2^31 - 1 (corpus) and < 2^31 (queries).
  *  - Document ids must be < 2^30 (bits 30/31 are flags inside pools, query.cu:503).
  *  - dim must be 1024 (utils.cuh:31 DIM).
  */
@@ -56,7 +56,7 @@ int apoe_ctx_synchronize(apoe_ctx* ctx);
  * (index.cu:842-872) and search_index_impl (query.cu:1909-1934). The rows are
  * repacked on the device into one record per document (dense row followed by the
  * SPLADE and BM25 (id, value) pairs) so that one evaluation is one contiguous read.
- * Term ids must be below 2^31.
+ * Term ids must be below 2^31 - 1.
  */
 int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* dense,
                        const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,

@@ -91,3 +91,69 @@ def test_ragged_rows(gpu_ctx):
     a, b = np.meshgrid(np.arange(n, dtype=np.uint32), np.arange(n, dtype=np.uint32))
     assert_dist_close(apoe.distance_pairs(gpu_ctx, gc, 7.0, a.ravel(), b.ravel()), O.distance_pairs(C, 7.0, a.ravel(), b.ravel()), "ragged pairs")
     assert_dist_close(apoe.norms(gpu_ctx, gc, 7.0), O.norms(C, 7.0), "ragged norms")
+
+
+@pytest.mark.parametrize("top_id", [65535, 65536])
+def test_pair_format_boundary(gpu_ctx, top_id):
+    """Term id 65535 is the last one a narrow record holds; one id of 65536 anywhere in the corpus turns every
+    record wide. Query terms beyond 65535 never match a narrow corpus. Distances, norms and a search on a ring
+    graph agree with the oracle on both sides of the boundary, and rows that do not hold the top id do not change."""
+    import apoe
+    import oracle as O
+    rng = np.random.default_rng(31)
+    n, d = 40, 4
+    dense = (rng.standard_normal((n, 1024)) / 32).astype(np.float32)
+
+    def csr(rows_):
+        off = np.zeros(len(rows_) + 1, np.uint32)
+        off[1:] = np.cumsum([len(r) for r in rows_])
+        idx = np.array([t for r in rows_ for t in r], np.uint32)
+        val = rng.uniform(0.5, 2.0, len(idx)).astype(np.float32)
+        return off, idx, val
+
+    s_rows = [sorted(set(rng.integers(0, 65000, 30).tolist())) for _ in range(n)]
+    b_rows = [sorted(set(rng.integers(0, 65000, 12).tolist())) for _ in range(n)]
+    s_rows[3].append(top_id)   # SPLADE side
+    b_rows[5].append(top_id)   # BM25 side
+    b_rows[6].append(65535)
+    corpus = (dense,) + csr(s_rows) + csr(b_rows)
+    # queries: copies of some docs plus terms beyond 16 bits that no narrow record can hold
+    q_s = [s_rows[3] + [70000, 131071 + 65536], s_rows[8], [65535, 65536], []]
+    q_b = [b_rows[5] + [65536 + 5], b_rows[6], [65535, 65536, 70000], [top_id]]
+    queries = (dense[:4].copy(),) + csr(q_s) + csr(q_b)
+    C, Q = O.HybridSet(*corpus), O.HybridSet(*queries)
+    gc, gq = apoe.Corpus(gpu_ctx, *corpus), apoe.Queries(gpu_ctx, *queries)
+    assert gc.pair_bytes() == (6 if top_id == 65535 else 8)
+    ids = np.tile(np.arange(n, dtype=np.uint32), (4, 1))
+    for w3 in [(1, 1, 1), (0, 1, 0), (0, 0, 1), (1, 0, 2)]:
+        assert_dist_close(apoe.distance_batch(gpu_ctx, gc, gq, w3, ids), O.distance_batch(C, Q, w3, ids), f"boundary {top_id} {w3}")
+    a, b = np.meshgrid(np.arange(n, dtype=np.uint32), np.arange(n, dtype=np.uint32))
+    assert_dist_close(apoe.distance_pairs(gpu_ctx, gc, 7.0, a.ravel(), b.ravel()), O.distance_pairs(C, 7.0, a.ravel(), b.ravel()), "boundary pairs")
+    assert_dist_close(apoe.norms(gpu_ctx, gc, 7.0), O.norms(C, 7.0), "boundary norms")
+    rows = np.zeros((n, d + 8), np.uint32)
+    for v in range(n):
+        rows[v, :d] = [(v + 1) % n, (v - 1) % n, (v + 7) % n, (v + 13) % n]
+    entry = np.array([0, 20], np.uint32)
+    gg = apoe.Graph(gpu_ctx, rows, entry)
+    for w3 in [(1, 1, 1), (0, 1, 1)]:
+        got, gd, _ = apoe.search(gpu_ctx, gc, gq, gg, w3, 16)
+        want, wd, _ = O.search(C, Q, rows, entry, w3, 16)
+        assert np.array_equal(got, want)
+        assert_dist_close(gd, wd, f"boundary search {top_id} {w3}")
+    gg.close()
+    gq.close()
+    gc.close()
+
+
+def test_term_id_with_bit_31_is_rejected(gpu_ctx):
+    """Bit 31 of a stored term id is the path bit of the device records: a corpus that uses it is refused."""
+    import apoe
+    dense = np.zeros((2, 1024), np.float32)
+    off = np.array([0, 1, 2], np.uint32)
+    val = np.ones(2, np.float32)
+    ok_idx = np.array([5, 0x7FFFFFFE], np.uint32)
+    c = apoe.Corpus(gpu_ctx, dense, off, ok_idx, val, off, ok_idx, val)
+    assert c.pair_bytes() == 8
+    c.close()
+    with pytest.raises(apoe.ApoeError, match="31 bits"):
+        apoe.Corpus(gpu_ctx, dense, off, np.array([5, 0x80000001], np.uint32), val, off, ok_idx, val)
