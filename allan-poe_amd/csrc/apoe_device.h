@@ -336,10 +336,6 @@ __device__ __forceinline__ void eval_issue_desc(PendingEval& p, const CorpusView
     }
 }
 
-__device__ __forceinline__ void eval_issue(PendingEval& p, const CorpusView& C, uint32_t id, float pv_norm, uint32_t paths, float dense_mul) {
-    eval_issue_desc(p, C, C.desc[id], C.dnorm[id], pv_norm, paths, dense_mul);
-}
-
 // Lane `src` of a 64-bit / float register as a wave-uniform value (src is wave-uniform).
 __device__ __forceinline__ uint64_t readlane64(uint64_t v, uint32_t src) {
     const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)v, src), hi = __builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), src);
