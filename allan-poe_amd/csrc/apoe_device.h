@@ -582,7 +582,7 @@ __device__ __forceinline__ float pivot_dense_norm_lds(const float4* pivot) {
 }
 
 // ---- four-entry bucket table: a document's terms as pivot (NN-Descent) ----
-// Same idea as BucketTab with 32-byte buckets (two ds_read_b128 per lookup), which keeps the table
+// Same idea as QueryTabs with 32-byte buckets (two ds_read_b128 per lookup), which keeps the table
 // at 8 bytes per slot for rows of several hundred terms. A term whose bucket is full goes to the
 // overflow list (wave-uniform length, walked only when not empty); should even that list be full,
 // lookups fall back to scanning the pivot's own pair array in global memory (correct, slow, and

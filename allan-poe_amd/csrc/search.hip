@@ -1,6 +1,6 @@
-// Greedy beam search over the hybrid graph: one workgroup per query, the candidate
-// pool, the query's sparse-term table and the fresh-neighbour list in LDS, the
-// query's dense row in registers, an exact visited bitmap per workgroup in HBM.
+// Greedy beam search over the hybrid graph: one workgroup per query; the candidate pool, the
+// query's dense row, its sparse-term tables and the fresh-neighbour list in LDS; an exact
+// visited bitmap per workgroup in HBM.
 #include "apoe_internal.h"
 
 namespace apoe {
