@@ -37,7 +37,7 @@ class SearchStats(C.Structure):
 
 EXPORTS = [
     "apoe_last_error_string", "apoe_ctx_create", "apoe_ctx_destroy", "apoe_ctx_synchronize", "apoe_corpus_create",
-    "apoe_corpus_destroy", "apoe_corpus_info", "apoe_corpus_bytes", "apoe_corpus_pair_bytes", "apoe_queries_create", "apoe_queries_destroy",
+    "apoe_corpus_destroy", "apoe_corpus_info", "apoe_corpus_bytes", "apoe_corpus_pair_bytes", "apoe_corpus_make_half_rows", "apoe_queries_create", "apoe_queries_destroy",
     "apoe_kg_create", "apoe_kg_destroy", "apoe_calibrate_weights", "apoe_hybrid_distance_batch", "apoe_hybrid_distance_pairs", "apoe_norms",
     "apoe_knn_create", "apoe_knn_destroy", "apoe_nnd_init", "apoe_nnd_iterate", "apoe_nnd_merge_reverse",
     "apoe_knn_download", "apoe_knn_upload", "apoe_prune", "apoe_prune_download", "apoe_finalize_graph",
@@ -138,6 +138,10 @@ class Corpus:
 
     def pair_bytes(self):
         return int(lib().apoe_corpus_pair_bytes(self.h))
+
+    def make_half_rows(self):
+        """Half-precision copy of the dense rows, for searches with variant | 0x200."""
+        _check(lib().apoe_corpus_make_half_rows(self.ctx.h, self.h))
 
     def close(self):
         if self.h:

@@ -570,6 +570,32 @@ __device__ __forceinline__ float dense_finish_lds(const DenseRow& d, const float
     }
     return dense_mul * wave_sum_dpp(acc);
 }
+// The same with the row taken from the half-precision copy of the dense rows (2 KB instead of 4 KB): lane l
+// loads the four halves that stand where its float4 number l + 64*i stands in the fp32 row, so the pivot is read
+// from LDS exactly as above. Products and sums stay fp32.
+struct DenseRowHalf {
+    uint2 h[NV];
+};
+__device__ __forceinline__ void dense_issue_half(DenseRowHalf& d, const uint16_t* row) {
+    const uint2* r = reinterpret_cast<const uint2*>(row);
+    const int lane = lane_id();
+#pragma unroll
+    for (int i = 0; i < NV; i++) d.h[i] = r[lane + WAVE * i];
+}
+__device__ __forceinline__ float half_bits_to_float(uint32_t bits16) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16); }
+__device__ __forceinline__ float dense_finish_lds_half(const DenseRowHalf& d, const float4* pivot, float dense_mul) {
+    const int lane = lane_id();
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const float4 p = pivot[lane + WAVE * i];
+        acc = fmaf(half_bits_to_float(d.h[i].x & 0xFFFFu), p.x, acc);
+        acc = fmaf(half_bits_to_float(d.h[i].x >> 16), p.y, acc);
+        acc = fmaf(half_bits_to_float(d.h[i].y & 0xFFFFu), p.z, acc);
+        acc = fmaf(half_bits_to_float(d.h[i].y >> 16), p.w, acc);
+    }
+    return dense_mul * wave_sum_dpp(acc);
+}
 __device__ __forceinline__ float pivot_dense_norm_lds(const float4* pivot) {
     const int lane = lane_id();
     float a = 0.f;

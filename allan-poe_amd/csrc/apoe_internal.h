@@ -95,6 +95,7 @@ struct apoe_corpus {
     apoe::DevBuf<uint64_t> desc;
     apoe::DevBuf<char> recs;
     apoe::DevBuf<float> dnorm;
+    apoe::DevBuf<uint16_t> half; // optional half-precision copy of the dense rows, [n][dim] (apoe_corpus_make_half_rows)
     apoe::CorpusView view() const { return apoe::CorpusView{desc.p, recs.p, dnorm.p, n, narrow ? 1u : 0u}; }
 };
 
@@ -149,6 +150,7 @@ int launch_pack(apoe_ctx* ctx, uint32_t n, const float* dense, const uint32_t* s
                 const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, const uint64_t* desc, char* recs, float* dnorm,
                 bool narrow);
 int launch_max_u32(apoe_ctx* ctx, const uint32_t* a_dev, size_t n, uint32_t* out_dev);
+int launch_half_rows(apoe_ctx* ctx, const apoe_corpus* c, uint16_t* out_dev);
 int launch_distance_batch(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const float* w3, const uint32_t* ids_dev,
                           uint32_t M, float* out_dev);
 int launch_distance_pairs(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale, const uint32_t* a_dev, const uint32_t* b_dev,

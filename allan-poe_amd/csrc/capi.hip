@@ -201,6 +201,16 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
     return APOE_OK;
 }
 
+int apoe_corpus_make_half_rows(apoe_ctx* ctx, apoe_corpus* c) {
+    APOE_REQUIRE(ctx && c, "ctx/corpus is null");
+    if (c->half.p) return APOE_OK;
+    APOE_HIP(hipSetDevice(ctx->device));
+    APOE_TRY(c->half.alloc((size_t)c->n * c->dim));
+    APOE_TRY(launch_half_rows(ctx, c, c->half.p));
+    APOE_HIP(hipStreamSynchronize(ctx->stream));
+    return APOE_OK;
+}
+
 void apoe_corpus_destroy(apoe_corpus* c) { delete c; }
 
 int apoe_corpus_info(const apoe_corpus* c, uint32_t* info4) {
@@ -214,7 +224,7 @@ int apoe_corpus_info(const apoe_corpus* c, uint32_t* info4) {
 
 uint32_t apoe_corpus_pair_bytes(const apoe_corpus* c) { return c ? (c->narrow ? 6u : 8u) : 0u; }
 
-uint64_t apoe_corpus_bytes(const apoe_corpus* c) { return c ? c->rec_bytes + (uint64_t)c->n * 12 : 0; }
+uint64_t apoe_corpus_bytes(const apoe_corpus* c) { return c ? c->rec_bytes + (uint64_t)c->n * 12 + c->half.bytes() : 0; }
 
 int apoe_queries_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* dense, const uint32_t* s_off, const uint32_t* s_idx,
                         const float* s_val, const uint32_t* b_off, const uint32_t* b_idx, const float* b_val, apoe_queries** out) {

@@ -169,6 +169,31 @@ int launch_distance_pairs(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale
     return APOE_OK;
 }
 
+// One wave per document: the dense row rounded to half precision (round to nearest even), 2 KB per row.
+__global__ __launch_bounds__(256) void half_rows_kernel(CorpusView C, uint16_t* __restrict__ out) {
+    const int lane = lane_id();
+    const uint32_t waves = gridDim.x * (blockDim.x / WAVE);
+    for (uint32_t doc = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE; doc < C.n; doc += waves) {
+        const float4* r = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[doc]) * 16);
+        uint2* o = reinterpret_cast<uint2*>(out + (size_t)doc * DIM);
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const float4 x = r[lane + WAVE * i];
+            const uint32_t a = __builtin_bit_cast(uint16_t, (_Float16)x.x), b = __builtin_bit_cast(uint16_t, (_Float16)x.y);
+            const uint32_t c = __builtin_bit_cast(uint16_t, (_Float16)x.z), d = __builtin_bit_cast(uint16_t, (_Float16)x.w);
+            o[lane + WAVE * i] = make_uint2(a | (b << 16), c | (d << 16));
+        }
+    }
+}
+
+int launch_half_rows(apoe_ctx* ctx, const apoe_corpus* c, uint16_t* out_dev) {
+    if (c->n == 0) return APOE_OK;
+    uint32_t grid = std::min<uint32_t>((c->n + 3) / 4, 1u << 16);
+    half_rows_kernel<<<grid, 256, 0, ctx->stream>>>(c->view(), out_dev);
+    APOE_HIP(hipGetLastError());
+    return APOE_OK;
+}
+
 // One wave per document: dense_mul*|dense|^2 + sum of squared pair values.
 __global__ __launch_bounds__(256) void norms_kernel(CorpusView C, float dense_mul, float* __restrict__ out) {
     const int lane = lane_id();

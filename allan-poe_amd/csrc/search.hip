@@ -47,8 +47,10 @@ struct SearchArgs {
     uint32_t cands, max_iter, q_count;
     uint32_t* bitmaps;     // one visited bitmap per workgroup
     uint32_t bitmap_words; // multiple of 4
-    unsigned long long* work; // [0] next query, [1] expansions, [2] evaluations, [3] nnz splade, [4] nnz bm25, [5] dense rows read
+    unsigned long long* work; // [0] next query, [1] expansions, [2] evaluations, [3] nnz splade, [4] nnz bm25, [5] dense rows read,
+                              // [6] pool entries evaluated again in fp32, [7] their pairs
     uint32_t full_eval;       // 1: read the dense row of every candidate (no bound test)
+    const uint16_t* half;     // not null: the walk takes dense parts from the half-precision rows, the final pool is evaluated again in fp32
     uint32_t slots;
     // knowledge graph (KG kernels only)
     const uint32_t *e2e_off, *e2e_idx, *e2d_off, *e2d_idx;
@@ -242,7 +244,7 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
     return lo0;
 }
 
-template <int NW, int MODE, bool NARROW>
+template <int NW, int MODE, bool NARROW, bool HALF>
 __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(APOE_SEARCH_WAVES_PER_EU, 8))) void search_kernel(SearchArgs a) {
     constexpr bool KG = MODE == MODE_KG, KWD = MODE == MODE_KEYWORD;
     a.C.narrow = NARROW ? 1u : 0u; // the pair format as a compile-time constant: no branch at the loads
@@ -325,7 +327,7 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(APOE_S
 
         __syncthreads();
         const float pv_norm = pivot_dense_norm_lds(qd);
-        uint64_t st_exp = 0, st_eval = 0, st_dense = 0; // wave-uniform counters
+        uint64_t st_exp = 0, st_eval = 0, st_dense = 0, st_again = 0, st_again_pairs = 0; // wave-uniform counters
         uint32_t ln_s = 0, ln_b = 0;                    // pairs read for the candidates this lane decided
         uint32_t hint = 0;                                       // wave 0: every pool slot below hint is explored
 
@@ -512,8 +514,29 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(APOE_S
                 need = __ballot(undecided);
             }
             wave_fence();
-            // stage 2: the dense rows of the survivors, DENSE_BATCH rows in flight
-            while (need) {
+            // stage 2: the dense rows of the survivors, DENSE_BATCH rows in flight (two of the half-precision rows)
+            while (HALF && need) {
+                DenseRowHalf row[2];
+                uint32_t jj[2];
+#pragma unroll
+                for (int b = 0; b < 2; b++) {
+                    jj[b] = EMPTY;
+                    if (need) {
+                        jj[b] = __builtin_ctzll(need);
+                        need &= need - 1;
+                        dense_issue_half(row[b], a.half + (size_t)uniform(new_id[jj[b]]) * DIM);
+                    }
+                }
+#pragma unroll
+                for (int b = 0; b < 2; b++) {
+                    if (jj[b] != EMPTY) {
+                        const float dsum = dense_finish_lds_half(row[b], qd, 1.0f);
+                        st_dense++;
+                        if (lane == 0) new_dist[jj[b]] = 1.0f - (dsum + new_dist[jj[b]]) - 0.f;
+                    }
+                }
+            }
+            while (!HALF && need) {
                 DenseRow row[DENSE_BATCH];
                 uint32_t jj[DENSE_BATCH];
 #pragma unroll
@@ -670,6 +693,56 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(APOE_S
             }
             __syncthreads();
         }
+        // ---- half-precision walk: every pool entry again with its fp32 row, then the pool in order again ----
+        if (HALF) {
+            __syncthreads();
+            const uint32_t n_ovf = uniform(ctl[CTL_NOVF]);
+            for (uint32_t e = wave; e < cands; e += NW) {
+                const uint32_t id = uniform(P.id[e]) & ~FLAG;
+                if (id >= a.C.n) continue; // empty slot
+                RowLoad rl;
+                RowInfo ri;
+                row_issue<NARROW>(rl, ri, a.C, a.C.desc[id], true, a.paths);
+                bool hit = false;
+                const float acc = row_probe<NARROW, false>(a.C, rl, ri, T, n_ovf, nullptr, 0, hit);
+                const float ssum = (a.paths & (PATH_SPARSE | PATH_BM25)) ? wave_sum_dpp(acc) : 0.f;
+                // the same expressions as in the walk, so an entry gets the bits the default search gives it
+                float dist = 1.0f - ssum - 0.f;
+                if (a.paths & PATH_DENSE) {
+                    DenseRow row;
+                    dense_issue(row, ri.rec);
+                    dist = 1.0f - (dense_finish_lds(row, qd, 1.0f) + ssum) - 0.f;
+                }
+                if (lane == 0) P.dist[e] = dist;
+                st_again++;
+                st_again_pairs += ri.n;
+            }
+            __syncthreads();
+            if (wave == 0) {
+                // nearly sorted already: odd-even transposition until a double pass moves nothing (stable)
+                bool moved = true;
+                while (moved) {
+                    moved = false;
+                    for (uint32_t phase = 0; phase < 2; phase++) {
+                        bool sw = false;
+                        for (uint32_t i = phase + 2 * lane; i + 1 < cands; i += 2 * WAVE) {
+                            const float d0 = P.dist[i], d1 = P.dist[i + 1];
+                            if (d1 < d0) {
+                                const uint32_t i0 = P.id[i], i1 = P.id[i + 1];
+                                P.dist[i] = d1;
+                                P.dist[i + 1] = d0;
+                                P.id[i] = i1;
+                                P.id[i + 1] = i0;
+                                sw = true;
+                            }
+                        }
+                        wave_fence();
+                        moved |= __any(sw) != 0;
+                    }
+                }
+            }
+            __syncthreads();
+        }
         // ---- results (query.cu:566-569) ----
         if (!KWD) {
             for (uint32_t i = tid; i < cands; i += NW * WAVE) {
@@ -719,19 +792,24 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(APOE_S
             if (st_ns) atomicAdd(a.work + 3, (unsigned long long)st_ns);
             if (st_nb) atomicAdd(a.work + 4, (unsigned long long)st_nb);
             if (st_dense) atomicAdd(a.work + 5, st_dense);
+            if (st_again) atomicAdd(a.work + 6, st_again);
+            if (st_again_pairs) atomicAdd(a.work + 7, st_again_pairs);
         }
     }
 }
 
-template <int NW, int MODE, bool NARROW>
+template <int NW, int MODE, bool NARROW, bool HALF = false>
 static int launch_format(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, size_t lds, int* per_cu) {
-    const void* fn = reinterpret_cast<const void*>(&search_kernel<NW, MODE, NARROW>);
+    if constexpr (MODE == MODE_PLAIN && !HALF) {
+        if (a.half) return launch_format<NW, MODE, NARROW, true>(ctx, a, grid, lds, per_cu);
+    }
+    const void* fn = reinterpret_cast<const void*>(&search_kernel<NW, MODE, NARROW, HALF>);
     APOE_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     if (per_cu) { // occupancy query only
         APOE_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, fn, NW * WAVE, lds));
         return APOE_OK;
     }
-    search_kernel<NW, MODE, NARROW><<<grid, NW * WAVE, lds, ctx->stream>>>(a);
+    search_kernel<NW, MODE, NARROW, HALF><<<grid, NW * WAVE, lds, ctx->stream>>>(a);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
 }
@@ -792,6 +870,12 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     a.slots = next_pow2(std::max(32u, 2 * std::max(q->max_nnz_s, q->max_nnz_b)));
     a.kg_weight = p->kg_weight;
     a.full_eval = (p->variant & 0x100u) ? 1u : 0u;
+    a.half = nullptr;
+    if (p->variant & 0x200u) {
+        APOE_REQUIRE(c->half.p != nullptr, "variant 0x200 needs the half-precision rows: call apoe_corpus_make_half_rows first");
+        APOE_REQUIRE(kg == nullptr && !p->keyword_filter, "variant 0x200 (half-precision rows) is for the plain search only");
+        a.half = c->half.p;
+    }
 
     const bool use_kg = kg != nullptr;
     const bool use_kw = p->keyword_filter != 0;
@@ -853,8 +937,9 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
         stats->nnz_bm25 = h[4];
         stats->dense_rows = h[5];
         // dense rows actually needed + pairs + descriptor and dense norm (12 B per evaluation)
-        uint64_t bytes = h[5] * (uint64_t)DENSE_BYTES;
+        uint64_t bytes = h[5] * (uint64_t)(a.half ? DENSE_BYTES / 2 : DENSE_BYTES);
         bytes += (c->narrow ? 6 : 8) * (h[3] + h[4]) + 12 * h[2];
+        bytes += h[6] * (uint64_t)(DENSE_BYTES + 8) + (c->narrow ? 6 : 8) * h[7]; // the pool evaluated again in fp32
         bytes += h[1] * 4ull * a.W;
         uint64_t qbytes = (uint64_t)q_count * DENSE_BYTES + 8 * (q->h_s_off[p->q_begin + q_count] - q->h_s_off[p->q_begin]) +
                           8 * (q->h_b_off[p->q_begin + q_count] - q->h_b_off[p->q_begin]);

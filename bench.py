@@ -231,6 +231,16 @@ def main():
         del host
         extras["corpus handed over as host buffers"] = dict(seconds=h2d_s, gb=gc.bytes() / 1e9, gbs=gc.bytes() / 1e9 / h2d_s)
         log(f"[bench] extras: corpus from host buffers: {h2d_s:.2f}s for {gc.bytes() / 1e9:.2f} GB")
+        # the walk on half-precision dense rows with the final pool evaluated again in fp32 (variant | 0x200)
+        gc.make_half_rows()
+        for hc, hw in ((ec, w3), (cands, w3), (ec, (1.0, 0.0, 0.0))):
+            apoe.search(ctx, gc, gq, graph, hw, hc, variant=0x200 | args.variant)
+            ids_h, _, sh = apoe.search(ctx, gc, gq, graph, hw, hc, variant=0x200 | args.variant)
+            ids_d, _, sd = apoe.search(ctx, gc, gq, graph, hw, hc, variant=args.variant)
+            key = f"half-precision rows, weights {hw}, cands {hc}"
+            extras[key] = dict(kernel_ms=sh.kernel_ms, default_kernel_ms=sd.kernel_ms, same_top10=float((ids_h[:, :10] == ids_d[:, :10]).mean()),
+                               algo_gbs=sh.algo_bytes / (sh.kernel_ms / 1e3) / 1e9)
+            log(f"[bench] extras: {key}: {sh.kernel_ms:.2f} ms (fp32 rows {sd.kernel_ms:.2f} ms), top-10 ids equal at {extras[key]['same_top10']:.4f}")
         kg = S.knowledge_graph(200_000, args.docs, args.queries, device=dev)
         gkg = apoe.KnowledgeGraph(ctx, *kg)
         apoe.search(ctx, gc, gq, graph, w3, ec, kg=gkg, kg_weight=40.0)

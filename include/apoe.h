@@ -62,6 +62,13 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
                        const uint32_t* s_off, const uint32_t* s_idx, const float* s_val,
                        const uint32_t* b_off, const uint32_t* b_idx, const float* b_val,
                        apoe_corpus** out);
+/* Optional second copy of the dense rows in half precision (IEEE binary16, round to nearest even; 2 KB per
+ * row beside the 4 KB fp32 row, which stays). The reference keeps ONLY such a copy and multiplies and adds in
+ * half precision (f2h, utils.cuh:78-83; query.cu:459-465); here it is an option for callers that trade
+ * exactness during the graph walk for bytes: apoe_search with variant | 0x200 takes the dense part of a
+ * candidate from this copy (fp32 products and sums) and re-evaluates the final pool with the fp32 rows.
+ * Idempotent. */
+int apoe_corpus_make_half_rows(apoe_ctx* ctx, apoe_corpus* c);
 void apoe_corpus_destroy(apoe_corpus* c);
 /* info4 = {n, dim, max splade nnz per row, max bm25 nnz per row} (index.cu:829-835). */
 int apoe_corpus_info(const apoe_corpus* c, uint32_t* info4);
@@ -164,7 +171,15 @@ typedef struct {
                                         1/4/8 waves. 0x100: read the dense row of every candidate; by
                                         default a candidate whose sparse part plus the Cauchy-Schwarz
                                         bound of its dense part cannot beat the worst entry of the full
-                                        pool is dropped without reading its dense row (same results) */
+                                        pool is dropped without reading its dense row (same results).
+                                        0x200: while the graph is walked, the dense part of a candidate is
+                                        taken from the half-precision copy of the rows (needs
+                                        apoe_corpus_make_half_rows; plain search only); when the walk has
+                                        ended every pool entry is evaluated again with its fp32 row and
+                                        the pool sorted again, so the reported distances are the exact
+                                        ones; an id can differ from the default search's where the
+                                        rounding (at most 2^-11 |q_d| |d_d| w_dense per candidate)
+                                        changed a decision of the walk */
     uint32_t keyword_filter;         /* 1: keyword-filter search (search_with_keyword, query.cu:1271-1483);
                                         kg must be NULL */
 } apoe_search_params;

@@ -1,0 +1,65 @@
+"""Search that walks the graph on the half-precision copy of the dense rows (variant | 0x200) and evaluates the final
+pool again with the fp32 rows: the reported distances are the exact ones, the rows are sorted, and the ids are the
+oracle's except where the rounding of the walk changed a decision."""
+import numpy as np
+import pytest
+
+from parity import assert_dist_close, assert_topk_match, recall_at_k
+
+pytestmark = pytest.mark.gpu
+
+HALF = 0x200
+
+
+@pytest.mark.parametrize("shape", [0, 1, 2])
+@pytest.mark.parametrize("cands,w3", [(64, (1.0, 1.0, 1.0)), (16, (1.0, 0.5, 2.0)), (128, (1.0, 0.0, 0.0)), (64, (0.0, 1.0, 1.0))])
+def test_half_row_search_reports_exact_distances(gpu_world, cands, w3, shape):
+    import apoe
+    import oracle as O
+    w = gpu_world
+    w["gc"].make_half_rows()
+    w["gc"].make_half_rows()  # idempotent
+    ids, dist, st = apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], w3, cands, variant=HALF | shape)
+    ref_ids, ref_dist, ref_st = apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], w3, cands, variant=shape)
+    assert np.all(np.diff(dist, axis=1) >= 0)
+    real = ids != 0x7FFFFFFF
+    assert real[:, :10].all()
+    for q in range(0, ids.shape[0], 17):
+        r = ids[q][real[q]]
+        assert len(set(r.tolist())) == len(r)
+    # every reported distance is the fp32 metric of that pair: where the default search reports the same id, the same bits
+    same = ids == ref_ids
+    assert same.mean() > (0.98 if (w3[1] > 0 or w3[2] > 0) else 0.9)
+    assert np.array_equal(dist[same], ref_dist[same])
+    safe = np.where(real, ids, 0).astype(np.uint32)
+    again = apoe.distance_batch(w["ctx"], w["gc"], w["gq"], w3, safe)
+    assert_dist_close(dist[real], again[real], "re-evaluated pool vs distance_batch")
+    if w3[1] > 0 or w3[2] > 0:
+        # the rows are the oracle's (the dense part is a small share of these distances)
+        oid, odist, _ = O.search(w["C"], w["Q"], w["rows"], w["entry"], w3, cands)
+        assert assert_topk_match(ids, dist, oid, odist, 10, f"half rows, cands {cands}, weights {w3}") > 0.97
+    else:
+        # dense only: neighbouring candidates differ by less than the rounding of a half-precision row, so the walk may
+        # take other turns; what it finds is as good (recall against brute force)
+        truth, _ = O.bruteforce_topk(w["C"], w["Q"], w3, 10)
+        assert abs(recall_at_k(ids, truth, 10) - recall_at_k(ref_ids, truth, 10)) < 0.02
+        assert same.mean() > 0.9
+    if w3[0] > 0:
+        assert st.dense_rows > 0
+
+
+def test_half_rows_need_the_copy_and_the_plain_search(gpu_ctx, small_world):
+    import apoe
+    gc = apoe.Corpus(gpu_ctx, *small_world["corpus"])
+    gq = apoe.Queries(gpu_ctx, *small_world["queries"])
+    gg = apoe.Graph(gpu_ctx, small_world["rows"], small_world["entry"])
+    with pytest.raises(apoe.ApoeError, match="apoe_corpus_make_half_rows"):
+        apoe.search(gpu_ctx, gc, gq, gg, (1, 1, 1), 32, variant=HALF)
+    before = gc.bytes()
+    gc.make_half_rows()
+    assert gc.bytes() == before + gc.n * 2048
+    with pytest.raises(apoe.ApoeError, match="plain search"):
+        apoe.search(gpu_ctx, gc, gq, gg, (1, 1, 1), 32, variant=HALF, keyword_filter=True)
+    gg.close()
+    gq.close()
+    gc.close()
