@@ -131,6 +131,7 @@ struct apoe_knn {
     float elapsed_ms = 0.f;
     bool pruned = false;
     bool force_sequential_prune = false; // K = 64 handles use the gather-once prune unless this is set
+    bool half_rows = false;              // NN-Descent steps take dense parts from the corpus' half-precision rows
     apoe::DevBuf<uint32_t> ids, rev_cnt;
     apoe::DevBuf<unsigned long long> rev; // [n][K] reverse lists: (distance key << 32 | id) per slot
     apoe::DevBuf<float> dist, norms;

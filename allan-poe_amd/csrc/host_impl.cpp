@@ -283,6 +283,10 @@ void build_index_impl(const std::string& dense_data_path, const std::string& spa
         load_knn(opt.knn_load_path, points_num, opt.nnd_k, ids, dist);
         check(apoe_knn_upload(h.knn, ids.data(), dist.data()), "apoe_knn_upload");
     } else {
+        if (opt.half_rows) {
+            check(apoe_corpus_make_half_rows(h.ctx, h.corpus), "apoe_corpus_make_half_rows");
+            check(apoe_knn_use_half_rows(h.knn, 1), "apoe_knn_use_half_rows");
+        }
         check(apoe_nnd_init(h.knn, opt.seed), "apoe_nnd_init");
         for (unsigned it = 0; it < opt.nnd_iters; it++) check(apoe_nnd_iterate(h.knn, it + 1 == opt.nnd_iters, nullptr), "apoe_nnd_iterate");
         check(apoe_nnd_merge_reverse(h.knn), "apoe_nnd_merge_reverse");

@@ -26,6 +26,9 @@ struct BuildOptions {
     // File: "APKN", n, K (u32 each), then ids [n][K] u32, then distances [n][K] f32.
     std::string knn_save_path;
     std::string knn_load_path;
+    // NN-Descent steps on a half-precision copy of the dense rows (what the reference stores), stored distances
+    // recomputed from the fp32 rows before the prune. Off: every step reads fp32 rows.
+    bool half_rows = false;
 };
 
 struct SearchOptions {

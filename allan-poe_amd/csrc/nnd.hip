@@ -102,10 +102,12 @@ struct NndLds {
 // duplicates and ids already in u's list, evaluate the rest against u, merge those
 // closer than u's current worst into the list, and register u with every member of
 // the merged list when the list changed.
-template <bool NARROW> // the pair format of the corpus as a compile-time constant: no branch at the loads
+// NARROW: the pair format of the corpus as a compile-time constant (no branch at the loads).
+// HALF: the dense part of a candidate comes from the half-precision copy of the rows (`half`, [n][DIM]).
+template <bool NARROW, bool HALF>
 __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, float dense_mul, uint32_t K, uint32_t* ids, float* dist,
                                                                   unsigned long long* rev, uint32_t* rev_cnt, uint32_t term_slots,
-                                                                  uint32_t seen_slots, unsigned long long* inserted) {
+                                                                  uint32_t seen_slots, unsigned long long* inserted, const uint16_t* half) {
     C.narrow = NARROW ? 1u : 0u;
     extern __shared__ __align__(16) char smem[];
     const NndLds L(term_slots, seen_slots, K);
@@ -233,7 +235,9 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
                     const SparseOut so = sparse_decide(pe[b], acc[b], ALLP, 0.f, thr);
                     if (lane == 0) {
                         cand_dist[jj] = so.v;
-                        if (!so.decided) need[atomicAdd(&ctl[9], 1u)] = ((unsigned long long)jj << 40) | desc_off(readlane64(my_desc, t + b));
+                        // what stage 2 needs to find the row: the record offset, or the document id for the half-precision copy
+                        if (!so.decided)
+                            need[atomicAdd(&ctl[9], 1u)] = ((unsigned long long)jj << 40) | (HALF ? (uint64_t)cand_id[jj] : desc_off(readlane64(my_desc, t + b)));
                     }
                 }
             }
@@ -241,7 +245,29 @@ __global__ __launch_bounds__(NND_THREADS) void nnd_iterate_kernel(CorpusView C, 
     }
     __syncthreads();
     const uint32_t n_need = ctl[9];
-    for (uint32_t t = wave; t < n_need; t += NW * NND_DENSE_BATCH) {
+    for (uint32_t t = wave; HALF && t < n_need; t += NW * NND_DENSE_BATCH * 2) {
+        DenseRowHalf row[NND_DENSE_BATCH * 2];
+        uint32_t jj[NND_DENSE_BATCH * 2];
+#pragma unroll
+        for (int b = 0; b < NND_DENSE_BATCH * 2; b++) {
+            const uint32_t tt = t + b * NW;
+            jj[b] = EMPTY;
+            if (tt < n_need) {
+                const unsigned long long e = need[tt];
+                const uint32_t lo = uniform((uint32_t)e), hi = uniform((uint32_t)(e >> 32));
+                jj[b] = hi >> 8;
+                dense_issue_half(row[b], half + (size_t)lo * DIM);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < NND_DENSE_BATCH * 2; b++) {
+            if (jj[b] != EMPTY) {
+                const float dsum = dense_finish_lds_half(row[b], qd, dense_mul);
+                if (lane == 0) cand_dist[jj[b]] = 1.0f - (dsum + cand_dist[jj[b]]) - 0.f;
+            }
+        }
+    }
+    for (uint32_t t = wave; !HALF && t < n_need; t += NW * NND_DENSE_BATCH) {
         DenseRow row[NND_DENSE_BATCH];
         uint32_t jj[NND_DENSE_BATCH];
 #pragma unroll
@@ -357,10 +383,11 @@ int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted) {
     APOE_REQUIRE(L.total <= 64 * 1024, "NN-Descent needs %u bytes of LDS (rows with up to %u sparse terms)", L.total,
                  g->corpus->max_nnz_s + g->corpus->max_nnz_b);
     APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), ctx->stream)); // [0] inserted; [2], [3] accumulate over the build
-    auto kernel = g->corpus->narrow ? &nnd_iterate_kernel<true> : &nnd_iterate_kernel<false>;
+    auto kernel = g->half_rows ? (g->corpus->narrow ? &nnd_iterate_kernel<true, true> : &nnd_iterate_kernel<false, true>)
+                               : (g->corpus->narrow ? &nnd_iterate_kernel<true, false> : &nnd_iterate_kernel<false, false>);
     APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
     kernel<<<g->n, NND_THREADS, L.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->K, g->ids.p, g->dist.p, g->rev.p,
-                                                        g->rev_cnt.p, term_slots, seen_slots, g->counter.p);
+                                                        g->rev_cnt.p, term_slots, seen_slots, g->counter.p, g->half_rows ? g->corpus->half.p : nullptr);
     APOE_HIP(hipGetLastError());
     if (inserted) {
         unsigned long long h = 0;
@@ -368,6 +395,61 @@ int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted) {
         APOE_HIP(hipStreamSynchronize(ctx->stream));
         *inserted = h;
     }
+    return APOE_OK;
+}
+
+// Every stored distance again from the fp32 rows, then each list in (distance, id) order again: what follows a build
+// whose steps took the dense parts from the half-precision rows. One workgroup per node: the node is the pivot (dense
+// row in registers, terms in the LDS table), each wave takes every fourth list entry.
+__global__ __launch_bounds__(NND_THREADS) void knn_refine_kernel(CorpusView C, float dense_mul, uint32_t K, uint32_t* ids, float* dist, uint32_t slots) {
+    extern __shared__ __align__(16) char smem[];
+    uint2* tab = reinterpret_cast<uint2*>(smem);
+    uint32_t* l_id = reinterpret_cast<uint32_t*>(smem + (size_t)slots * 8);
+    float* l_dist = reinterpret_cast<float*>(l_id + K);
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const uint32_t u = blockIdx.x, mask = slots - 1;
+    const size_t base = (size_t)u * K;
+    term_table_clear(tab, slots, tid, NND_THREADS);
+    for (uint32_t j = tid; j < K; j += NND_THREADS) {
+        l_id[j] = ids[base + j];
+        l_dist[j] = dist[base + j];
+    }
+    const uint64_t du = C.desc[u];
+    const char* rec = C.recs + desc_off(du) * 16;
+    PivotDense pv;
+    pivot_dense_load(pv, reinterpret_cast<const float*>(rec), 1.0f);
+    __syncthreads();
+    pivot_terms_from_record(tab, mask, record_pairs(C, du), tid, NND_THREADS);
+    __syncthreads();
+    for (uint32_t j = wave; j < K; j += NND_THREADS / WAVE) {
+        const uint32_t v = l_id[j] & ~FLAG;
+        if (v >= C.n || !(l_dist[j] < INF_DIS)) continue; // an empty slot keeps what it holds
+        const EvalOut e = eval_wave(C, v, pv, tab, mask, PATH_DENSE | PATH_SPARSE | PATH_BM25, dense_mul);
+        if (lane == 0) l_dist[j] = 1.0f - e.ip;
+    }
+    __syncthreads();
+    // counting rank by (distance, id): the flag bit of an id stays where it is
+    for (uint32_t j = tid; j < K; j += NND_THREADS) {
+        const float d = l_dist[j];
+        const uint32_t id = l_id[j];
+        uint32_t rank = 0;
+        for (uint32_t i = 0; i < K; i++) {
+            const float di = l_dist[i];
+            const uint32_t ii = l_id[i];
+            rank += (di < d) || (di == d && ((ii & ~FLAG) < (id & ~FLAG) || ((ii & ~FLAG) == (id & ~FLAG) && i < j)));
+        }
+        ids[base + rank] = id;
+        dist[base + rank] = d;
+    }
+}
+
+int launch_knn_refine(apoe_knn* g) {
+    apoe_ctx* ctx = g->ctx;
+    const uint32_t slots = doc_term_slots(g->corpus);
+    const size_t lds = (size_t)slots * 8 + (size_t)g->K * 8;
+    APOE_REQUIRE(lds <= 64 * 1024, "document rows with %u sparse terms exceed the LDS term table", g->corpus->max_nnz_s + g->corpus->max_nnz_b);
+    knn_refine_kernel<<<g->n, NND_THREADS, lds, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->K, g->ids.p, g->dist.p, slots);
+    APOE_HIP(hipGetLastError());
     return APOE_OK;
 }
 
@@ -410,6 +492,13 @@ int apoe_knn_create(apoe_ctx* ctx, const apoe_corpus* c, uint32_t K, float dense
 
 void apoe_knn_destroy(apoe_knn* g) { delete g; }
 
+int apoe_knn_use_half_rows(apoe_knn* g, int on) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_REQUIRE(!on || g->corpus->half.p != nullptr, "the corpus has no half-precision rows: call apoe_corpus_make_half_rows first");
+    g->half_rows = on != 0;
+    return APOE_OK;
+}
+
 int apoe_nnd_init(apoe_knn* g, uint64_t seed) {
     APOE_REQUIRE(g, "null argument");
     APOE_HIP(hipSetDevice(g->ctx->device));
@@ -449,6 +538,7 @@ int apoe_nnd_merge_reverse(apoe_knn* g) {
         APOE_TRY(launch_nnd_merge_reverse(g));
         fill_u32_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->rev_cnt.p, g->n, 0u); // index.cu:899
         APOE_HIP(hipGetLastError());
+        if (g->half_rows) APOE_TRY(launch_knn_refine(g)); // the lists leave the build with fp32 distances
         return APOE_OK;
     }));
     g->elapsed_ms += ms;

@@ -241,6 +241,26 @@ def main():
             extras[key] = dict(kernel_ms=sh.kernel_ms, default_kernel_ms=sd.kernel_ms, same_top10=float((ids_h[:, :10] == ids_d[:, :10]).mean()),
                                algo_gbs=sh.algo_bytes / (sh.kernel_ms / 1e3) / 1e9)
             log(f"[bench] extras: {key}: {sh.kernel_ms:.2f} ms (fp32 rows {sd.kernel_ms:.2f} ms), top-10 ids equal at {extras[key]['same_top10']:.4f}")
+        # the build with NN-Descent steps on the half-precision rows (stored distances recomputed in fp32 before the prune)
+        knn_h = apoe.Knn(ctx, gc, args.nnd_k, 7.0)
+        knn_h.use_half_rows()
+        knn_h.init(20251125)
+        for it in range(args.nnd_iters):
+            knn_h.iterate(last=(it == args.nnd_iters - 1))
+        nnd_h_ms = knn_h.elapsed_ms()
+        knn_h.merge_reverse()
+        knn_h.prune(args.degree)
+        graph_h = knn_h.finalize()
+        build_h_ms = knn_h.elapsed_ms()
+        knn_h.close()
+        ids_gh, _, _ = apoe.search(ctx, gc, gq, graph_h, w3, ec)
+        ids_gf, _, _ = apoe.search(ctx, gc, gq, graph, w3, ec)
+        extras["build with half-precision rows"] = dict(build_seconds_gpu=build_h_ms / 1e3, nnd_seconds_gpu=nnd_h_ms / 1e3,
+                                                        recall_at_10=recall_at_k(ids_gh[:nq_truth], truth, 10),
+                                                        recall_at_10_fp32_build=recall_at_k(ids_gf[:nq_truth], truth, 10))
+        log(f"[bench] extras: build with half-precision rows: {build_h_ms / 1e3:.2f}s (NN-Descent {nnd_h_ms / 1e3:.2f}s); recall@10 at cands {ec}: "
+            f"{extras['build with half-precision rows']['recall_at_10']:.4f} (fp32 build {extras['build with half-precision rows']['recall_at_10_fp32_build']:.4f})")
+        graph_h.close()
         kg = S.knowledge_graph(200_000, args.docs, args.queries, device=dev)
         gkg = apoe.KnowledgeGraph(ctx, *kg)
         apoe.search(ctx, gc, gq, graph, w3, ec, kg=gkg, kg_weight=40.0)

@@ -128,6 +128,13 @@ int apoe_calibrate_weights(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queri
 int apoe_knn_create(apoe_ctx* ctx, const apoe_corpus* c, uint32_t K, float dense_scale,
                     apoe_knn** out);
 void apoe_knn_destroy(apoe_knn* g);
+/* on != 0: the NN-Descent steps take the dense part of a candidate from the half-precision copy of the rows
+ * (apoe_corpus_make_half_rows; 2 KB instead of 4 KB per row read, fp32 products and sums), and
+ * apoe_nnd_merge_reverse ends with a pass that computes every stored distance again from the fp32 rows and
+ * puts each list in order again, so the prune sees exact distances. Which neighbours the lists hold can
+ * differ from the fp32 build's where the rounding (at most 2^-11 dense_scale^2 |a_d| |b_d| per pair) decided.
+ * No counterpart in the reference, which has only half-precision rows. */
+int apoe_knn_use_half_rows(apoe_knn* g, int on);
 /* initialize_graph + cal_power (index.cu:890-892). */
 int apoe_nnd_init(apoe_knn* g, uint64_t seed);
 /* One nn_descent_gpu + reset_reverse_num step (index.cu:894-897). last != 0 keeps the

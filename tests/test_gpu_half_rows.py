@@ -63,3 +63,70 @@ def test_half_rows_need_the_copy_and_the_plain_search(gpu_ctx, small_world):
     gg.close()
     gq.close()
     gc.close()
+
+
+def test_half_row_build_leaves_exact_lists_and_the_same_recall(gpu_world):
+    """NN-Descent steps on the half-precision rows: after the reverse merge every stored distance is the fp32 metric
+    again and every list is in order; the K-NN recall and the recall of a search on the finished index are within
+    0.5 points of the fp32 build's."""
+    import apoe
+    import oracle as O
+    w = gpu_world
+    n = w["C"].n
+    w["gc"].make_half_rows()
+
+    def run(half):
+        knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+        if half:
+            knn.use_half_rows()
+        knn.init(5)
+        for it in range(8):
+            knn.iterate(last=(it == 7))
+        ev, dense = knn.counters()
+        knn.merge_reverse()
+        ids, dist = knn.download()
+        knn.prune(32)
+        graph = knn.finalize()
+        knn.close()
+        return ids, dist, graph, ev, dense
+
+    ids_h, dist_h, graph_h, ev_h, dense_h = run(True)
+    ids_f, dist_f, graph_f, ev_f, dense_f = run(False)
+    # invariants of a finished list
+    assert np.all(np.diff(dist_h, axis=1) >= 0) and ids_h.max() < n
+    assert not (ids_h == np.arange(n, dtype=np.uint32)[:, None]).any()
+    srt = np.sort(ids_h, axis=1)
+    assert (np.diff(srt.astype(np.int64), axis=1) != 0).all()
+    # stored distance == the fp32 metric of the pair (an independent kernel and the oracle)
+    rng = np.random.default_rng(3)
+    r, c = rng.integers(0, n, 5000), rng.integers(0, 64, 5000)
+    want = O.distance_pairs(w["C"], 7.0, r.astype(np.uint32), ids_h[r, c])
+    assert_dist_close(dist_h[r, c], want, "stored distance after the fp32 pass")
+    # the lists are as good as the fp32 build's
+    truth, _ = O.bruteforce_knn_self(w["C"], 7.0, 10)
+    rec_h = recall_at_k(ids_h, truth, 10)
+    rec_f = recall_at_k(ids_f, truth, 10)
+    assert rec_h >= rec_f - 0.005, (rec_h, rec_f)
+    # NN-Descent is a chaotic iteration (which neighbours get sampled depends on every earlier insertion), so the
+    # two builds do not end in the same lists; most neighbours are shared all the same
+    shared = np.mean([len(set(a.tolist()) & set(b.tolist())) / 64 for a, b in zip(ids_h[::40], ids_f[::40])])
+    assert shared > 0.6, shared
+    assert abs(ev_h - ev_f) <= 0.02 * ev_f and dense_h > 0
+    # and so is the finished index
+    w3 = (1.0, 1.0, 1.0)
+    t2, _ = O.bruteforce_topk(w["C"], w["Q"], w3, 10)
+    a, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], graph_h, w3, 128)
+    b, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], graph_f, w3, 128)
+    assert recall_at_k(a, t2, 10) >= recall_at_k(b, t2, 10) - 0.005
+    graph_h.close()
+    graph_f.close()
+
+
+def test_half_row_build_needs_the_copy(gpu_ctx, small_world):
+    import apoe
+    gc = apoe.Corpus(gpu_ctx, *small_world["corpus"])
+    knn = apoe.Knn(gpu_ctx, gc, 64, 7.0)
+    with pytest.raises(apoe.ApoeError, match="apoe_corpus_make_half_rows"):
+        knn.use_half_rows()
+    knn.close()
+    gc.close()
