@@ -159,6 +159,28 @@ def test_knn_graph_save_and_reprune(files, capfd):
         hybrid_search.build_index(output_graph_path=c_path, nnd_k=128, knn_load_path=knn_path, **common)
 
 
+def test_build_on_half_precision_rows(files, capfd):
+    """build_index(half_rows=True): the saved K-NN lists carry fp32 distances and the index file passes the checker."""
+    import hybrid_search
+    import oracle as O
+    p = files["paths"]
+    d = os.path.dirname(p["index.poe"])
+    knn_path, h_path = os.path.join(d, "half.knn"), os.path.join(d, "half.poe")
+    hybrid_search.build_index(dense_data_path=p["dense.fvecs"], sparse_data_path=p["sparse.bin"], bm25_data_path=p["bm25.bin"],
+                              output_graph_path=h_path, nnd_iters=6, knn_save_path=knn_path, half_rows=True)
+    capfd.readouterr()
+    n = files["n"]
+    ids = np.fromfile(knn_path, np.uint32, n * 64, offset=12).reshape(n, 64)
+    dist = np.fromfile(knn_path, np.float32, n * 64, offset=12 + n * 64 * 4).reshape(n, 64)
+    assert ids.max() < n and np.all(np.diff(dist, axis=1) >= 0)
+    rng = np.random.default_rng(2)
+    r, c = rng.integers(0, n, 3000), rng.integers(0, 64, 3000)
+    want = O.distance_pairs(files["C"], 7.0, r.astype(np.uint32), ids[r, c])
+    assert np.allclose(dist[r, c], want, rtol=1e-4, atol=1e-4)
+    rep = hybrid_search.validate_graph(h_path, n)
+    assert rep["ok"] and rep["degree"] == 32
+
+
 def test_errors_raise(files):
     import hybrid_search
     p = files["paths"]
