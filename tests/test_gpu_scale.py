@@ -112,3 +112,46 @@ def test_recall_grows_with_the_pool_and_beats_a_random_graph(world):
     ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], g2, (1, 1, 1), 128, q_count=nq)
     assert recall_at_k(ids, truth, 10) < rec[1]
     g2.close()
+
+
+def test_pair_format_does_not_change_results(world):
+    """The same corpus with its BM25 terms relabelled past 65 535 (8-byte pairs on the device instead of 6-byte ones)
+    gives the same search rows on the same graph, and K-NN lists of the same quality after one NN-Descent step."""
+    import torch
+    import apoe
+    w = world
+    shift = 70000
+    corpus_w = tuple(w["corpus"][:5]) + (w["corpus"][5] + shift,) + tuple(w["corpus"][6:])
+    queries_w = tuple(w["queries"][:5]) + (w["queries"][5] + shift,) + tuple(w["queries"][6:])
+    torch.cuda.synchronize()
+    gc2 = apoe.Corpus(w["ctx"], *corpus_w)
+    gq2 = apoe.Queries(w["ctx"], *queries_w)
+    assert w["gc"].pair_bytes() == 6 and gc2.pair_bytes() == 8
+    for w3 in ((1, 1, 1), (0, 0, 1)):
+        a, ad, sa = apoe.search(w["ctx"], w["gc"], w["gq"], w["graph"], w3, CANDS, q_count=1000)
+        b, bd, sb = apoe.search(w["ctx"], gc2, gq2, w["graph"], w3, CANDS, q_count=1000)
+        assert np.array_equal(a, b)
+        assert_dist_close(ad, bd, f"narrow vs wide pairs, weights {w3}")
+        assert sa.evaluations == sb.evaluations and sa.dense_rows == sb.dense_rows
+
+    def one_step(gc):
+        knn = apoe.Knn(w["ctx"], gc, 64, 7.0)
+        knn.init(3)
+        knn.iterate(last=True)
+        knn.merge_reverse()
+        ids, dist = knn.download()
+        knn.close()
+        return ids, dist
+
+    i1, d1 = one_step(w["gc"])
+    i2, d2 = one_step(gc2)
+    # a step reads lists that other workgroups are rewriting, so no two runs give the same lists; they are equally good
+    assert abs(float(d1.mean()) - float(d2.mean())) < 0.01 * abs(float(d1.mean()))
+    import apoe_synth as S
+    import oracle as O
+    C = O.HybridSet(*S.to_numpy(w["corpus"]))
+    rng = np.random.default_rng(4)
+    r, c = rng.integers(0, N_DOCS, 3000), rng.integers(0, 64, 3000)
+    assert_dist_close(d2[r, c], O.distance_pairs(C, 7.0, r.astype(np.uint32), i2[r, c]), "wide pairs: stored distance == metric")
+    gq2.close()
+    gc2.close()
