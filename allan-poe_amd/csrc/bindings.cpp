@@ -16,11 +16,12 @@ static hs::SearchResult run_search(const std::string& dense_data_path, const std
                                    const std::string& keyword_id_path, const std::string& knowledge_path, const std::string& entity2doc_path,
                                    const std::string& query_entity_path, const std::string& graph_path, const std::string& ground_truth_path,
                                    int top_k, int cands, float sparse_weight, float bm25_weight, float dense_weight, float kg_weight,
-                                   unsigned max_queries, bool calibrate, int device) {
+                                   unsigned max_queries, bool calibrate, int device, bool half_rows = false) {
     hs::SearchOptions opt;
     opt.max_queries = max_queries;
     opt.calibrate = calibrate;
     opt.device = device;
+    opt.half_rows = half_rows;
     py::gil_scoped_release release;
     return hs::search_index_impl(dense_data_path, dense_query_path, sparse_data_path, sparse_query_path, bm25_data_path, bm25_query_path,
                                  keyword_id_path, knowledge_path, entity2doc_path, query_entity_path, graph_path, ground_truth_path, top_k, cands,
@@ -73,9 +74,9 @@ PYBIND11_MODULE(hybrid_search, m) {
         [](const std::string& a, const std::string& b, const std::string& c, const std::string& d, const std::string& e, const std::string& f,
            const std::string& g, const std::string& h, const std::string& i, const std::string& j, const std::string& k, const std::string& l,
            int top_k, int cands, float sparse_weight, float bm25_weight, float dense_weight, float kg_weight, unsigned max_queries,
-           bool calibrate, int device) {
+           bool calibrate, int device, bool half_rows) {
             hs::SearchResult r = run_search(a, b, c, d, e, f, g, h, i, j, k, l, top_k, cands, sparse_weight, bm25_weight, dense_weight,
-                                            kg_weight, max_queries, calibrate, device);
+                                            kg_weight, max_queries, calibrate, device, half_rows);
             py::array_t<uint32_t> ids({(py::ssize_t)r.query_num, (py::ssize_t)r.cands});
             py::array_t<float> dist({(py::ssize_t)r.query_num, (py::ssize_t)r.cands});
             std::copy(r.ids.begin(), r.ids.end(), ids.mutable_data());
@@ -97,7 +98,7 @@ PYBIND11_MODULE(hybrid_search, m) {
         py::arg("bm25_query_path"), py::arg("keyword_id_path"), py::arg("knowledge_path"), py::arg("entity2doc_path"),
         py::arg("query_entity_path"), py::arg("graph_path"), py::arg("ground_truth_path"), py::arg("top_k"), py::arg("cands"),
         py::arg("sparse_weight"), py::arg("bm25_weight"), py::arg("dense_weight"), py::arg("kg_weight"), py::arg("max_queries") = 100,
-        py::arg("calibrate") = true, py::arg("device") = 0);
+        py::arg("calibrate") = true, py::arg("device") = 0, py::arg("half_rows") = false);
 
     // ---- host-side pieces exposed for tests of the file formats and of nDCG ----
     m.def("_read_fvecs", [](const std::string& path) {

@@ -420,6 +420,10 @@ SearchResult search_index_impl(const std::string& dense_data_path, const std::st
     p.kg_weight = kg_weight;
     p.cands = (unsigned)cands;
     p.keyword_filter = use_keywords ? 1u : 0u;
+    if (opt.half_rows && !use_kg && !use_keywords) {
+        check(apoe_corpus_make_half_rows(h.ctx, h.corpus), "apoe_corpus_make_half_rows");
+        p.variant |= 0x200u;
+    }
     apoe_search_stats st{};
     const auto start = std::chrono::high_resolution_clock::now();
     check(apoe_search(h.ctx, h.corpus, h.queries, h.graph, use_kg ? h.kg : nullptr, &p, res.ids.data(), res.dist.data(), &st), "apoe_search");

@@ -35,6 +35,9 @@ struct SearchOptions {
     unsigned max_queries = 100; // query.cu:1825
     bool calibrate = true;      // query.cu:1847-1869
     int device = 0;
+    // Plain search only (ignored with keywords or a knowledge graph): walk the graph on a half-precision copy of the
+    // dense rows and evaluate the final pool again from the fp32 rows.
+    bool half_rows = false;
 };
 
 struct SearchResult {

@@ -68,6 +68,12 @@ def test_build_and_search_roundtrip(files, capfd):
     assert abs(r["ndcg"] - want_ndcg) < 1e-5 and abs(r["recall"] - want_recall) < 1e-5
     assert r["ndcg"] > 0.5
 
+    # the same search walking on half-precision rows: same rows (the dense part is a small share here), exact distances
+    rh = hybrid_search.search(knowledge_path="", entity2doc_path="", query_entity_path="", kg_weight=0.0, half_rows=True, **common)
+    capfd.readouterr()
+    same = rh["ids"] == r["ids"]
+    assert same.mean() > 0.98 and np.array_equal(rh["dist"][same], r["dist"][same])
+
     # dense-only dispatch and the print-only entry point
     hybrid_search.search_index(knowledge_path="", entity2doc_path="", query_entity_path="", kg_weight=0.0,
                                **{**common, "sparse_weight": 0.0, "bm25_weight": 0.0})
