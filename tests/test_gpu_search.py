@@ -87,3 +87,23 @@ def test_bad_graph_ids_are_skipped(gpu_world):
     oid, odist, _ = O.search(w["C"], w["Q"], rows, w["entry"], (1, 1, 1), 64)
     assert assert_topk_match(ids, dist, oid, odist, 10, "bad ids") > 0.95
     g.close()
+
+
+@pytest.mark.parametrize("cands", [1, 7, 100, 2048])
+def test_pool_sizes_at_the_edges(gpu_world, cands):
+    """Pools of one entry, of sizes that are no multiple of a wave, and of the largest size the library takes
+    (more than the 1 000 iterations can explore) against the oracle; one more is refused."""
+    import apoe
+    import oracle as O
+    w = gpu_world
+    nq = 60
+    ids, dist, st = apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], (1, 1, 1), cands, q_count=nq)
+    oid, odist, cnt = O.search(w["C"], w["Q"].head(nq), w["rows"], w["entry"], (1, 1, 1), cands)
+    assert ids.shape == (nq, cands)
+    k = min(10, cands)
+    assert assert_topk_match(ids, dist, oid, odist, k, f"cands {cands}") > 0.95
+    assert np.all(np.diff(dist, axis=1) >= 0)
+    assert abs(int(st.evaluations) - int(cnt[:, 1].sum())) <= 0.01 * cnt[:, 1].sum()
+    if cands == 2048:
+        with pytest.raises(apoe.ApoeError, match="cands"):
+            apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], (1, 1, 1), cands + 1, q_count=nq)
