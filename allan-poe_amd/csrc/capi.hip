@@ -277,6 +277,15 @@ int apoe_queries_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* de
     APOE_TRY(copy_in(ctx, q->s_val.p, s_val, nnz_s * sizeof(float)));
     APOE_TRY(copy_in(ctx, q->b_idx.p, b_idx, nnz_b * sizeof(uint32_t)));
     APOE_TRY(copy_in(ctx, q->b_val.p, b_val, nnz_b * sizeof(float)));
+    if (nnz_s) { // bit 31 of a BM25 term id is the keyword flag; on a SPLADE term id it would send the term to the BM25 table
+        DevBuf<uint32_t> d_max;
+        uint32_t max_term = 0;
+        APOE_TRY(d_max.alloc(1));
+        APOE_TRY(copy_in(ctx, d_max.p, &max_term, sizeof(uint32_t)));
+        APOE_TRY(launch_max_u32(ctx, q->s_idx.p, nnz_s, d_max.p));
+        APOE_TRY(copy_out(ctx, &max_term, d_max.p, sizeof(uint32_t)));
+        APOE_REQUIRE(max_term < BM25_BIT, "query sparse term id %u does not fit 31 bits", max_term);
+    }
     *out = q.release();
     return APOE_OK;
 }

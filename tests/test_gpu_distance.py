@@ -157,3 +157,15 @@ def test_term_id_with_bit_31_is_rejected(gpu_ctx):
     c.close()
     with pytest.raises(apoe.ApoeError, match="31 bits"):
         apoe.Corpus(gpu_ctx, dense, off, np.array([5, 0x80000001], np.uint32), val, off, ok_idx, val)
+
+
+def test_query_sparse_term_with_bit_31_is_rejected(gpu_ctx):
+    """Bit 31 marks a required keyword on a BM25 query term; a SPLADE query term must not carry it."""
+    import apoe
+    dense = np.zeros((1, 1024), np.float32)
+    off = np.array([0, 1], np.uint32)
+    val = np.ones(1, np.float32)
+    q = apoe.Queries(gpu_ctx, dense, off, np.array([7], np.uint32), val, off, np.array([0x80000007], np.uint32), val)
+    q.close()
+    with pytest.raises(apoe.ApoeError, match="31 bits"):
+        apoe.Queries(gpu_ctx, dense, off, np.array([0x80000007], np.uint32), val, off, np.array([7], np.uint32), val)
