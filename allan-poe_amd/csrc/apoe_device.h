@@ -346,7 +346,7 @@ __device__ __forceinline__ float readlane_f32(float v, uint32_t src) {
 }
 
 // ---- query term tables for the search kernels ----
-// One table per path (SPLADE first, BM25 second, the same number of buckets each), two (key, value)
+// One table per path (SPLADE first, BM25 second, each sized for the longest row of its path), two (key, value)
 // entries per 16-byte bucket, so a lookup is ONE ds_read_b128 and no probe loop: every lane can issue
 // the reads for all its pairs (of several candidates) back to back instead of walking a chain of
 // dependent LDS reads whose length is set by the unluckiest lane. Keys are stored the way the record
@@ -356,10 +356,10 @@ __device__ __forceinline__ float readlane_f32(float v, uint32_t src) {
 // the row (with at least twice as many buckets as terms it is empty for most rows); its length is
 // wave-uniform and the list is only walked when it is not zero.
 struct QueryTabs {
-    uint4* b;        // [2 * (mask + 1)] buckets: (key0, value0, key1, value1)
+    uint4* b;        // [(mask_s + 1) + (mask_b + 1)] buckets: (key0, value0, key1, value1)
     uint2* ovf;      // overflow entries: (term | path bit, value)
     uint32_t* n_ovf; // their number
-    uint32_t mask;   // buckets per table - 1
+    uint32_t mask_s, mask_b; // buckets of the SPLADE / BM25 table - 1
 };
 
 // Hash of a raw key. The 24-bit multiply is a full-rate instruction (the 32-bit one is not).
@@ -371,7 +371,7 @@ __device__ __forceinline__ uint32_t query_hash(uint32_t raw) {
 }
 
 __device__ __forceinline__ void query_tabs_clear(const QueryTabs& T, int tid, int nthreads) {
-    for (uint32_t i = tid; i < 2 * (T.mask + 1); i += nthreads) T.b[i] = make_uint4(EMPTY, 0u, EMPTY, 0u);
+    for (uint32_t i = tid; i < T.mask_s + T.mask_b + 2; i += nthreads) T.b[i] = make_uint4(EMPTY, 0u, EMPTY, 0u);
     if (tid == 0) *T.n_ovf = 0;
 }
 
@@ -379,7 +379,8 @@ __device__ __forceinline__ void query_tabs_clear(const QueryTabs& T, int tid, in
 template <bool NARROW>
 __device__ __forceinline__ void query_tabs_insert(const QueryTabs& T, uint32_t key, float val) {
     const uint32_t raw = NARROW ? key & ~BM25_BIT : key;
-    uint4* e = T.b + ((key & BM25_BIT) ? T.mask + 1 : 0u) + (query_hash<NARROW>(raw) & T.mask);
+    const uint32_t h = query_hash<NARROW>(raw);
+    uint4* e = T.b + ((key & BM25_BIT) ? T.mask_s + 1 + (h & T.mask_b) : (h & T.mask_s));
     if (atomicCAS(&e->x, EMPTY, raw) == EMPTY) { e->y = __float_as_uint(val); return; }
     if (atomicCAS(&e->z, EMPTY, raw) == EMPTY) { e->w = __float_as_uint(val); return; }
     T.ovf[atomicAdd(T.n_ovf, 1u)] = make_uint2(key, __float_as_uint(val));
@@ -481,12 +482,12 @@ __device__ __forceinline__ float row_probe(const CorpusView& C, const RowLoad& r
     bool in[3], bm[3];
     uint4 e[3];
     const uint4* tab_s = T.b;
-    const uint4* tab_b = T.b + T.mask + 1;
+    const uint4* tab_b = T.b + T.mask_s + 1;
 #pragma unroll
     for (int c = 0; c < 3; c++) {
         in[c] = lane < (int)s.n - WAVE * c;
         bm[c] = NARROW ? lane >= (int)s.nsr - WAVE * c : (int)r.k[c] < 0;
-        e[c] = (bm[c] ? tab_b : tab_s)[query_hash<NARROW>(r.k[c]) & T.mask];
+        e[c] = (bm[c] ? tab_b : tab_s)[query_hash<NARROW>(r.k[c]) & (bm[c] ? T.mask_b : T.mask_s)];
     }
     // keep the three reads together: nothing below may be scheduled between them
     asm volatile("" : "+v"(e[0].x), "+v"(e[1].x), "+v"(e[2].x));
@@ -502,7 +503,8 @@ __device__ __forceinline__ float row_probe(const CorpusView& C, const RowLoad& r
         for (uint32_t j = s.begin + 3 * WAVE + lane; j < s.begin + s.n; j += WAVE) {
             const uint2 kv = sp.raw(j);
             const bool b = NARROW ? j >= s.ns : (int)kv.x < 0;
-            query_match<NARROW, KWD>((b ? tab_b : tab_s)[query_hash<NARROW>(kv.x) & T.mask], kv.x, kv.y, true, b, acc, kwset, kwmask, hit);
+            query_match<NARROW, KWD>((b ? tab_b : tab_s)[query_hash<NARROW>(kv.x) & (b ? T.mask_b : T.mask_s)], kv.x, kv.y, true, b, acc, kwset, kwmask,
+                                     hit);
             query_overflow<NARROW, KWD>(T, n_ovf, kv.x, kv.y, true, b, acc, kwset, kwmask, hit);
         }
     }

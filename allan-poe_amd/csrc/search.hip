@@ -14,7 +14,7 @@ constexpr int MAX_NEW = 64;   // fresh candidates per step: one lane each in wav
 #define APOE_DENSE_BATCH 1
 #endif
 #ifndef APOE_SEARCH_WAVES_PER_EU
-#define APOE_SEARCH_WAVES_PER_EU 5
+#define APOE_SEARCH_WAVES_PER_EU 6 // plain search: 12 queries per CU fit its LDS; the other modes need more LDS per query and stay at 5
 #endif
 constexpr int EVAL_BATCH = APOE_EVAL_BATCH;   // candidates whose sparse parts a wave keeps in flight together
 constexpr int DENSE_BATCH = APOE_DENSE_BATCH; // dense rows a wave keeps in flight together
@@ -51,7 +51,7 @@ struct SearchArgs {
                               // [6] pool entries evaluated again in fp32, [7] their pairs
     uint32_t full_eval;       // 1: read the dense row of every candidate (no bound test)
     const uint16_t* half;     // not null: the walk takes dense parts from the half-precision rows, the final pool is evaluated again in fp32
-    uint32_t slots;
+    uint32_t slots_s, slots_b, ovf_cap; // buckets of the query's SPLADE / BM25 term table, entries of the overflow list
     // knowledge graph (KG kernels only)
     const uint32_t *e2e_off, *e2e_idx, *e2d_off, *e2d_idx;
     uint32_t n_entities;
@@ -63,7 +63,7 @@ struct SearchArgs {
 struct SearchLds {
     uint32_t qd, part, tab, ovf, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ring_id,
         ring_dist, kwset, ctl, total;
-    __host__ __device__ SearchLds(uint32_t slots, uint32_t cands, int mode, uint32_t kw_slots) {
+    __host__ __device__ SearchLds(uint32_t slots_s, uint32_t slots_b, uint32_t ovf_cap, uint32_t cands, int mode, uint32_t kw_slots) {
         const bool kg = mode == MODE_KG, kwd = mode == MODE_KEYWORD;
         // fixed-size arrays first: their offsets are compile-time constants
         uint32_t o = 0;
@@ -78,9 +78,9 @@ struct SearchLds {
         link = o; o += kg ? MAX_NEW * 4 : 0;
         ring_id = o; o += kwd ? RING * 4 : 0;
         ring_dist = o; o += kwd ? RING * 4 : 0;
-        tab = o; o += 2 * slots * 16; // two tables (SPLADE, BM25) of `slots` buckets of two (key, value) entries; slots >= 2 x the
-                                      // longest row of either path keeps overflows rare
-        ovf = o; o += slots * 8;      // overflow entries: up to every term of the longest query row
+        tab = o; o += (slots_s + slots_b) * 16; // two tables (SPLADE, BM25) of buckets of two (key, value) entries; twice as many
+                                                // buckets as the longest row of the path has terms keep overflows rare
+        ovf = o; o += ovf_cap * 8;              // overflow entries: up to every term of the longest query row
         pool_id = o; o += cands * 4;
         pool_dist = o; o += cands * 4;
         pool_ent = o; o += kg ? cands * 4 : 0;
@@ -245,11 +245,11 @@ __device__ __forceinline__ uint32_t sort_merge(const Pool& P, uint32_t* nid, flo
 }
 
 template <int NW, int MODE, bool NARROW, bool HALF>
-__global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(APOE_SEARCH_WAVES_PER_EU, 8))) void search_kernel(SearchArgs a) {
+__global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(MODE == MODE_PLAIN && !HALF ? APOE_SEARCH_WAVES_PER_EU : 5, 8))) void search_kernel(SearchArgs a) {
     constexpr bool KG = MODE == MODE_KG, KWD = MODE == MODE_KEYWORD;
     a.C.narrow = NARROW ? 1u : 0u; // the pair format as a compile-time constant: no branch at the loads
     extern __shared__ __align__(16) char smem[];
-    const SearchLds L(a.slots, a.cands, MODE, a.kw_slots);
+    const SearchLds L(a.slots_s, a.slots_b, a.ovf_cap, a.cands, MODE, a.kw_slots);
     volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
     float4* qd = reinterpret_cast<float4*>(smem + L.qd);
     float* part = reinterpret_cast<float*>(smem + L.part);
@@ -257,7 +257,8 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(APOE_S
     T.b = reinterpret_cast<uint4*>(smem + L.tab);
     T.ovf = reinterpret_cast<uint2*>(smem + L.ovf);
     T.n_ovf = const_cast<uint32_t*>(&ctl[CTL_NOVF]);
-    T.mask = a.slots - 1;
+    T.mask_s = a.slots_s - 1;
+    T.mask_b = a.slots_b - 1;
     Pool P;
     P.id = reinterpret_cast<uint32_t*>(smem + L.pool_id);
     P.dist = reinterpret_cast<float*>(smem + L.pool_dist);
@@ -867,7 +868,9 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     a.q_count = q_count;
     cold.out_ids = out_ids_dev;
     cold.out_dist = out_dist_dev;
-    a.slots = next_pow2(std::max(32u, 2 * std::max(q->max_nnz_s, q->max_nnz_b)));
+    a.slots_s = next_pow2(std::max(16u, 2 * q->max_nnz_s));
+    a.slots_b = next_pow2(std::max(16u, 2 * q->max_nnz_b));
+    a.ovf_cap = (q->max_nnz + 7u) & ~7u;
     a.kg_weight = p->kg_weight;
     a.full_eval = (p->variant & 0x100u) ? 1u : 0u;
     a.half = nullptr;
@@ -896,7 +899,7 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
         cold.q2e_idx = kg->q2e_idx.p;
         a.n_entities = kg->n_entities;
     }
-    const SearchLds L(a.slots, a.cands, mode, a.kw_slots);
+    const SearchLds L(a.slots_s, a.slots_b, a.ovf_cap, a.cands, mode, a.kw_slots);
     APOE_REQUIRE(L.total <= 64 * 1024, "search needs %u bytes of LDS (query rows with up to %u sparse terms)", L.total, q->max_nnz);
 
     // variant 0: two waves per query (the measured best); 1, 2, 3: one, four, eight waves
