@@ -231,6 +231,19 @@ def main():
         del host
         extras["corpus handed over as host buffers"] = dict(seconds=h2d_s, gb=gc.bytes() / 1e9, gbs=gc.bytes() / 1e9 / h2d_s)
         log(f"[bench] extras: corpus from host buffers: {h2d_s:.2f}s for {gc.bytes() / 1e9:.2f} GB")
+        # a batch four times as long: 10 000 queries are three and a bit rounds of the resident workgroups, and the last
+        # round runs on a draining machine
+        queries4 = S.queries(4 * args.queries, seed=4321, device=dev)
+        torch.cuda.synchronize()
+        gq4 = apoe.Queries(ctx, *queries4)
+        apoe.search(ctx, gc, gq4, graph, w3, cands, variant=args.variant)
+        _, _, s4 = apoe.search(ctx, gc, gq4, graph, w3, cands, variant=args.variant)
+        extras[f"{4 * args.queries} queries, cands {cands}"] = dict(kernel_ms=s4.kernel_ms, qps=4 * args.queries / (s4.kernel_ms / 1e3),
+                                                                   algo_gbs=s4.algo_bytes / (s4.kernel_ms / 1e3) / 1e9)
+        log(f"[bench] extras: {4 * args.queries} queries at cands {cands}: {s4.kernel_ms:.2f} ms = {4 * args.queries / (s4.kernel_ms / 1e3):.0f} QPS, "
+            f"{s4.algo_bytes / (s4.kernel_ms / 1e3) / 1e9:.0f} GB/s algorithmic")
+        gq4.close()
+        del queries4
         # the walk on half-precision dense rows with the final pool evaluated again in fp32 (variant | 0x200)
         gc.make_half_rows()
         for hc, hw in ((ec, w3), (cands, w3), (ec, (1.0, 0.0, 0.0))):
