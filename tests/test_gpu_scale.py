@@ -155,3 +155,38 @@ def test_pair_format_does_not_change_results(world):
     assert_dist_close(d2[r, c], O.distance_pairs(C, 7.0, r.astype(np.uint32), i2[r, c]), "wide pairs: stored distance == metric")
     gq2.close()
     gc2.close()
+
+
+def test_kg_and_keyword_samples_match_oracle(world):
+    """Knowledge-graph and keyword-filter search at this size against the oracle on the GPU-built graph (200 queries)."""
+    import apoe
+    import apoe_synth as S
+    import oracle as O
+    w = world
+    nq = 200
+    corpus_np = S.to_numpy(w["corpus"])
+    queries_np = S.to_numpy(w["queries"])
+    C = O.HybridSet(*corpus_np)
+    Q = O.HybridSet(*queries_np).head(nq)
+    kg = S.to_numpy(S.knowledge_graph(20000, N_DOCS, N_QUERIES, seed=21, device="cpu"))
+    gkg = apoe.KnowledgeGraph(w["ctx"], *kg)
+    okg = O.Kg(kg[0], kg[1], kg[2], kg[3], kg[4][:nq + 1], kg[5][:kg[4][nq]])
+    ids, dist, _ = apoe.search(w["ctx"], w["gc"], w["gq"], w["graph"], (1, 1, 1), CANDS, kg=gkg, kg_weight=40.0, q_count=nq)
+    oid, odist, _ = O.search(C, Q, w["rows"], w["entry"], (1, 1, 1), CANDS, kg=okg, kg_weight=40.0)
+    assert assert_topk_match(ids, dist, oid, odist, 10, "100k docs, knowledge graph") > 0.97
+    gkg.close()
+    # keyword filter: the rarest BM25 term of each query is required
+    b_off, b_idx = queries_np[4], queries_np[5].copy()
+    df = np.bincount(corpus_np[5], minlength=int(max(corpus_np[5].max(), b_idx.max())) + 1)
+    for q in range(nq):
+        t = b_idx[b_off[q]:b_off[q + 1]]
+        ok = np.where(df[t] > 0)[0] if len(t) else []
+        if len(ok):
+            b_idx[b_off[q] + ok[np.argmin(df[t][ok])]] |= 0x80000000
+    qk = queries_np[:5] + (b_idx,) + queries_np[6:]
+    gqk = apoe.Queries(w["ctx"], *qk)
+    kid, kdist, _ = apoe.search(w["ctx"], w["gc"], gqk, w["graph"], (1, 1, 1), CANDS, keyword_filter=True, q_count=nq)
+    okid, okdist, _ = O.search(C, O.HybridSet(*qk).head(nq), w["rows"], w["entry"], (1, 1, 1), CANDS, keyword_filter=True)
+    assert (kid == okid).all(axis=1).mean() > 0.97
+    assert (okid != EMPTY_ID).any()
+    gqk.close()
