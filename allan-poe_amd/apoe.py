@@ -358,9 +358,18 @@ def search(ctx, corpus, queries, graph, w3, cands, kg=None, kg_weight=0.0, max_i
     keyword_filter: rows hold only documents with a BM25 term that the query flags (bit 31 of the
     query's BM25 term id) as a required keyword."""
     nq = q_count if q_count else queries.n - q_begin
+    if q_begin > queries.n or nq > queries.n - q_begin:
+        raise ApoeError(f"query range of {nq} from {q_begin} beyond {queries.n} queries")
     if out_ids is None:
         out_ids = np.empty((nq, cands), np.uint32)
         out_dist = np.empty((nq, cands), np.float32)
+    for arr, dt, name in ((out_ids, np.uint32, "out_ids"), (out_dist, np.float32, "out_dist")):
+        # the library writes into these: a copy made here would be filled and thrown away
+        if isinstance(arr, np.ndarray):
+            if arr.dtype != dt or not arr.flags.c_contiguous or arr.shape != (nq, cands):
+                raise ApoeError(f"{name} must be a C-contiguous {np.dtype(dt).name} array of shape {(nq, cands)}")
+        elif not arr.is_contiguous() or tuple(arr.shape) != (nq, cands):
+            raise ApoeError(f"{name} must be a contiguous tensor of shape {(nq, cands)}")
     ki, kd = _ptr(out_ids, np.uint32), _ptr(out_dist, np.float32)
     p = SearchParams(w3[0], w3[1], w3[2], kg_weight, cands, max_iter, q_begin, q_count, variant, 1 if keyword_filter else 0)
     st = SearchStats()

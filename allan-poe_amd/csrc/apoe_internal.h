@@ -32,6 +32,14 @@ void set_error(const char* fmt, ...);
         }                                    \
     } while (0)
 
+#define APOE_REQUIRE_STATE(cond, ...)        \
+    do {                                     \
+        if (!(cond)) {                       \
+            apoe::set_error(__VA_ARGS__);    \
+            return APOE_ERR_STATE;           \
+        }                                    \
+    } while (0)
+
 #define APOE_TRY(expr)              \
     do {                            \
         int s_ = (expr);            \
@@ -129,6 +137,7 @@ struct apoe_knn {
     uint32_t n = 0, K = 0, degree = 0;
     float dense_scale = 1.f;
     float elapsed_ms = 0.f;
+    bool ready = false;  // lists hold something: apoe_nnd_init or apoe_knn_upload has run
     bool pruned = false;
     bool force_sequential_prune = false; // K = 64 handles use the gather-once prune unless this is set
     bool half_rows = false;              // NN-Descent steps take dense parts from the corpus' half-precision rows

@@ -439,6 +439,9 @@ int apoe_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, cons
     APOE_HIP(hipSetDevice(ctx->device));
     APOE_REQUIRE(p->q_begin <= q->n, "q_begin %u beyond %u queries", p->q_begin, q->n);
     const uint32_t q_count = p->q_count ? p->q_count : q->n - p->q_begin;
+    // before anything is sized from them
+    APOE_REQUIRE(q_count <= q->n - p->q_begin, "query range of %u from %u beyond %u queries", q_count, p->q_begin, q->n);
+    APOE_REQUIRE(p->cands >= 1 && p->cands <= APOE_MAX_CANDS, "cands must be in 1..%d, got %u", APOE_MAX_CANDS, p->cands);
     DevOutput<uint32_t> d_ids;
     DevOutput<float> d_dist;
     APOE_TRY(d_ids.init(out_ids, (size_t)q_count * p->cands));

@@ -227,7 +227,7 @@ void load_knn(const std::string& path, unsigned n, unsigned K, std::vector<unsig
     read_exact(in, ids.data(), ids.size(), path);
     read_exact(in, dist.data(), dist.size(), path);
     for (unsigned v : ids)
-        if (v >= n && v != 0xFFFFFFFFu) fail("K-NN graph in " + path + " names a point beyond the corpus");
+        if (v >= n) fail("K-NN graph in " + path + " names a point beyond the corpus");
 }
 
 // query.cu:111-145: IDCG over all ground-truth ids, DCG by position in the result

@@ -505,12 +505,14 @@ int apoe_nnd_init(apoe_knn* g, uint64_t seed) {
     float ms = 0.f;
     APOE_TRY(timed(g->ctx, &ms, [&]() { return launch_nnd_init(g, seed); }));
     g->elapsed_ms = ms;
+    g->ready = true;
     g->pruned = false;
     return APOE_OK;
 }
 
 int apoe_nnd_iterate(apoe_knn* g, int last, uint64_t* inserted) {
     APOE_REQUIRE(g, "null argument");
+    APOE_REQUIRE_STATE(g->ready, "the lists are empty: call apoe_nnd_init or apoe_knn_upload first");
     APOE_HIP(hipSetDevice(g->ctx->device));
     float ms = 0.f;
     APOE_TRY(timed(g->ctx, &ms, [&]() -> int {
@@ -532,6 +534,7 @@ int apoe_nnd_iterate(apoe_knn* g, int last, uint64_t* inserted) {
 
 int apoe_nnd_merge_reverse(apoe_knn* g) {
     APOE_REQUIRE(g, "null argument");
+    APOE_REQUIRE_STATE(g->ready, "the lists are empty: call apoe_nnd_init or apoe_knn_upload first");
     APOE_HIP(hipSetDevice(g->ctx->device));
     float ms = 0.f;
     APOE_TRY(timed(g->ctx, &ms, [&]() -> int {
@@ -551,6 +554,7 @@ __global__ __launch_bounds__(256) static void strip_flags_kernel(const uint32_t*
 
 int apoe_knn_download(apoe_knn* g, uint32_t* ids, float* dist) {
     APOE_REQUIRE(g, "null argument");
+    APOE_REQUIRE_STATE(g->ready, "the lists are empty: call apoe_nnd_init or apoe_knn_upload first");
     APOE_HIP(hipSetDevice(g->ctx->device));
     const size_t total = (size_t)g->n * g->K;
     if (ids) {
@@ -564,14 +568,46 @@ int apoe_knn_download(apoe_knn* g, uint32_t* ids, float* dist) {
     return APOE_OK;
 }
 
+// How many uploaded neighbour ids do not name a document (flag bits count as such).
+__global__ __launch_bounds__(256) static void knn_count_bad_kernel(uint32_t n, uint64_t total, const uint32_t* ids, unsigned long long* bad) {
+    unsigned long long mine = 0;
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (uint64_t)gridDim.x * blockDim.x) mine += ids[t] >= n;
+    if (mine) atomicAdd(bad, mine);
+}
+
+__global__ __launch_bounds__(256) static void rev_reset_kernel(uint32_t n, uint32_t K, unsigned long long* rev, uint32_t* rev_cnt) {
+    const uint64_t total = (uint64_t)n * K;
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (uint64_t)gridDim.x * blockDim.x) {
+        rev[t] = ~0ull;
+        if (t < n) rev_cnt[t] = 0;
+    }
+}
+
+// The steps index other nodes' lists and reverse lists with whatever a list holds, so an id that names no
+// document is refused here; the reverse lists start empty, as after apoe_nnd_init. A refused upload leaves
+// the handle as it was.
 int apoe_knn_upload(apoe_knn* g, const uint32_t* ids, const float* dist) {
     APOE_REQUIRE(g && ids && dist, "null argument");
     APOE_HIP(hipSetDevice(g->ctx->device));
+    hipStream_t st = g->ctx->stream;
     const size_t total = (size_t)g->n * g->K;
-    APOE_TRY(copy_in(g->ctx, g->ids.p, ids, total * sizeof(uint32_t)));
+    DevBuf<uint32_t> tmp;
+    APOE_TRY(tmp.alloc(total));
+    APOE_TRY(copy_in(g->ctx, tmp.p, ids, total * sizeof(uint32_t)));
+    APOE_HIP(hipMemsetAsync(g->counter.p + 1, 0, sizeof(unsigned long long), st));
+    const uint32_t grid = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 16);
+    knn_count_bad_kernel<<<grid, 256, 0, st>>>(g->n, total, tmp.p, g->counter.p + 1);
+    APOE_HIP(hipGetLastError());
+    unsigned long long bad = 0;
+    APOE_TRY(copy_out(g->ctx, &bad, g->counter.p + 1, sizeof(bad)));
+    APOE_REQUIRE(bad == 0, "%llu uploaded neighbour ids are not below the %u documents of the corpus", bad, g->n);
+    APOE_HIP(hipMemcpyAsync(g->ids.p, tmp.p, total * sizeof(uint32_t), hipMemcpyDeviceToDevice, st));
     APOE_TRY(copy_in(g->ctx, g->dist.p, dist, total * sizeof(float)));
+    rev_reset_kernel<<<grid, 256, 0, st>>>(g->n, g->K, g->rev.p, g->rev_cnt.p);
+    APOE_HIP(hipGetLastError());
     APOE_TRY(launch_norms(g->ctx, g->corpus, g->dense_scale, g->norms.p));
-    APOE_HIP(hipStreamSynchronize(g->ctx->stream));
+    APOE_HIP(hipStreamSynchronize(st));
+    g->ready = true;
     g->pruned = false;
     return APOE_OK;
 }

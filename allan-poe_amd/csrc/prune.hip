@@ -689,6 +689,7 @@ extern "C" {
 int apoe_prune(apoe_knn* g, uint32_t degree) {
     APOE_REQUIRE(g, "null argument");
     APOE_REQUIRE(degree >= 2 && degree <= 64 && degree % 2 == 0 && degree <= g->K, "degree must be even, in [2, 64] and <= K, got %u", degree);
+    APOE_REQUIRE_STATE(g->ready, "the lists are empty: call apoe_nnd_init or apoe_knn_upload first");
     APOE_HIP(hipSetDevice(g->ctx->device));
     g->degree = degree;
     APOE_TRY(g->fwd.alloc((size_t)g->n * degree));

@@ -845,7 +845,7 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     APOE_REQUIRE(g->n == c->n, "graph has %u nodes but the corpus has %u documents", g->n, c->n);
     APOE_REQUIRE(p->q_begin <= q->n, "q_begin %u beyond %u queries", p->q_begin, q->n);
     const uint32_t q_count = p->q_count ? p->q_count : q->n - p->q_begin;
-    APOE_REQUIRE(p->q_begin + q_count <= q->n, "query range [%u,%u) beyond %u queries", p->q_begin, p->q_begin + q_count, q->n);
+    APOE_REQUIRE(q_count <= q->n - p->q_begin, "query range of %u from %u beyond %u queries", q_count, p->q_begin, q->n);
     if (stats) *stats = apoe_search_stats{};
     if (q_count == 0) return APOE_OK;
 

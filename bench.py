@@ -103,7 +103,7 @@ def main():
     ap.add_argument("--cpu-queries", type=int, default=10000)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--no-membench", action="store_true", help="do not run allan-poe_amd/membench for roofline.random_read_ceiling")
+    ap.add_argument("--no-membench", action="store_true", help="do not run bench/membench for roofline.random_read_ceiling")
     ap.add_argument("--extras", action="store_true",
                     help="also time the other search paths at cands=128: the query-time weight sweep, the knowledge-graph search "
                          "(200k entities, 1-3 entities per query, kg_weight 40) and the keyword-filter search (rarest BM25 term of each query)")
@@ -374,7 +374,7 @@ def main():
                      "equivalent_if_every_evaluation_read_its_dense_row": {"bytes_per_launch": full_bytes,
                                                                             "gbs": full_bytes / (avg_kernel_ms / 1e3) / 1e9},
                      "every_dense_row_read": full_eval,
-                     # what this GPU gives a kernel that does nothing but such loads (allan-poe_amd/membench, run now)
+                     # what this GPU gives a kernel that does nothing but such loads (bench/membench, run now)
                      "random_read_ceiling": None if args.no_membench else membench()},
         "cpu_baseline": cpu,
     }
@@ -384,7 +384,7 @@ def main():
 def membench():
     """GB/s of random 128-byte aligned chunk reads on this GPU, by chunk size, with nothing but the loads in the kernel:
     the ceiling of a gather of records (the search reads about 1.1 KB per evaluation, 5.2 KB when it needs the dense row)."""
-    exe = os.path.join(ROOT, "allan-poe_amd", "membench")
+    exe = os.path.join(ROOT, "bench", "membench")
     if not os.path.exists(exe):
         return None
     try:

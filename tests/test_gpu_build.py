@@ -236,3 +236,45 @@ def test_prune_k128_sequential_kernel_matches_oracle(gpu_world):
     assert rows.shape == (C.n, 72)
     graph.close()
     knn.close()
+
+
+def test_upload_refuses_ids_beyond_the_corpus_and_calls_out_of_order(gpu_world):
+    """An uploaded list is indexed by later steps: an id that names no document is an error, not a read past
+    the arrays; steps on a handle whose lists were never filled are a call-sequence error."""
+    import apoe
+    w = gpu_world
+    n = w["C"].n
+    knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+    with pytest.raises(apoe.ApoeError, match="status -3"):
+        knn.iterate()
+    with pytest.raises(apoe.ApoeError, match="status -3"):
+        knn.merge_reverse()
+    with pytest.raises(apoe.ApoeError, match="status -3"):
+        knn.prune(32)
+    knn.init(9)
+    good_ids, good_dist = knn.download()
+    for bad in (n, 0x7FFFFFFF, 0xFFFFFFFF, 5 | 0x80000000):
+        ids = good_ids.copy()
+        ids[n // 2, 17] = bad
+        with pytest.raises(apoe.ApoeError, match="not below"):
+            knn.upload(ids, good_dist)
+        assert np.array_equal(knn.download()[0], good_ids)  # a refused upload changes nothing
+    knn.upload(good_ids, good_dist)
+    knn.iterate(last=True)   # reverse lists start empty after an upload: this step and the merge index them
+    knn.merge_reverse()
+    ids, dist = knn.download()
+    assert ids.max() < n and np.all(np.diff(dist, axis=1) >= 0)
+    knn.close()
+
+
+def test_search_refuses_a_query_range_that_wraps(gpu_world):
+    """q_begin + q_count wraps in 32 bits: the C-ABI must refuse it before it sizes anything from it."""
+    import ctypes as C
+    import apoe
+    w = gpu_world
+    ids = np.empty((1, 16), np.uint32)
+    dist = np.empty((1, 16), np.float32)
+    p = apoe.SearchParams(1.0, 1.0, 1.0, 0.0, 16, 0, 3, 0xFFFFFFFE, 0, 0)
+    assert apoe.lib().apoe_search(w["ctx"].h, w["gc"].h, w["gq"].h, w["gg"].h, C.c_void_p(0), C.byref(p), C.c_void_p(ids.ctypes.data),
+                                  C.c_void_p(dist.ctypes.data), C.c_void_p(0)) == -1
+    assert b"beyond" in apoe.lib().apoe_last_error_string()

@@ -1,4 +1,4 @@
-"""allan-poe_amd/membench runs and reports sane ceilings (needs the GPU): what bench.py puts beside its roofline."""
+"""bench/membench runs and reports sane ceilings (needs the GPU): what bench.py puts beside its roofline."""
 import os
 import re
 import subprocess
@@ -7,11 +7,11 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-EXE = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "allan-poe_amd", "membench")
+EXE = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench", "membench")
 
 
 def test_membench_reports_chunk_read_rates():
-    assert os.path.exists(EXE), "membench is not built: make -C allan-poe_amd/csrc"
+    assert os.path.exists(EXE), "membench is not built: make -C bench"
     out = subprocess.run([EXE], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stderr
     rates = {int(m.group(1)): float(m.group(2)) for m in re.finditer(r"random reads,\s+(\d+) B chunks, .*:\s+(\d+) GB/s", out.stdout)}
