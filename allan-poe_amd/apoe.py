@@ -42,7 +42,7 @@ EXPORTS = [
     "apoe_knn_create", "apoe_knn_destroy", "apoe_knn_use_half_rows", "apoe_nnd_init", "apoe_nnd_iterate", "apoe_nnd_merge_reverse",
     "apoe_knn_download", "apoe_knn_upload", "apoe_prune", "apoe_prune_download", "apoe_finalize_graph",
     "apoe_knn_elapsed_ms", "apoe_knn_counters", "apoe_graph_create", "apoe_graph_destroy", "apoe_graph_info", "apoe_graph_download",
-    "apoe_search",
+    "apoe_search", "apoe_search_noalloc",
 ]
 
 
@@ -376,3 +376,17 @@ def search(ctx, corpus, queries, graph, w3, cands, kg=None, kg_weight=0.0, max_i
     _check(lib().apoe_search(ctx.h, corpus.h, queries.h, graph.h, kg.h if kg is not None else C.c_void_p(0), C.byref(p), ki[1], kd[1],
                              C.byref(st)))
     return out_ids, out_dist, st
+
+
+def search_noalloc(ctx, corpus, queries, graph, w3, cands, out_ids, out_dist, kg=None, kg_weight=0.0, max_iter=0, q_begin=0, q_count=0,
+                   variant=0, keyword_filter=False, want_stats=True):
+    """apoe_search_noalloc: the search with a static device workspace; out_ids / out_dist are device tensors
+    [q, cands] that the kernels write in place. Without stats the call does not wait for the GPU."""
+    nq = q_count if q_count else queries.n - q_begin
+    assert tuple(out_ids.shape) == (nq, cands) and tuple(out_dist.shape) == (nq, cands) and out_ids.is_contiguous() and out_dist.is_contiguous()
+    ki, kd = _ptr(out_ids, np.uint32), _ptr(out_dist, np.float32)
+    p = SearchParams(w3[0], w3[1], w3[2], kg_weight, cands, max_iter, q_begin, q_count, variant, 1 if keyword_filter else 0)
+    st = SearchStats() if want_stats else None
+    _check(lib().apoe_search_noalloc(ctx.h, corpus.h, queries.h, graph.h, kg.h if kg is not None else C.c_void_p(0), C.byref(p), ki[1], kd[1],
+                                     C.byref(st) if want_stats else C.c_void_p(0)))
+    return st

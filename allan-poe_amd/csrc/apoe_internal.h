@@ -88,6 +88,7 @@ struct apoe_ctx {
     // request and is kept until the context is destroyed, so that repeated searches do not pay for
     // a device allocation each. One search at a time per context.
     apoe::DevBuf<char> search_ws;
+    char* static_ws = nullptr; // this GPU's copy of the static workspace of apoe_search_noalloc
     int search_workspace(size_t bytes, char** out) {
         if (search_ws.n < bytes) APOE_TRY(search_ws.alloc(bytes));
         *out = search_ws.p;
@@ -167,7 +168,8 @@ int launch_distance_pairs(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale
                           uint32_t n_pairs, float* out_dev);
 int launch_norms(apoe_ctx* ctx, const apoe_corpus* c, float dense_scale, float* out_dev);
 int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g, const apoe_kg* kg,
-                  const apoe_search_params* p, uint32_t* out_ids_dev, float* out_dist_dev, apoe_search_stats* stats);
+                  const apoe_search_params* p, uint32_t* out_ids_dev, float* out_dist_dev, apoe_search_stats* stats, char* static_ws);
+int search_static_workspace(int device, char** out); // device address of the static search workspace on that GPU
 int launch_nnd_init(apoe_knn* g, uint64_t seed);
 int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted);
 int launch_nnd_merge_reverse(apoe_knn* g);

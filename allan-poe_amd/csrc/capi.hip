@@ -108,6 +108,10 @@ int apoe_ctx_create(int device, apoe_ctx** out) {
     ctx->device = device;
     ctx->num_cus = prop.multiProcessorCount;
     ctx->lds_per_block = prop.sharedMemPerBlock;
+    if (search_static_workspace(device, &ctx->static_ws) != APOE_OK) {
+        delete ctx;
+        return APOE_ERR_HIP;
+    }
     if (hipStreamCreate(&ctx->stream) != hipSuccess || hipEventCreate(&ctx->ev0) != hipSuccess || hipEventCreate(&ctx->ev1) != hipSuccess) {
         set_error("could not create the HIP stream/events: %s", hipGetErrorString(hipGetLastError()));
         apoe_ctx_destroy(ctx);
@@ -446,9 +450,19 @@ int apoe_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, cons
     DevOutput<float> d_dist;
     APOE_TRY(d_ids.init(out_ids, (size_t)q_count * p->cands));
     APOE_TRY(d_dist.init(out_dist, (size_t)q_count * p->cands));
-    APOE_TRY(launch_search(ctx, c, q, g, kg, p, d_ids.p, d_dist.p, stats));
+    APOE_TRY(launch_search(ctx, c, q, g, kg, p, d_ids.p, d_dist.p, stats, nullptr));
     APOE_TRY(d_ids.finish(ctx));
     return d_dist.finish(ctx);
+}
+
+int apoe_search_noalloc(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g, const apoe_kg* kg,
+                        const apoe_search_params* p, uint32_t* out_ids, float* out_dist, apoe_search_stats* stats) {
+    APOE_REQUIRE(ctx && c && q && g && p && out_ids && out_dist, "null argument");
+    APOE_HIP(hipSetDevice(ctx->device));
+    APOE_REQUIRE(c->n <= APOE_NOALLOC_MAX_DOCS, "apoe_search_noalloc serves corpora of up to %u documents, this one has %u", (unsigned)APOE_NOALLOC_MAX_DOCS,
+                 c->n);
+    APOE_REQUIRE(is_device_ptr(out_ids) && is_device_ptr(out_dist), "apoe_search_noalloc writes its results in place: out_ids and out_dist must be device memory");
+    return launch_search(ctx, c, q, g, kg, p, out_ids, out_dist, stats, ctx->static_ws);
 }
 
 } // extern "C"

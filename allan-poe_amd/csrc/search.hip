@@ -1,6 +1,8 @@
 // Greedy beam search over the hybrid graph: one workgroup per query; the candidate pool, the
 // query's dense row, its sparse-term tables and the fresh-neighbour list in LDS; an exact
 // visited bitmap per workgroup in HBM.
+#include <mutex>
+
 #include "apoe_internal.h"
 
 namespace apoe {
@@ -799,6 +801,37 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(MODE =
     }
 }
 
+// Counters and once-per-query arguments of a launch, written on the stream (no host copy from a stack frame,
+// no memset node for a caller that records the stream).
+__global__ void search_setup_kernel(unsigned long long* work, SearchCold* dst, SearchCold cold) {
+    if (threadIdx.x < 8) work[threadIdx.x] = 0ull;
+    if (threadIdx.x == 0) *dst = cold;
+}
+
+// Workspace of apoe_search_noalloc: counters, once-per-query arguments and the visited bitmaps of as many
+// workgroups as fit. One copy per GPU, held until the process ends; every call on a GPU uses it, so calls
+// that overlap on one GPU race. Host code never uses the array's name as an address: the device address is
+// asked for once per device (search_static_workspace) and kept.
+static __device__ __align__(256) unsigned char search_scratch[APOE_NOALLOC_WS_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+static std::mutex scratch_mutex;
+static char* scratch_ptr[MAX_DEVICES]; // per device: address of search_scratch on that GPU, null until asked for
+
+int search_static_workspace(int device, char** out) {
+    APOE_REQUIRE(device >= 0 && device < MAX_DEVICES, "device %d outside [0,%d)", device, MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[device]) {
+        APOE_HIP(hipSetDevice(device));
+        void* p = nullptr;
+        APOE_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(search_scratch)));
+        APOE_REQUIRE(p != nullptr, "no device address for the static search workspace on device %d", device);
+        scratch_ptr[device] = static_cast<char*>(p);
+    }
+    *out = scratch_ptr[device];
+    return APOE_OK;
+}
+
 template <int NW, int MODE, bool NARROW, bool HALF = false>
 static int launch_format(apoe_ctx* ctx, const SearchArgs& a, uint32_t grid, size_t lds, int* per_cu) {
     if constexpr (MODE == MODE_PLAIN && !HALF) {
@@ -838,8 +871,10 @@ static int launch_mode(apoe_ctx* ctx, int mode, int nw, const SearchArgs& a, uin
     }
 }
 
+// static_ws: null, or the device address of this GPU's search_scratch: then nothing is allocated, the grid is cut to
+// the bitmaps that fit, and a call without `stats` returns with the work still running on the context's stream.
 int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g, const apoe_kg* kg,
-                  const apoe_search_params* p, uint32_t* out_ids_dev, float* out_dist_dev, apoe_search_stats* stats) {
+                  const apoe_search_params* p, uint32_t* out_ids_dev, float* out_dist_dev, apoe_search_stats* stats, char* static_ws) {
     APOE_REQUIRE(p->cands >= 1 && p->cands <= APOE_MAX_CANDS, "cands must be in 1..%d, got %u", APOE_MAX_CANDS, p->cands);
     APOE_REQUIRE(g->width > APOE_KW_SLOTS && g->width - APOE_KW_SLOTS <= MAX_NEW, "graph degree must be in 1..64, got width %u", g->width);
     APOE_REQUIRE(g->n == c->n, "graph has %u nodes but the corpus has %u documents", g->n, c->n);
@@ -912,21 +947,28 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     int per_cu = 1;
     APOE_TRY(launch_mode(ctx, mode, nw, a, 0, L.total, &per_cu));
     if (per_cu < 1) per_cu = 1;
-    const uint32_t grid = std::min<uint32_t>(q_count, (uint32_t)per_cu * (uint32_t)ctx->num_cus);
+    uint32_t grid = std::min<uint32_t>(q_count, (uint32_t)per_cu * (uint32_t)ctx->num_cus);
 
     a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;
     // workspace: [counters: 8 x u64][once-per-query arguments][visited bitmaps]
     const size_t cold_at = 8 * sizeof(unsigned long long), bitmaps_at = (cold_at + sizeof(SearchCold) + 255) & ~(size_t)255;
-    char* ws = nullptr;
-    APOE_TRY(ctx->search_workspace(bitmaps_at + (size_t)grid * a.bitmap_words * sizeof(uint32_t), &ws));
+    const size_t bitmap_bytes = (size_t)a.bitmap_words * sizeof(uint32_t);
+    char* ws = static_ws;
+    if (static_ws) {
+        const size_t fit = (APOE_NOALLOC_WS_BYTES - bitmaps_at) / bitmap_bytes;
+        APOE_REQUIRE(fit >= 1, "the static workspace of %u bytes holds no visited bitmap of %zu bytes", (unsigned)APOE_NOALLOC_WS_BYTES, bitmap_bytes);
+        grid = (uint32_t)std::min<size_t>(grid, fit);
+    } else {
+        APOE_TRY(ctx->search_workspace(bitmaps_at + (size_t)grid * bitmap_bytes, &ws));
+    }
     unsigned long long* work = reinterpret_cast<unsigned long long*>(ws);
-    APOE_HIP(hipMemcpyAsync(ws + cold_at, &cold, sizeof(cold), hipMemcpyHostToDevice, ctx->stream));
-    APOE_HIP(hipStreamSynchronize(ctx->stream)); // `cold` lives on this stack frame
+    search_setup_kernel<<<1, WAVE, 0, ctx->stream>>>(work, reinterpret_cast<SearchCold*>(ws + cold_at), cold);
+    APOE_HIP(hipGetLastError());
     a.cold = reinterpret_cast<const SearchCold*>(ws + cold_at);
-    APOE_HIP(hipMemsetAsync(work, 0, 8 * sizeof(unsigned long long), ctx->stream));
     a.bitmaps = reinterpret_cast<uint32_t*>(ws + bitmaps_at);
     a.work = work;
 
+    if (static_ws && !stats) return launch_mode(ctx, mode, nw, a, grid, L.total, nullptr);
     float ms = 0.f;
     APOE_TRY(timed(ctx, &ms, [&]() { return launch_mode(ctx, mode, nw, a, grid, L.total, nullptr); }));
     APOE_HIP(hipStreamSynchronize(ctx->stream));

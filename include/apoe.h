@@ -217,6 +217,25 @@ int apoe_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, cons
                 const apoe_kg* kg, const apoe_search_params* p, uint32_t* out_ids, float* out_dist,
                 apoe_search_stats* stats);
 
+/*
+ * apoe_search without any allocation. No counterpart in the reference: it is for callers that cannot
+ * allocate device memory -- code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc. Same kernels, arguments and results as apoe_search, except that
+ *  - out_ids / out_dist must be device memory of the context's GPU (results are written in place);
+ *  - the counters, the once-per-query arguments and the visited bitmaps live in one static device array of
+ *    APOE_NOALLOC_WS_BYTES that each GPU holds from the first apoe_ctx_create on it until the process
+ *    ends; the launch uses as many workgroups as bitmaps of n bits fit there (255 at 1 M documents), so a
+ *    large batch runs slower than through apoe_search; corpora above APOE_NOALLOC_MAX_DOCS are refused;
+ *  - with stats == NULL the call returns with the search still running on the context's stream
+ *    (apoe_ctx_synchronize waits for it); with stats it blocks like apoe_search;
+ *  - all calls on one GPU share that array: calls that overlap on a GPU (two contexts, two threads) race.
+ */
+#define APOE_NOALLOC_WS_BYTES (32u << 20)
+#define APOE_NOALLOC_MAX_DOCS (1u << 21)
+int apoe_search_noalloc(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, const apoe_graph* g,
+                        const apoe_kg* kg, const apoe_search_params* p, uint32_t* out_ids, float* out_dist,
+                        apoe_search_stats* stats);
+
 #ifdef __cplusplus
 }
 #endif
