@@ -53,7 +53,8 @@ def build(force=False):
 def lib():
     global _LIB
     if _LIB is None:
-        so = os.path.join(_HERE, "liboracle.so")
+        # APOE_ORACLE_LIB names another build of the same sources (the sanitizer build of `make asan`)
+        so = os.environ.get("APOE_ORACLE_LIB") or os.path.join(_HERE, "liboracle.so")
         if not os.path.exists(so):
             build()
         _LIB = C.CDLL(so)
