@@ -39,7 +39,7 @@ EXPORTS = [
     "apoe_last_error_string", "apoe_ctx_create", "apoe_ctx_destroy", "apoe_ctx_synchronize", "apoe_corpus_create",
     "apoe_corpus_destroy", "apoe_corpus_info", "apoe_corpus_bytes", "apoe_corpus_pair_bytes", "apoe_corpus_make_half_rows", "apoe_queries_create", "apoe_queries_destroy",
     "apoe_kg_create", "apoe_kg_destroy", "apoe_calibrate_weights", "apoe_hybrid_distance_batch", "apoe_hybrid_distance_pairs", "apoe_norms",
-    "apoe_knn_create", "apoe_knn_destroy", "apoe_knn_use_half_rows", "apoe_nnd_init", "apoe_nnd_iterate", "apoe_nnd_merge_reverse",
+    "apoe_knn_create", "apoe_knn_destroy", "apoe_knn_use_half_rows", "apoe_knn_set_join", "apoe_nnd_init", "apoe_nnd_iterate", "apoe_nnd_merge_reverse",
     "apoe_knn_download", "apoe_knn_upload", "apoe_prune", "apoe_prune_download", "apoe_finalize_graph",
     "apoe_knn_elapsed_ms", "apoe_knn_counters", "apoe_graph_create", "apoe_graph_destroy", "apoe_graph_info", "apoe_graph_download",
     "apoe_search", "apoe_search_noalloc",
@@ -243,6 +243,10 @@ class Knn:
         """NN-Descent steps on the half-precision rows; merge_reverse() then recomputes the stored distances in fp32."""
         _check(lib().apoe_knn_use_half_rows(self.h, C.c_int(1 if on else 0)))
 
+    def set_join(self, mode):
+        """0: the reference's expansion step; 1: local join around the picked neighbour; 2: the same, both endpoints updated."""
+        _check(lib().apoe_knn_set_join(self.h, C.c_int(mode)))
+
     def init(self, seed):
         _check(lib().apoe_nnd_init(self.h, C.c_uint64(seed)))
 
@@ -303,9 +307,11 @@ class Knn:
             pass
 
 
-def build_graph(ctx, corpus, K=64, iters=25, degree=32, dense_scale=7.0, seed=1, half_rows=False):
+def build_graph(ctx, corpus, K=64, iters=25, degree=32, dense_scale=7.0, seed=1, half_rows=False, join=0):
     """NN-Descent + reverse merge + prune + final assembly; returns (Graph, gpu_ms)."""
     knn = Knn(ctx, corpus, K, dense_scale)
+    if join:
+        knn.set_join(join)
     if half_rows:
         corpus.make_half_rows()
         knn.use_half_rows()

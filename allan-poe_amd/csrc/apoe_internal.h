@@ -99,6 +99,7 @@ struct apoe_ctx {
 struct apoe_corpus {
     apoe_ctx* ctx = nullptr;
     uint32_t n = 0, dim = 0, max_nnz_s = 0, max_nnz_b = 0;
+    uint32_t max_term = 0; // largest term id of either path
     uint64_t rec_bytes = 0, total_pairs = 0;
     bool narrow = false; // pair format of the records (6 instead of 8 bytes a pair when every term id is below 65536)
     apoe::DevBuf<uint64_t> desc;
@@ -146,6 +147,12 @@ struct apoe_knn {
     apoe::DevBuf<unsigned long long> rev; // [n][K] reverse lists: (distance key << 32 | id) per slot
     apoe::DevBuf<float> dist, norms;
     apoe::DevBuf<unsigned long long> counter;
+    // local-join step (apoe_knn_set_join): the picks of a step grouped by the picked node, the tiles, the proposal rows
+    int join = 0; // 0: expansion step, 1: local join, 2: local join that offers a pair to both endpoints
+    bool join_symmetric = false;
+    apoe::DevBuf<uint32_t> picks, pick_cnt, pick_off, pick_fill, pick_src, tile_cnt, tile_off, tile_v;
+    apoe::DevBuf<unsigned long long> prop, join_work;
+    apoe::DevBuf<char> scan_tmp;
     // prune outputs
     apoe::DevBuf<uint32_t> fwd, det, cnt, kw;
 };
@@ -172,6 +179,8 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
 int search_static_workspace(int device, char** out); // device address of the static search workspace on that GPU
 int launch_nnd_init(apoe_knn* g, uint64_t seed);
 int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted);
+int launch_nnd_join_iterate(apoe_knn* g);
+int join_step_counters(apoe_knn* g, unsigned long long* out3);
 int launch_nnd_merge_reverse(apoe_knn* g);
 int launch_prune(apoe_knn* g, uint32_t degree);
 int launch_final_graph(apoe_knn* g, uint32_t* rows_dev);

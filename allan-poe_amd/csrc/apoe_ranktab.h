@@ -1,0 +1,291 @@
+// Sparse inner products of many rows against a small group of pivot rows at once: the pivots' terms go
+// into ONE LDS table that is addressed through a bitmap with running counts (a "rank table"), and every
+// other row then looks each of its pairs up exactly once for the whole group.
+//
+//   word[w] = (bits, count of set bits in words before w)      one ds_read_b64 per look-up
+//   slot of a term = count + popcount(bits below its bit)      no hashing, no probe loop, no key compare
+//   vals[slot] = one value per pivot of the group (zero where the pivot lacks the term): one ds_read_b128
+//
+// A corpus in the narrow pair format (term ids below 65536, the path known from the position in the row)
+// maps a term to bit (term | path * span) with span = the power of two above the largest term id: distinct
+// terms have distinct bits, the table is a perfect hash and a miss costs one 8-byte read whose 64 lanes
+// mostly fall into different banks. Wide corpora hash the 32-bit key to a bit; two terms of a group that
+// fall on one bit are told apart by the stored key and the loser goes to a short overflow list.
+#pragma once
+
+#include "apoe_device.h"
+
+namespace apoe {
+
+#ifdef __HIPCC__
+
+constexpr int RT_T = 4;     // pivots per table: one float4 per term
+constexpr int RT_OVF = 32;  // overflow entries (wide corpora only)
+
+struct RankTabLds { // byte offsets inside the table region
+    uint32_t word, keys, vals, ovf_key, ovf_val, total;
+    __host__ __device__ RankTabLds(uint32_t index_bits, uint32_t slot_cap, bool narrow) {
+        uint32_t o = 0;
+        vals = o; o += slot_cap * RT_T * 4;
+        word = o; o += (index_bits / 32) * 8;
+        keys = o; o += narrow ? 0 : slot_cap * 4;
+        ovf_key = o; o += narrow ? 0 : RT_OVF * 4;
+        o = (o + 15) & ~15u;
+        ovf_val = o; o += narrow ? 0 : RT_OVF * RT_T * 4;
+        total = o;
+    }
+};
+
+struct RankTab {
+    uint2* word;      // [index_bits / 32]
+    uint32_t* keys;   // [slot_cap], wide only
+    float4* vals;     // [slot_cap]
+    uint32_t* ovf_key;
+    float4* ovf_val;
+    uint32_t index_bits, slot_cap;
+    uint32_t span; // narrow: bit index of a BM25 term = term + span
+};
+
+__device__ __forceinline__ RankTab ranktab_at(char* region, uint32_t index_bits, uint32_t slot_cap, uint32_t span, bool narrow) {
+    const RankTabLds L(index_bits, slot_cap, narrow);
+    RankTab T;
+    T.word = reinterpret_cast<uint2*>(region + L.word);
+    T.keys = reinterpret_cast<uint32_t*>(region + L.keys);
+    T.vals = reinterpret_cast<float4*>(region + L.vals);
+    T.ovf_key = reinterpret_cast<uint32_t*>(region + L.ovf_key);
+    T.ovf_val = reinterpret_cast<float4*>(region + L.ovf_val);
+    T.index_bits = index_bits;
+    T.slot_cap = slot_cap;
+    T.span = span;
+    return T;
+}
+
+// Bit index of a pair. key: raw key as the record load delivers it (narrow: the 16-bit term; wide: term | path bit).
+template <bool NARROW>
+__device__ __forceinline__ uint32_t ranktab_index(const RankTab& T, uint32_t key, bool bm25) {
+    if (NARROW) return key + (bm25 ? T.span : 0u);
+    const uint32_t k = key ^ (key >> 15);
+    return ((k * 0x9E3779B1u) >> 12) & (T.index_bits - 1);
+}
+
+// Builds the table of pivots [0, nt) (nt <= RT_T); pivot(t) gives the Pairs of pivot t. All threads of the block
+// call it (the block size is a multiple of 64, at most 1024); `scan` is LDS scratch of 20 words. Returns the
+// number of distinct terms, or EMPTY if they exceed the slot capacity or the overflow list (the table is then
+// unusable: the caller retries with fewer pivots). Ends with a barrier: the table is ready on return.
+template <bool NARROW, typename PivotFn>
+__device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivot, uint32_t nt, uint32_t* scan, int tid, int nthreads) {
+    const uint32_t W = T.index_bits / 32;
+    const int lane = tid & (WAVE - 1), wave = tid / WAVE, nwaves = nthreads / WAVE;
+    for (uint32_t w = tid; w < W; w += nthreads) T.word[w] = make_uint2(0u, 0u);
+    if (tid == 0) scan[16] = 0; // overflow count
+    __syncthreads();
+    // 1. bits
+    for (uint32_t t = 0; t < nt; t++) {
+        const Pairs sp = pivot(t);
+        for (uint32_t j = tid; j < sp.nnz; j += nthreads) {
+            const uint32_t idx = ranktab_index<NARROW>(T, NARROW ? sp.raw(j).x : sp.key(j), j >= sp.ns);
+            atomicOr(&T.word[idx >> 5].x, 1u << (idx & 31));
+        }
+    }
+    __syncthreads();
+    // 2. running counts: thread i owns the words [i * per, (i + 1) * per)
+    const uint32_t per = (W + nthreads - 1) / nthreads;
+    uint32_t mine = 0;
+    for (uint32_t k = 0; k < per; k++) {
+        const uint32_t w = tid * per + k;
+        if (w < W) mine += __popc(T.word[w].x);
+    }
+    uint32_t incl = mine;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const uint32_t up = __shfl_up(incl, o, WAVE);
+        if (lane >= o) incl += up;
+    }
+    if (lane == WAVE - 1) scan[wave] = incl;
+    __syncthreads();
+    uint32_t before = incl - mine, total = 0;
+    for (int w = 0; w < nwaves; w++) {
+        const uint32_t s = scan[w];
+        if (w < wave) before += s;
+        total += s;
+    }
+    if (total > T.slot_cap) {
+        __syncthreads();
+        return EMPTY;
+    }
+    for (uint32_t k = 0; k < per; k++) {
+        const uint32_t w = tid * per + k;
+        if (w < W) {
+            T.word[w].y = before;
+            before += __popc(T.word[w].x);
+        }
+    }
+    for (uint32_t s = tid; s < total; s += nthreads) {
+        T.vals[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (!NARROW) T.keys[s] = EMPTY;
+    }
+    if (!NARROW) {
+        for (uint32_t s = tid; s < RT_OVF; s += nthreads) { T.ovf_key[s] = EMPTY; T.ovf_val[s] = make_float4(0.f, 0.f, 0.f, 0.f); }
+    }
+    __syncthreads();
+    // 3. values (and keys)
+    for (uint32_t t = 0; t < nt; t++) {
+        const Pairs sp = pivot(t);
+        for (uint32_t j = tid; j < sp.nnz; j += nthreads) {
+            const uint2 kv = NARROW ? sp.raw(j) : sp[j];
+            const uint32_t idx = ranktab_index<NARROW>(T, kv.x, j >= sp.ns);
+            const uint2 w = T.word[idx >> 5];
+            const uint32_t slot = w.y + __popc(w.x & ((1u << (idx & 31)) - 1u));
+            if (NARROW) {
+                reinterpret_cast<uint32_t*>(&T.vals[slot])[t] = kv.y;
+            } else {
+                const uint32_t old = atomicCAS(&T.keys[slot], EMPTY, kv.x);
+                if (old == EMPTY || old == kv.x) {
+                    reinterpret_cast<uint32_t*>(&T.vals[slot])[t] = kv.y;
+                } else { // another term of the group sits on this bit
+                    uint32_t at = EMPTY;
+                    for (uint32_t s = 0; s < RT_OVF; s++) {
+                        const uint32_t o = atomicCAS(&T.ovf_key[s], EMPTY, kv.x);
+                        if (o == EMPTY) atomicAdd(&scan[16], 1u);
+                        if (o == EMPTY || o == kv.x) { at = s; break; }
+                    }
+                    if (at != EMPTY) reinterpret_cast<uint32_t*>(&T.ovf_val[at])[t] = kv.y;
+                    else atomicAdd(&scan[16], RT_OVF + 1u);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (!NARROW && scan[16] > RT_OVF) return EMPTY;
+    return total;
+}
+
+// One pair against the table: acc[t] += value * (pivot t's value of the term). `in` = the lane holds a pair.
+// The value slot is read whatever the bitmap says (a miss reads slot 0 with multiplier zero): the reads of several
+// pairs can then be issued together, and the 64 lanes of a miss read one address, which LDS serves as a broadcast.
+struct RankProbe {
+    uint32_t slot;
+    float mul;
+};
+template <bool NARROW>
+__device__ __forceinline__ RankProbe ranktab_locate(const RankTab& T, uint2 w, uint32_t idx, uint32_t val_bits, bool in) {
+    const bool hit = in && ((w.x >> (idx & 31)) & 1u);
+    RankProbe p;
+    p.slot = hit ? w.y + __popc(w.x & ((1u << (idx & 31)) - 1u)) : 0u;
+    p.mul = hit ? __uint_as_float(val_bits) : 0.f;
+    return p;
+}
+
+// Sum of four per-lane accumulators over the wave, all four at once: after two exchange-and-add steps inside
+// each quad, lane l holds pivot t(l) = 2 * (l & 1) + ((l >> 1) & 1) summed over its quad; then one sum per lane.
+// Returns that pivot's total in every lane whose (l & 3) names it; *t_out = the pivot this lane holds.
+__device__ __forceinline__ float wave_sum4_dpp(const float acc[4], int lane, uint32_t* t_out) {
+    const bool odd = lane & 1, hi = lane & 2;
+    const float keep0 = odd ? acc[2] : acc[0], keep1 = odd ? acc[3] : acc[1];
+    const float give0 = odd ? acc[0] : acc[2], give1 = odd ? acc[1] : acc[3];
+    const float x0 = keep0 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give0), 0xB1, 0xF, 0xF, false));
+    const float x1 = keep1 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give1), 0xB1, 0xF, 0xF, false));
+    const float keep = hi ? x1 : x0, give = hi ? x0 : x1;
+    float z = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give), 0x4E, 0xF, 0xF, false));
+    z += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, z), 0x124, 0xF, 0xF, false)); // row_ror:4
+    z += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, z), 0x128, 0xF, 0xF, false)); // row_ror:8
+    z += __shfl_xor(z, 16, WAVE);
+    z += __shfl_xor(z, 32, WAVE);
+    *t_out = 2u * (lane & 1) + ((lane >> 1) & 1);
+    return z;
+}
+
+constexpr int RT_CHUNKS = 5; // 64-pair chunks of a streamed row kept in registers (320 pairs); longer rows loop
+
+struct RtRow { // raw pairs of a streamed row
+    uint2 kv[RT_CHUNKS];
+};
+__device__ __forceinline__ void rt_row_load(RtRow& r, const Pairs& sp, int lane) {
+#pragma unroll
+    for (int c = 0; c < RT_CHUNKS; c++) {
+        const uint32_t j = c * WAVE + lane;
+        r.kv[c] = j < sp.nnz ? sp.raw(j) : make_uint2(0u, 0u);
+    }
+}
+
+// The streamed row `cur` (nnz pairs, ns of them SPLADE; sp gives the pairs beyond the register window) against
+// the table: acc[0..3] += per-pivot sums of this lane's pairs.
+template <bool NARROW>
+__device__ __forceinline__ void ranktab_probe_row(const RankTab& T, const RtRow& cur, const Pairs& sp, uint32_t n_ovf, float acc[4], int lane) {
+    const uint32_t nnz = sp.nnz, ns = sp.ns;
+    auto overflow = [&](uint32_t key, uint32_t val_bits, bool in) {
+        for (uint32_t o = 0; o < n_ovf; o++) { // wave-uniform count, zero for narrow corpora
+            if (in && T.ovf_key[o] == key) {
+                const float4 v = T.ovf_val[o];
+                const float val = __uint_as_float(val_bits);
+                acc[0] = fmaf(val, v.x, acc[0]);
+                acc[1] = fmaf(val, v.y, acc[1]);
+                acc[2] = fmaf(val, v.z, acc[2]);
+                acc[3] = fmaf(val, v.w, acc[3]);
+            }
+        }
+    };
+    auto key_of = [&](uint2 kv, uint32_t j) -> uint32_t { return NARROW ? kv.x : kv.x; };
+    // the first three chunks as one batch: three bitmap reads, then three value reads
+    {
+        uint32_t idx[3];
+        uint2 w[3];
+        bool in[3];
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            const uint32_t j = c * WAVE + lane;
+            in[c] = j < nnz;
+            idx[c] = ranktab_index<NARROW>(T, key_of(cur.kv[c], j), NARROW ? j >= ns : (int)cur.kv[c].x < 0);
+            w[c] = T.word[in[c] ? idx[c] >> 5 : 0u];
+        }
+        asm volatile("" : "+v"(w[0].x), "+v"(w[1].x), "+v"(w[2].x));
+        RankProbe p[3];
+        float4 v[3];
+        bool ok[3];
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            p[c] = ranktab_locate<NARROW>(T, w[c], idx[c], cur.kv[c].y, in[c]);
+            v[c] = T.vals[p[c].slot];
+            ok[c] = true;
+            if (!NARROW) ok[c] = p[c].mul == 0.f || T.keys[p[c].slot] == cur.kv[c].x;
+        }
+        asm volatile("" : "+v"(v[0].x), "+v"(v[1].x), "+v"(v[2].x));
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            const float m = ok[c] ? p[c].mul : 0.f;
+            acc[0] = fmaf(m, v[c].x, acc[0]);
+            acc[1] = fmaf(m, v[c].y, acc[1]);
+            acc[2] = fmaf(m, v[c].z, acc[2]);
+            acc[3] = fmaf(m, v[c].w, acc[3]);
+        }
+        if (!NARROW && n_ovf) {
+#pragma unroll
+            for (int c = 0; c < 3; c++) overflow(cur.kv[c].x, cur.kv[c].y, in[c] && !ok[c]);
+        }
+    }
+    auto one = [&](uint2 kv, uint32_t j, bool in) {
+        const uint32_t idx = ranktab_index<NARROW>(T, kv.x, NARROW ? j >= ns : (int)kv.x < 0);
+        const uint2 w = T.word[in ? idx >> 5 : 0u];
+        const RankProbe p = ranktab_locate<NARROW>(T, w, idx, kv.y, in);
+        const float4 v = T.vals[p.slot];
+        bool ok = true;
+        if (!NARROW) ok = p.mul == 0.f || T.keys[p.slot] == kv.x;
+        const float m = ok ? p.mul : 0.f;
+        acc[0] = fmaf(m, v.x, acc[0]);
+        acc[1] = fmaf(m, v.y, acc[1]);
+        acc[2] = fmaf(m, v.z, acc[2]);
+        acc[3] = fmaf(m, v.w, acc[3]);
+        if (!NARROW && n_ovf) overflow(kv.x, kv.y, in && !ok);
+    };
+#pragma unroll
+    for (int c = 3; c < RT_CHUNKS; c++)
+        if (c * WAVE < (int)nnz) one(cur.kv[c], c * WAVE + lane, (uint32_t)(c * WAVE + lane) < nnz); // wave-uniform branch
+    for (uint32_t j0 = RT_CHUNKS * WAVE; j0 < nnz; j0 += WAVE) { // rows longer than the register window
+        const uint32_t j = j0 + lane;
+        one(j < nnz ? sp.raw(j) : make_uint2(0u, 0u), j, j < nnz);
+    }
+}
+
+#endif // __HIPCC__
+
+} // namespace apoe

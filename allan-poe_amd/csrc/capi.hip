@@ -178,6 +178,7 @@ int apoe_corpus_create(apoe_ctx* ctx, uint32_t n, uint32_t dim, const float* den
         // bit 31 is the path bit of a stored key, and a BM25 key of all ones would read as an empty table slot
         APOE_REQUIRE(max_term < BM25_BIT - 1, "term id %u does not fit 31 bits (the largest usable id is %u)", max_term, BM25_BIT - 2);
         c->narrow = max_term < 65536u;
+        c->max_term = max_term;
         std::vector<uint64_t> desc(n);
         uint64_t off16 = 0;
         for (uint32_t i = 0; i < n; i++) {

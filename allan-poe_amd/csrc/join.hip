@@ -1,0 +1,450 @@
+// NN-Descent step as a local join around the picked neighbour (K = 64).
+//
+// The reference's step (index.cu:156-376) lets node u meet the forward list N(v) and the reverse list R(v) of
+// each neighbour v it picks: one pivot against many rows, every row gathered for one evaluation. Here the same
+// pairs are formed the other way round: all pickers of one v are the ROWS of a tile (32 at a time), N(v) and R(v)
+// are its COLUMNS (up to 128), every row of the tile is gathered once and meets every column:
+//   dense part   32 x 128 x 1024 contraction on the matrix cores (fp32 MFMA 32x32x2, one 32-column block per wave)
+//   sparse part  four picker rows at a time in an LDS rank table that the column rows probe (apoe_ranktab.h)
+//   insertion    a pair closer than the row's last list entry (and not in that list) is offered to the row node
+//                with a 64-bit atomicMin on slot hash(id) of its proposal row: (distance, id), the smallest wins;
+//                in symmetric mode the pair is offered to the column node as well (both endpoints, as the classic
+//                NN-Descent join does; the reference's step updates u only)
+// and a second kernel merges every node's proposals into its sorted list (wave-level rank merge, new before old
+// on equal distance, index.cu:333-351) and registers reverse edges as the expansion step does (index.cu:362-372).
+// Lists are read as the step found them, proposals are minima under a total order: the step does not depend on
+// the order in which tiles run.
+#include <hipcub/hipcub.hpp>
+
+#include <algorithm>
+
+#include "apoe_gram.h"
+#include "apoe_internal.h"
+#include "apoe_ranktab.h"
+
+namespace apoe {
+
+constexpr int JT_ROWS = 32;
+constexpr int JT_COLS = 128;
+constexpr int JT_THREADS = 256;
+constexpr int JT_STRIDE = JT_COLS + 1;
+constexpr int JT_SEEN = 512; // slots of the id set that removes repeated columns
+constexpr uint32_t JOIN_K = 64;
+constexpr int JOIN_PICKS = 4; // index.cu:157,171-181
+
+__device__ __forceinline__ uint32_t prop_slot(uint32_t id, uint32_t P) { return (uint32_t)(mix64(id) >> 40) & (P - 1); }
+
+__device__ __forceinline__ float join_key_dist(unsigned long long key) {
+    uint32_t u = (uint32_t)(key >> 32);
+    u ^= (u >> 31) ? 0x80000000u : 0xFFFFFFFFu;
+    return __uint_as_float(u);
+}
+
+// One wave per node: the picking rule of the expansion step (group g takes the first unsampled slot >= g; none
+// left: slot 0 again), the picked neighbours counted per target.
+__global__ __launch_bounds__(256) void join_pick_kernel(uint32_t n, uint32_t* ids, uint32_t* picks, uint32_t* pick_cnt) {
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const uint32_t u = blockIdx.x * 4 + wave;
+    if (u >= n) return;
+    const size_t base = (size_t)u * JOIN_K;
+    const uint32_t own = ids[base + lane];
+    uint64_t m0 = __ballot(!(own & FLAG));
+    uint32_t slot[JOIN_PICKS], mine = EMPTY; // everything here is wave-uniform except `mine`: lane g keeps the g-th pick
+#pragma unroll
+    for (int g = 0; g < JOIN_PICKS; g++) {
+        const uint64_t a = m0 & ~((1ull << g) - 1);
+        uint32_t s = 0;
+        if (a) {
+            s = __ffsll((unsigned long long)a) - 1;
+            m0 &= ~(1ull << s);
+            if ((uint32_t)lane == s) ids[base + s] = own | FLAG;
+        }
+        slot[g] = s;
+        bool dup = false;
+#pragma unroll
+        for (int t = 0; t < g; t++) dup |= slot[t] == s;
+        uint32_t v = (uint32_t)__builtin_amdgcn_readlane((int)own, s) & ~FLAG;
+        if (dup || v >= n) v = EMPTY;
+        if (lane == g) mine = v;
+    }
+    if (lane < JOIN_PICKS) {
+        picks[(size_t)u * JOIN_PICKS + lane] = mine;
+        if (mine != EMPTY) atomicAdd(&pick_cnt[mine], 1u);
+    }
+}
+
+__global__ __launch_bounds__(256) void join_tile_count_kernel(uint32_t n, const uint32_t* pick_cnt, uint32_t* tile_cnt) {
+    const uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
+    if (v < n) tile_cnt[v] = (pick_cnt[v] + JT_ROWS - 1) / JT_ROWS;
+    if (v == n) tile_cnt[v] = 0;
+}
+
+// The pickers of every v side by side, and the node of every tile.
+__global__ __launch_bounds__(256) void join_fill_kernel(uint32_t n, const uint32_t* picks, const uint32_t* pick_off, const uint32_t* tile_off,
+                                                        uint32_t* pick_fill, uint32_t* pick_src, uint32_t* tile_v) {
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (uint64_t)n * JOIN_PICKS) return;
+    const uint32_t v = picks[t];
+    if (v == EMPTY) return;
+    const uint32_t k = atomicAdd(&pick_fill[v], 1u);
+    pick_src[pick_off[v] + k] = (uint32_t)(t / JOIN_PICKS);
+    if (k % JT_ROWS == 0) tile_v[tile_off[v] + k / JT_ROWS] = v;
+}
+
+struct JoinArgs {
+    CorpusView C;
+    float dense_mul;
+    uint32_t n, P, symmetric;
+    const uint32_t* ids;
+    const float* dist;
+    const unsigned long long* rev;
+    const uint32_t *pick_off, *pick_src, *tile_off, *tile_v;
+    unsigned long long* prop;
+    unsigned long long* work; // [0] next tile, [1] pairs evaluated, [2] rows gathered, [3] a row did not fit the table
+    uint32_t index_bits, slot_cap, span;
+};
+
+struct JoinLds {
+    uint32_t G, tab, row_list, rowptr, rownnz, row_id, col_id, row_worst, col_worst, seen, scan, ctl, total;
+    __host__ __device__ JoinLds(uint32_t index_bits, uint32_t slot_cap, bool narrow) {
+        uint32_t o = 0;
+        tab = o; o += RankTabLds(index_bits, slot_cap, narrow).total;
+        o = (o + 15) & ~15u;
+        G = o; o += JT_ROWS * JT_STRIDE * 4;
+        row_list = o; o += JT_ROWS * JOIN_K * 4;
+        o = (o + 7) & ~7u;
+        rowptr = o; o += (JT_ROWS + JT_COLS) * 8;
+        rownnz = o; o += (JT_ROWS + JT_COLS) * 4;
+        row_id = o; o += JT_ROWS * 4;
+        col_id = o; o += JT_COLS * 4;
+        row_worst = o; o += JT_ROWS * 4;
+        col_worst = o; o += JT_COLS * 4;
+        seen = o; o += JT_SEEN * 4;
+        scan = o; o += 20 * 4;
+        ctl = o; o += 8 * 4;
+        total = o;
+    }
+};
+
+// acc = <rows, cols> over all 1024 dimensions for the 32 x 32 block of row ids `ra` (nr of them) and column ids
+// `cb` (nc of them); operand layout as gram_dense_tile. Rows / columns beyond the counts repeat the last one.
+__device__ __forceinline__ floatx16 join_dense_block(const CorpusView& C, const uint32_t* ra, uint32_t nr, const uint32_t* cb, uint32_t nc, int lane) {
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.f;
+    const uint32_t ia = min((uint32_t)(lane & 31), nr - 1), ib = min((uint32_t)(lane & 31), nc - 1);
+    const float4* pa = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ra[ia]]) * 16) + (lane >> 5);
+    const float4* pb = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[cb[ib]]) * 16) + (lane >> 5);
+    for (int b = 0; b < DIM / 8; b += 4) {
+        float4 a[4], bb[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) { a[u] = pa[2 * (b + u)]; bb[u] = pb[2 * (b + u)]; }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].x, bb[u].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].y, bb[u].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].z, bb[u].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].w, bb[u].w, acc, 0, 0, 0);
+        }
+    }
+    return acc;
+}
+
+template <bool NARROW>
+__global__ __launch_bounds__(JT_THREADS) void join_tile_kernel(JoinArgs a) {
+    a.C.narrow = NARROW ? 1u : 0u;
+    extern __shared__ __align__(16) char smem[];
+    const JoinLds L(a.index_bits, a.slot_cap, NARROW);
+    const RankTab T = ranktab_at(smem + L.tab, a.index_bits, a.slot_cap, a.span, NARROW);
+    float* G = reinterpret_cast<float*>(smem + L.G);
+    uint32_t* row_list = reinterpret_cast<uint32_t*>(smem + L.row_list);
+    unsigned long long* rowptr = reinterpret_cast<unsigned long long*>(smem + L.rowptr);
+    uint32_t* rownnz = reinterpret_cast<uint32_t*>(smem + L.rownnz);
+    uint32_t* row_id = reinterpret_cast<uint32_t*>(smem + L.row_id);
+    uint32_t* col_id = reinterpret_cast<uint32_t*>(smem + L.col_id);
+    float* row_worst = reinterpret_cast<float*>(smem + L.row_worst);
+    float* col_worst = reinterpret_cast<float*>(smem + L.col_worst);
+    uint32_t* seen = reinterpret_cast<uint32_t*>(smem + L.seen);
+    uint32_t* scan = reinterpret_cast<uint32_t*>(smem + L.scan);
+    volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl); // [0] tile, [1] columns
+
+    const int tid = threadIdx.x, wave = (int)uniform(tid / WAVE), lane = lane_id();
+    constexpr int NW = JT_THREADS / WAVE;
+    const uint32_t n_tiles = a.tile_off[a.n];
+
+    while (true) {
+        __syncthreads();
+        if (tid == 0) { ctl[0] = (uint32_t)atomicAdd(a.work, 1ull); ctl[1] = 0; }
+        for (uint32_t i = tid; i < JT_SEEN; i += JT_THREADS) seen[i] = EMPTY;
+        __syncthreads();
+        const uint32_t tile = uniform(ctl[0]);
+        if (tile >= n_tiles) break;
+        const uint32_t v = uniform(a.tile_v[tile]);
+        const uint32_t p0 = uniform(a.pick_off[v]), cnt = uniform(a.pick_off[v + 1]) - p0;
+        const uint32_t r0 = (tile - uniform(a.tile_off[v])) * JT_ROWS;
+        const uint32_t R = min((uint32_t)JT_ROWS, cnt - r0);
+
+        // rows: pickers of v; columns: N(v) and R(v) without repeats
+        if (tid < JT_ROWS) {
+            const uint32_t u = (uint32_t)tid < R ? a.pick_src[p0 + r0 + tid] : EMPTY;
+            row_id[tid] = u;
+            row_worst[tid] = u != EMPTY ? a.dist[(size_t)u * JOIN_K + JOIN_K - 1] : -INF_DIS;
+        }
+        if (tid < 2 * (int)JOIN_K) {
+            uint32_t c;
+            if (tid < (int)JOIN_K) c = a.ids[(size_t)v * JOIN_K + tid] & ~FLAG;
+            else c = (uint32_t)a.rev[(size_t)v * JOIN_K + (tid - JOIN_K)];
+            if (c < a.n && id_set_insert(seen, JT_SEEN - 1, c)) col_id[atomicAdd(const_cast<uint32_t*>(&ctl[1]), 1u)] = c;
+        }
+        __syncthreads();
+        const uint32_t M = uniform(ctl[1]);
+        if (M == 0) continue;
+        // the rows' own lists (who is already a neighbour), the columns' thresholds, where every row's pairs are
+        for (uint32_t t = tid; t < R * JOIN_K; t += JT_THREADS) row_list[t] = a.ids[(size_t)row_id[t / JOIN_K] * JOIN_K + (t % JOIN_K)] & ~FLAG;
+        if ((uint32_t)tid < M) col_worst[tid] = a.symmetric ? a.dist[(size_t)col_id[tid] * JOIN_K + JOIN_K - 1] : -INF_DIS;
+        gram_rows_gather(a.C, row_id, R, rowptr, rownnz, tid, JT_THREADS);
+        gram_rows_gather(a.C, col_id, M, rowptr + JT_ROWS, rownnz + JT_ROWS, tid, JT_THREADS);
+        __syncthreads();
+        // each row's list in ascending id order, in place: a wave reads a whole list before it writes any of it
+        for (uint32_t r = wave; r < R; r += NW) {
+            uint32_t* lst = row_list + r * JOIN_K;
+            const uint32_t mine = lst[lane];
+            uint32_t rank = 0;
+            for (uint32_t i = 0; i < JOIN_K; i++) {
+                const uint32_t x = lst[i];
+                rank += x < mine || (x == mine && i < (uint32_t)lane);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            lst[rank] = mine;
+        }
+        // dense part: wave w owns the 32-column block w
+        if ((uint32_t)(wave * 32) < M) {
+            const uint32_t nc = min(32u, M - wave * 32);
+            const floatx16 acc = join_dense_block(a.C, row_id, R, col_id + wave * 32, nc, lane);
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int i = 8 * (e / 4) + 4 * (lane >> 5) + (e % 4), j = lane & 31;
+                G[i * JT_STRIDE + wave * 32 + j] = a.dense_mul * acc[e];
+            }
+        }
+        __syncthreads();
+        // sparse part: groups of four rows in the rank table, every column probes it once per group
+        uint32_t a0 = 0;
+        while (a0 < R) {
+            uint32_t nt = min((uint32_t)RT_T, R - a0);
+            uint32_t built;
+            while (true) {
+                built = ranktab_build<NARROW>(T, [&](uint32_t t) { Pairs p = gram_row(a.C, rowptr, rownnz, a0 + t); p.narrow = NARROW ? 1u : 0u; return p; }, nt, scan, tid, JT_THREADS);
+                if (built != EMPTY || nt == 1) break;
+                nt = (nt + 1) / 2;
+            }
+            if (built == EMPTY) { // one row alone does not fit: its sparse part is missing, the host is told
+                if (tid == 0) atomicAdd(a.work + 3, 1ull);
+                a0 += nt;
+                continue;
+            }
+            const uint32_t n_ovf = NARROW ? 0u : uniform(min(scan[16], (uint32_t)RT_OVF));
+            uint32_t b = wave;
+            RtRow cur;
+            Pairs sp_cur;
+            if (b < M) { sp_cur = gram_row(a.C, rowptr + JT_ROWS, rownnz + JT_ROWS, b); sp_cur.narrow = NARROW ? 1u : 0u; rt_row_load(cur, sp_cur, lane); }
+            while (b < M) {
+                const uint32_t bn = b + NW;
+                RtRow nxt;
+                Pairs sp_nxt = sp_cur;
+                if (bn < M) { sp_nxt = gram_row(a.C, rowptr + JT_ROWS, rownnz + JT_ROWS, bn); sp_nxt.narrow = NARROW ? 1u : 0u; rt_row_load(nxt, sp_nxt, lane); }
+                float acc[RT_T] = {0.f, 0.f, 0.f, 0.f};
+                ranktab_probe_row<NARROW>(T, cur, sp_cur, n_ovf, acc, lane);
+                uint32_t t;
+                const float z = wave_sum4_dpp(acc, lane, &t);
+                if (lane < RT_T && t < nt) G[(a0 + t) * JT_STRIDE + b] += z;
+                cur = nxt;
+                sp_cur = sp_nxt;
+                b = bn;
+            }
+            a0 += nt;
+            __syncthreads();
+        }
+        // proposals
+        for (uint32_t p = tid; p < R * M; p += JT_THREADS) {
+            const uint32_t r = p / M, c = p % M;
+            const uint32_t uid = row_id[r], cid = col_id[c];
+            if (uid == cid) continue;
+            const float d = 1.0f - G[r * JT_STRIDE + c];
+            if (d < row_worst[r]) {
+                const uint32_t* lst = row_list + r * JOIN_K;
+                uint32_t lo = 0, len = JOIN_K;
+                while (len > 0) {
+                    const uint32_t half = len >> 1;
+                    if (lst[lo + half] < cid) { lo += half + 1; len -= half + 1; } else len = half;
+                }
+                if (lo >= JOIN_K || lst[lo] != cid) atomicMin(&a.prop[(size_t)uid * a.P + prop_slot(cid, a.P)], dist_id_key(d, cid));
+            }
+            if (d < col_worst[c]) atomicMin(&a.prop[(size_t)cid * a.P + prop_slot(uid, a.P)], dist_id_key(d, uid));
+        }
+        if (tid == 0) {
+            atomicAdd(a.work + 1, (unsigned long long)R * M);
+            atomicAdd(a.work + 2, (unsigned long long)(R + M));
+        }
+    }
+}
+
+// One wave per node: its proposals (one slot per lane) merged into its list; a node whose list changed registers
+// with every entry of its list (as step 6 of the expansion kernel). Proposal slots are left empty.
+__global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* ids, float* dist, unsigned long long* prop, unsigned long long* rev,
+                                                         uint32_t* rev_cnt, unsigned long long* inserted) {
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const uint32_t u = blockIdx.x * 4 + wave;
+    if (u >= n) return;
+    const size_t base = (size_t)u * JOIN_K;
+    const unsigned long long key = prop[base + lane];
+    if (__ballot(key != ~0ull) == 0) return;
+    prop[base + lane] = ~0ull;
+    const uint32_t own_id = ids[base + lane];
+    const float own_d = dist[base + lane];
+    const uint32_t c = (uint32_t)key;
+    bool valid = key != ~0ull && c != u && c < n;
+    for (uint32_t i = 0; i < JOIN_K; i++) valid = valid && (((uint32_t)__builtin_amdgcn_readlane((int)own_id, i) & ~FLAG) != c);
+    const uint64_t nb = __ballot(valid);
+    if (nb == 0) return;
+    const float d = join_key_dist(key);
+    // new: rank among the new ones by (distance, id), plus the old entries strictly closer (new first on ties)
+    uint32_t rank_new = 0, le_old = 0;
+    for (uint64_t rest = nb; rest; rest &= rest - 1) {
+        const uint32_t i = __builtin_ctzll(rest);
+        const unsigned long long ki = readlane64(key, i);
+        rank_new += ki < key;
+        le_old += join_key_dist(ki) <= own_d; // old entry: new ones at or below its distance go first
+    }
+    for (uint32_t i = 0; i < JOIN_K; i++) rank_new += valid && readlane_f32(own_d, i) < d;
+    const uint32_t rank_old = (uint32_t)lane + le_old;
+    const bool new_in = valid && rank_new < JOIN_K, old_in = rank_old < JOIN_K;
+    const uint32_t n_ins = __popcll(__ballot(new_in));
+    if (n_ins == 0) return;
+    if (old_in) { ids[base + rank_old] = own_id; dist[base + rank_old] = own_d; }
+    if (new_in) { ids[base + rank_new] = c; dist[base + rank_new] = d; }
+    if (lane == 0) atomicAdd(inserted, (unsigned long long)n_ins);
+    // reverse registration (index.cu:362-372): (distance, u) in one word, slot count % K keeps the closer one beyond K
+    auto reg = [&](uint32_t e, float dv) {
+        const uint32_t v = e & ~FLAG;
+        if (v >= n) return;
+        const uint32_t slot = atomicAdd(&rev_cnt[v], 1u);
+        const unsigned long long k = dist_id_key(dv, u);
+        unsigned long long* at = rev + (size_t)v * JOIN_K + (slot % JOIN_K);
+        if (slot < JOIN_K) *at = k;
+        else atomicMin(at, k);
+    };
+    if (old_in) reg(own_id, own_d);
+    if (new_in) reg(c, d);
+}
+
+__global__ static void join_account_kernel(const unsigned long long* work, unsigned long long* counter) {
+    counter[2] += work[1]; // pairs evaluated
+    counter[3] += work[2]; // rows gathered (each read in full, dense part included)
+}
+
+__global__ __launch_bounds__(256) static void fill_u64_kernel(unsigned long long* p, uint64_t count, unsigned long long v) {
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < count; t += (uint64_t)gridDim.x * blockDim.x) p[t] = v;
+}
+__global__ __launch_bounds__(256) static void fill_u32_kernel2(uint32_t* p, uint64_t count, uint32_t v) {
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < count; t += (uint64_t)gridDim.x * blockDim.x) p[t] = v;
+}
+
+static void join_table_shape(const apoe_corpus* c, uint32_t* index_bits, uint32_t* slot_cap, uint32_t* span) {
+    *span = next_pow2(std::max(c->max_term + 1, 1024u));
+    *index_bits = c->narrow ? 2 * *span : 65536u;
+    const uint32_t want = RT_T * (c->max_nnz_s + c->max_nnz_b);
+    *slot_cap = std::min<uint32_t>(std::max<uint32_t>((want + 63) & ~63u, 256u), 2560u);
+}
+
+int join_alloc(apoe_knn* g) {
+    const size_t n = g->n;
+    APOE_TRY(g->picks.alloc(n * JOIN_PICKS));
+    APOE_TRY(g->pick_cnt.alloc(n + 1));
+    APOE_TRY(g->pick_off.alloc(n + 1));
+    APOE_TRY(g->pick_fill.alloc(n + 1));
+    APOE_TRY(g->pick_src.alloc(n * JOIN_PICKS));
+    APOE_TRY(g->tile_cnt.alloc(n + 1));
+    APOE_TRY(g->tile_off.alloc(n + 1));
+    APOE_TRY(g->tile_v.alloc(n + n * JOIN_PICKS / JT_ROWS + 1));
+    APOE_TRY(g->prop.alloc(n * JOIN_K));
+    APOE_TRY(g->join_work.alloc(4));
+    size_t temp_bytes = 0;
+    APOE_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, temp_bytes, g->pick_cnt.p, g->pick_off.p, (int)(n + 1), g->ctx->stream));
+    APOE_TRY(g->scan_tmp.alloc(temp_bytes));
+    fill_u64_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->prop.p, (uint64_t)n * JOIN_K, ~0ull);
+    APOE_HIP(hipGetLastError());
+    return APOE_OK;
+}
+
+int launch_nnd_join_iterate(apoe_knn* g) {
+    apoe_ctx* ctx = g->ctx;
+    hipStream_t st = ctx->stream;
+    const uint32_t n = g->n;
+    APOE_REQUIRE(g->K == JOIN_K, "the local-join step is built for K = %u lists, this handle has K = %u", JOIN_K, g->K);
+    if (!g->prop.p) APOE_TRY(join_alloc(g));
+    uint32_t index_bits, slot_cap, span;
+    join_table_shape(g->corpus, &index_bits, &slot_cap, &span);
+    const JoinLds L(index_bits, slot_cap, g->corpus->narrow);
+    APOE_REQUIRE(L.total <= 96 * 1024, "the local-join tile needs %u bytes of LDS", L.total);
+
+    APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), st)); // [0] inserted; [2], [3] accumulate over the build
+    fill_u32_kernel2<<<1024, 256, 0, st>>>(g->pick_cnt.p, (uint64_t)n + 1, 0u);
+    fill_u32_kernel2<<<1024, 256, 0, st>>>(g->pick_fill.p, (uint64_t)n + 1, 0u);
+    fill_u64_kernel<<<1, 64, 0, st>>>(g->join_work.p, 4, 0ull);
+    join_pick_kernel<<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->picks.p, g->pick_cnt.p);
+    APOE_HIP(hipGetLastError());
+    join_tile_count_kernel<<<(n + 256) / 256, 256, 0, st>>>(n, g->pick_cnt.p, g->tile_cnt.p);
+    APOE_HIP(hipGetLastError());
+    size_t temp_bytes = g->scan_tmp.n;
+    APOE_HIP(hipcub::DeviceScan::ExclusiveSum(g->scan_tmp.p, temp_bytes, g->pick_cnt.p, g->pick_off.p, (int)(n + 1), st));
+    temp_bytes = g->scan_tmp.n;
+    APOE_HIP(hipcub::DeviceScan::ExclusiveSum(g->scan_tmp.p, temp_bytes, g->tile_cnt.p, g->tile_off.p, (int)(n + 1), st));
+    const uint64_t total = (uint64_t)n * JOIN_PICKS;
+    join_fill_kernel<<<(uint32_t)((total + 255) / 256), 256, 0, st>>>(n, g->picks.p, g->pick_off.p, g->tile_off.p, g->pick_fill.p, g->pick_src.p, g->tile_v.p);
+    APOE_HIP(hipGetLastError());
+
+    JoinArgs a{};
+    a.C = g->corpus->view();
+    a.dense_mul = g->dense_scale * g->dense_scale;
+    a.n = n;
+    a.P = JOIN_K;
+    a.symmetric = g->join_symmetric ? 1u : 0u;
+    a.ids = g->ids.p;
+    a.dist = g->dist.p;
+    a.rev = g->rev.p;
+    a.pick_off = g->pick_off.p;
+    a.pick_src = g->pick_src.p;
+    a.tile_off = g->tile_off.p;
+    a.tile_v = g->tile_v.p;
+    a.prop = g->prop.p;
+    a.work = g->join_work.p;
+    a.index_bits = index_bits;
+    a.slot_cap = slot_cap;
+    a.span = span;
+    auto kernel = g->corpus->narrow ? &join_tile_kernel<true> : &join_tile_kernel<false>;
+    APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
+    int per_cu = 1;
+    APOE_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), JT_THREADS, L.total));
+    if (per_cu < 1) per_cu = 1;
+    kernel<<<(uint32_t)per_cu * (uint32_t)ctx->num_cus, JT_THREADS, L.total, st>>>(a);
+    APOE_HIP(hipGetLastError());
+    join_apply_kernel<<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->dist.p, g->prop.p, g->rev.p, g->rev_cnt.p, g->counter.p);
+    APOE_HIP(hipGetLastError());
+    join_account_kernel<<<1, 1, 0, st>>>(g->join_work.p, g->counter.p);
+    APOE_HIP(hipGetLastError());
+    return APOE_OK;
+}
+
+// Pairs evaluated and rows gathered by the tiles of the last step, and whether a row did not fit the table.
+int join_step_counters(apoe_knn* g, unsigned long long* out3) {
+    unsigned long long h[4] = {0, 0, 0, 0};
+    APOE_HIP(hipMemcpy(h, g->join_work.p, sizeof(h), hipMemcpyDeviceToHost));
+    out3[0] = h[1];
+    out3[1] = h[2];
+    out3[2] = h[3];
+    return APOE_OK;
+}
+
+} // namespace apoe

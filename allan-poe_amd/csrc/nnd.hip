@@ -377,6 +377,17 @@ int launch_nnd_init(apoe_knn* g, uint64_t seed) {
 
 int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted) {
     apoe_ctx* ctx = g->ctx;
+    if (g->join) {
+        APOE_REQUIRE(!g->half_rows, "the local-join step reads the fp32 rows: switch the half-precision rows off");
+        APOE_TRY(launch_nnd_join_iterate(g));
+        if (inserted) {
+            unsigned long long h = 0;
+            APOE_HIP(hipMemcpyAsync(&h, g->counter.p, sizeof(h), hipMemcpyDeviceToHost, ctx->stream));
+            APOE_HIP(hipStreamSynchronize(ctx->stream));
+            *inserted = h;
+        }
+        return APOE_OK;
+    }
     const uint32_t term_slots = doc_term_slots(g->corpus);
     const uint32_t seen_slots = next_pow2(2 * (NND_PICKS * 2 * g->K + g->K + 1));
     const NndLds L(term_slots, seen_slots, g->K);
@@ -496,6 +507,15 @@ int apoe_knn_use_half_rows(apoe_knn* g, int on) {
     APOE_REQUIRE(g, "null argument");
     APOE_REQUIRE(!on || g->corpus->half.p != nullptr, "the corpus has no half-precision rows: call apoe_corpus_make_half_rows first");
     g->half_rows = on != 0;
+    return APOE_OK;
+}
+
+int apoe_knn_set_join(apoe_knn* g, int mode) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_REQUIRE(mode >= 0 && mode <= 2, "join mode must be 0 (expansion step), 1 (local join) or 2 (local join, both endpoints), got %d", mode);
+    APOE_REQUIRE(mode == 0 || g->K == 64, "the local-join step is built for K = 64 lists, this handle has K = %u", g->K);
+    g->join = mode;
+    g->join_symmetric = mode == 2;
     return APOE_OK;
 }
 

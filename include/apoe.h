@@ -135,6 +135,17 @@ void apoe_knn_destroy(apoe_knn* g);
  * differ from the fp32 build's where the rounding (at most 2^-11 dense_scale^2 |a_d| |b_d| per pair) decided.
  * No counterpart in the reference, which has only half-precision rows. */
 int apoe_knn_use_half_rows(apoe_knn* g, int on);
+/* Which step apoe_nnd_iterate runs (replaces nn_descent_gpu, index.cu:156-376, either way):
+ *   0  the reference's expansion step: every node against the forward and reverse lists of the neighbours it
+ *      picks, one pivot against many rows (the default);
+ *   1  the same pairs as a local join around the picked neighbour: all pickers of a node v are the rows of a
+ *      tile, N(v) and R(v) its columns, every row gathered once, the dense part of the tile on the matrix
+ *      cores, survivors sent to the row nodes' lists by 64-bit atomicMin on proposal slots and merged by a
+ *      second kernel; lists are read as the step found them (the reference reads them while they change);
+ *   2  as 1, and every pair is offered to the column node as well (insertion into both endpoints' lists, as
+ *      the classic NN-Descent join does; the reference's step updates the picking node only).
+ * K must be 64 for 1 and 2. May be changed between steps. */
+int apoe_knn_set_join(apoe_knn* g, int mode);
 /* initialize_graph + cal_power (index.cu:890-892). */
 int apoe_nnd_init(apoe_knn* g, uint64_t seed);
 /* One nn_descent_gpu + reset_reverse_num step (index.cu:894-897). last != 0 keeps the

@@ -715,6 +715,127 @@ uint64_t orc_nnd_iterate(const orc_set* corpus, float dense_scale, uint32_t K, u
     return inserted;
 }
 
+/* ---- local-join NN-Descent (see apoe_oracle.h) ---- */
+
+static inline uint32_t float_key(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+static inline float key_float(uint32_t k) {
+    uint32_t u = k ^ ((k >> 31) ? 0x80000000u : 0xFFFFFFFFu);
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+uint64_t orc_join_iterate(const orc_set* corpus, float dense_scale, uint32_t K, uint32_t* ids, float* dist,
+                          uint32_t* rev, float* rev_dist, uint32_t* rev_cnt, const orc_join_params* prm,
+                          uint64_t* evals, int threads) {
+    const uint32_t n = corpus->n, P = prm->slots;
+    std::vector<uint32_t> picks((size_t)n * 4, ORC_EMPTY);
+    std::vector<uint64_t> prop((size_t)n * P, ~0ull);
+    auto amin = [](uint64_t* p, uint64_t v) {
+        uint64_t cur = __atomic_load_n(p, __ATOMIC_RELAXED);
+        while (v < cur && !__atomic_compare_exchange_n(p, &cur, v, true, __ATOMIC_RELAXED, __ATOMIC_RELAXED)) {}
+    };
+    auto slot_of = [P](uint32_t id) { return (uint32_t)(mix64(id) >> 40) & (P - 1); };
+    /* 1. picks, by the rule of the expansion step (index.cu:171-181) */
+#pragma omp parallel for num_threads(nthreads(threads)) schedule(static)
+    for (int64_t uu = 0; uu < (int64_t)n; uu++) {
+        uint32_t* my = ids + (size_t)uu * K;
+        uint32_t slots[4];
+        int np = 0;
+        for (uint32_t g = 0; g < 4; g++) {
+            uint32_t s = g;
+            while (s < K && (my[s] & ORC_FLAG)) s++;
+            if (s >= K) s = 0;
+            else my[s] |= ORC_FLAG;
+            bool seen = false;
+            for (int t = 0; t < np; t++) seen |= slots[t] == s;
+            if (!seen) slots[np++] = s;
+        }
+        for (int t = 0; t < np; t++) picks[(size_t)uu * 4 + t] = my[slots[t]] & ~ORC_FLAG;
+    }
+    /* 2. every picker u of v against N(v) and R(v), on the lists as the step found them */
+    uint64_t n_eval = 0;
+#pragma omp parallel num_threads(nthreads(threads)) reduction(+ : n_eval)
+    {
+        std::vector<uint32_t> own(K), cand;
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t uu = 0; uu < (int64_t)n; uu++) {
+            const uint32_t u = (uint32_t)uu;
+            const uint32_t* my = ids + (size_t)u * K;
+            for (uint32_t j = 0; j < K; j++) own[j] = my[j] & ~ORC_FLAG;
+            std::sort(own.begin(), own.end());
+            const float worst = dist[(size_t)u * K + K - 1];
+            for (int t = 0; t < 4; t++) {
+                const uint32_t v = picks[(size_t)u * 4 + t];
+                if (v == ORC_EMPTY || v >= n) continue;
+                cand.clear();
+                for (uint32_t j = 0; j < K; j++) cand.push_back(ids[(size_t)v * K + j] & ~ORC_FLAG);
+                /* every reverse slot ever written, as the expansion step reads them (index.cu:188) */
+                for (uint32_t j = 0; j < K; j++) if (rev[(size_t)v * K + j] != ORC_EMPTY) cand.push_back(rev[(size_t)v * K + j]);
+                std::sort(cand.begin(), cand.end());
+                cand.erase(std::unique(cand.begin(), cand.end()), cand.end());
+                for (uint32_t c : cand) {
+                    if (c == u || c >= n) continue;
+                    const bool mine = std::binary_search(own.begin(), own.end(), c);
+                    if (mine && !prm->symmetric) continue;
+                    const float d = build_dist(corpus, u, c, dense_scale);
+                    n_eval++;
+                    if (!mine && d < worst) amin(&prop[(size_t)u * P + slot_of(c)], ((uint64_t)float_key(d) << 32) | c);
+                    /* the column side is offered without a look into c's list: an id that c already holds
+                     * is dropped when c merges its proposals */
+                    if (prm->symmetric && d < dist[(size_t)c * K + K - 1])
+                        amin(&prop[(size_t)c * P + slot_of(u)], ((uint64_t)float_key(d) << 32) | u);
+                }
+            }
+        }
+    }
+    if (evals) *evals += n_eval;
+    /* 3. apply; a node whose list changed registers with every entry of its list (index.cu:362-372) */
+    uint64_t inserted = 0;
+#pragma omp parallel num_threads(nthreads(threads)) reduction(+ : inserted)
+    {
+        std::vector<Cand> fresh, list(K);
+#pragma omp for schedule(static)
+        for (int64_t xx = 0; xx < (int64_t)n; xx++) {
+            const uint32_t x = (uint32_t)xx;
+            uint32_t* my = ids + (size_t)x * K;
+            float* myd = dist + (size_t)x * K;
+            fresh.clear();
+            for (uint32_t s = 0; s < P; s++) {
+                const uint64_t k = prop[(size_t)x * P + s];
+                if (k == ~0ull) continue;
+                const uint32_t c = (uint32_t)k;
+                bool member = c == x;
+                for (uint32_t t = 0; t < K && !member; t++) member = (my[t] & ~ORC_FLAG) == c;
+                if (!member) fresh.push_back({key_float((uint32_t)(k >> 32)), c, 1, 0});
+            }
+            if (fresh.empty()) continue;
+            std::sort(fresh.begin(), fresh.end(), cand_less);
+            for (uint32_t j = 0; j < K; j++) list[j] = {myd[j], my[j], 0, 0};
+            merge_cands(list, fresh);
+            uint32_t ins = 0;
+            for (uint32_t j = 0; j < K; j++) { my[j] = list[j].id; myd[j] = list[j].dist; ins += list[j].ent; }
+            inserted += ins;
+            if (!ins) continue;
+            for (uint32_t j = 0; j < K; j++) {
+                const uint32_t v = list[j].id & ~ORC_FLAG;
+                if (v >= n) continue;
+                const float dv = list[j].dist;
+                const uint32_t slot = __atomic_fetch_add(&rev_cnt[v], 1u, __ATOMIC_RELAXED);
+                uint32_t* at = &rev[(size_t)v * K + slot % K];
+                float* atd = &rev_dist[(size_t)v * K + slot % K];
+                if (slot < K) { __atomic_store_n(at, x, __ATOMIC_RELAXED); *atd = dv; }
+                else if (dv < *atd) { __atomic_store_n(at, x, __ATOMIC_RELAXED); *atd = dv; }
+            }
+        }
+    }
+    return inserted;
+}
+
 /*
  * index.cu:386-478: merge a node's list with the reverse neighbours registered in
  * the last iteration (at most K of them). Reverse ids already in the list are

@@ -106,6 +106,31 @@ uint64_t orc_nnd_iterate(const orc_set* corpus, float dense_scale, uint32_t K, u
 void orc_nnd_merge_reverse(uint32_t n, uint32_t K, uint32_t* ids, float* dist, const uint32_t* rev,
                            const float* rev_dist, const uint32_t* rev_cnt, int threads);
 
+/*
+ * The NN-Descent step as a LOCAL JOIN around the picked neighbour. It stands where
+ * orc_nnd_iterate stands (index.cu:156-376) and evaluates the same pairs -- node u against
+ * the forward list N(v) and the reverse list R(v) of each neighbour v it picks, by the same
+ * picking rule -- but as the GPU's join kernels do it: all pickers of one v form the rows of a
+ * tile whose columns are N(v) and R(v), every list is read as it was when the step started,
+ * and a row's survivors travel to its list as proposals: slot (mix64(id) >> 40) mod `slots`
+ * of the node's proposal row keeps the smallest (distance, id), so a step is deterministic
+ * whatever the order of evaluation (the reverse lists keep the reference's arrival order).
+ * With `symmetric` a pair (u, c) is also offered to the COLUMN node c (u proposed to c's list
+ * when it is closer than c's last entry; whether c already holds u is only looked at when c
+ * merges): the classic join's insertion into both endpoints, which the reference's step does
+ * not do.
+ * Then every node merges its proposals (new before old on equal distance, index.cu:333-351);
+ * a node whose list changed registers with every entry of its list (index.cu:362-372).
+ */
+typedef struct {
+    uint32_t slots;      /* proposal slots per node, a power of two */
+    uint32_t symmetric;  /* 1: offer every evaluated pair to both endpoints */
+} orc_join_params;
+/* Returns the number of list entries inserted; *evals (optional) += distances computed. */
+uint64_t orc_join_iterate(const orc_set* corpus, float dense_scale, uint32_t K, uint32_t* ids,
+                          float* dist, uint32_t* rev, float* rev_dist, uint32_t* rev_cnt,
+                          const orc_join_params* prm, uint64_t* evals, int threads);
+
 /* RNG-IP prune + keyword recycling (index.cu:539-714).
  * out_fwd [n][d] ids, out_det [n][d] detour counts, out_cnt [n] real entries,
  * out_kw [n][1+ORC_KW_CAND] = count followed by keyword-edge candidates. */

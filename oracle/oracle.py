@@ -224,6 +224,19 @@ def nnd_iterate(corpus, dense_scale, st, threads=0):
     return int(lib().orc_nnd_iterate(corpus.ref(), C.c_float(dense_scale), C.c_uint32(st.K), *st._p(), threads))
 
 
+class JoinParams(C.Structure):
+    _fields_ = [("slots", C.c_uint32), ("symmetric", C.c_uint32)]
+
+
+def join_iterate(corpus, dense_scale, st, slots=64, symmetric=False, threads=0):
+    """One step as a local join around the picked neighbours; returns (inserted, distance evaluations)."""
+    prm = JoinParams(slots, 1 if symmetric else 0)
+    ev = C.c_uint64(0)
+    lib().orc_join_iterate.restype = C.c_uint64
+    ins = lib().orc_join_iterate(corpus.ref(), C.c_float(dense_scale), C.c_uint32(st.K), *st._p(), C.byref(prm), C.byref(ev), threads)
+    return int(ins), int(ev.value)
+
+
 def nnd_merge_reverse(st, threads=0):
     lib().orc_nnd_merge_reverse(C.c_uint32(st.n), C.c_uint32(st.K), *st._p(), threads)
 

@@ -1,0 +1,81 @@
+"""The local-join NN-Descent step on the GPU (apoe_knn_set_join) against its oracle restatement and against the
+reference-shaped expansion step."""
+import numpy as np
+import pytest
+
+from parity import assert_dist_close
+
+pytestmark = pytest.mark.gpu
+
+
+def knn_recall(ids, truth, k):
+    return float(np.mean([len(set(ids[i, :k].tolist()) & set(truth[i, :k].tolist())) / k for i in range(len(truth))]))
+
+
+@pytest.fixture(scope="module")
+def exact_knn(small_world):
+    import oracle as O
+    return O.bruteforce_knn_self(small_world["C"], 7.0, 64)
+
+
+@pytest.mark.parametrize("mode", [1, 2])
+def test_first_join_step_equals_the_oracle_step(gpu_world, mode):
+    """From the same random lists (reverse lists empty) a join step is a function of its input: the GPU's lists are
+    the oracle's, row for row, except where two float sums that differ in their last bits decide a comparison."""
+    import apoe
+    import oracle as O
+    w = gpu_world
+    knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+    knn.set_join(mode)
+    knn.init(77)
+    ins = knn.iterate(last=True)
+    ids, dist = knn.download()
+    st = O.nnd_init(w["C"].n, 64, 77)
+    oins, _ = O.join_iterate(w["C"], 7.0, st, slots=64, symmetric=(mode == 2))
+    oids = st.ids & 0x7FFFFFFF
+    same = np.all(ids == oids, axis=1)
+    print(f"mode {mode}: inserted {ins} (oracle {oins}); identical rows {same.mean():.4f}")
+    assert abs(ins - oins) <= 0.001 * oins
+    assert same.mean() >= 0.99
+    m = ids == oids
+    assert_dist_close(dist[m], st.dist[m], "stored distances")
+    knn.close()
+
+
+@pytest.mark.parametrize("mode", [1, 2])
+def test_join_lists_invariants_and_recall(gpu_world, exact_knn, mode):
+    import apoe
+    import oracle as O
+    w = gpu_world
+    C, n = w["C"], w["C"].n
+    knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+    knn.set_join(mode)
+    knn.init(5)
+    ins = [knn.iterate(last=(it == 7)) for it in range(8)]
+    knn.merge_reverse()
+    ids, dist = knn.download()
+    knn.close()
+    assert ins[0] > ins[-1] > 0
+    assert ids.max() < n and not np.any(ids == np.arange(n)[:, None])
+    assert np.all(np.diff(dist, axis=1) >= 0)
+    srt = np.sort(ids, axis=1)
+    assert not np.any(srt[:, 1:] == srt[:, :-1])
+    rows = np.repeat(np.arange(n, dtype=np.uint32), 64)
+    assert_dist_close(dist.ravel(), O.distance_pairs(C, 7.0, rows, ids.ravel()), "stored = recomputed")
+    # list quality: against the oracle's join and against the oracle's expansion step (the reference's algorithm)
+    st = O.nnd_init(n, 64, 5)
+    for it in range(8):
+        O.join_iterate(C, 7.0, st, slots=64, symmetric=(mode == 2))
+        if it < 7:
+            st.rev_cnt[:] = 0
+    O.nnd_merge_reverse(st)
+    se = O.nnd_init(n, 64, 5)
+    for it in range(8):
+        O.nnd_iterate(C, 7.0, se)
+        if it < 7:
+            se.rev_cnt[:] = 0
+    O.nnd_merge_reverse(se)
+    ex_ids, _ = exact_knn
+    r_g, r_j, r_e = (knn_recall(x, ex_ids, 10) for x in (ids, st.ids & 0x7FFFFFFF, se.ids & 0x7FFFFFFF))
+    print(f"mode {mode}: kNN recall@10 gpu join {r_g:.4f}, oracle join {r_j:.4f}, oracle expansion {r_e:.4f}")
+    assert r_g >= r_j - 0.005 and r_g >= r_e - 0.005
