@@ -68,23 +68,58 @@ __device__ __forceinline__ uint32_t ranktab_index(const RankTab& T, uint32_t key
     return ((k * 0x9E3779B1u) >> 12) & (T.index_bits - 1);
 }
 
-// Builds the table of pivots [0, nt) (nt <= RT_T); pivot(t) gives the Pairs of pivot t. All threads of the block
-// call it (the block size is a multiple of 64, at most 1024); `scan` is LDS scratch of 20 words. Returns the
-// number of distinct terms, or EMPTY if they exceed the slot capacity or the overflow list (the table is then
-// unusable: the caller retries with fewer pivots). Ends with a barrier: the table is ready on return.
+// The pairs of the pivots of one group, spread over the threads of the block: thread i holds pairs i and
+// i + nthreads of every pivot (rows with more pairs read the rest when the table is built). Loaded ahead of
+// time, while the previous group is still being probed, so that a build does not wait for memory.
+constexpr int RT_PV = 2;
+struct PivotRegs {
+    uint2 kv[RT_T][RT_PV]; // raw pairs
+};
+template <typename PivotFn>
+__device__ __forceinline__ void ranktab_pivots_load(PivotRegs& r, PivotFn pivot, uint32_t nt, int tid, int nthreads) {
+#pragma unroll
+    for (int t = 0; t < RT_T; t++) {
+        if ((uint32_t)t < nt) {
+            const Pairs sp = pivot(t);
+#pragma unroll
+            for (int k = 0; k < RT_PV; k++) {
+                const uint32_t j = tid + k * nthreads;
+                r.kv[t][k] = j < sp.nnz ? sp.raw(j) : make_uint2(0u, 0u);
+            }
+        }
+    }
+}
+
+// Builds the table of pivots [0, nt) (nt <= RT_T); pivot(t) gives the Pairs of pivot t, `regs` its first pairs
+// (ranktab_pivots_load). All threads of the block call it (the block size is a multiple of 64, at most 1024);
+// `scan` is LDS scratch of 20 words. Returns the number of distinct terms, or EMPTY if they exceed the slot
+// capacity or the overflow list (the table is then unusable: the caller retries with fewer pivots). Ends with
+// a barrier: the table is ready on return.
 template <bool NARROW, typename PivotFn>
-__device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivot, uint32_t nt, uint32_t* scan, int tid, int nthreads) {
+__device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivot, const PivotRegs& regs, uint32_t nt, uint32_t* scan, int tid,
+                                                  int nthreads) {
     const uint32_t W = T.index_bits / 32;
     const int lane = tid & (WAVE - 1), wave = tid / WAVE, nwaves = nthreads / WAVE;
     for (uint32_t w = tid; w < W; w += nthreads) T.word[w] = make_uint2(0u, 0u);
     if (tid == 0) scan[16] = 0; // overflow count
     __syncthreads();
     // 1. bits
-    for (uint32_t t = 0; t < nt; t++) {
-        const Pairs sp = pivot(t);
-        for (uint32_t j = tid; j < sp.nnz; j += nthreads) {
-            const uint32_t idx = ranktab_index<NARROW>(T, NARROW ? sp.raw(j).x : sp.key(j), j >= sp.ns);
-            atomicOr(&T.word[idx >> 5].x, 1u << (idx & 31));
+#pragma unroll
+    for (int t = 0; t < RT_T; t++) {
+        if ((uint32_t)t < nt) {
+            const Pairs sp = pivot(t);
+#pragma unroll
+            for (int k = 0; k < RT_PV; k++) {
+                const uint32_t j = tid + k * nthreads;
+                if (j < sp.nnz) {
+                    const uint32_t idx = ranktab_index<NARROW>(T, regs.kv[t][k].x, j >= sp.ns);
+                    atomicOr(&T.word[idx >> 5].x, 1u << (idx & 31));
+                }
+            }
+            for (uint32_t j = tid + RT_PV * nthreads; j < sp.nnz; j += nthreads) {
+                const uint32_t idx = ranktab_index<NARROW>(T, sp.raw(j).x, j >= sp.ns);
+                atomicOr(&T.word[idx >> 5].x, 1u << (idx & 31));
+            }
         }
     }
     __syncthreads();
@@ -129,30 +164,38 @@ __device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivo
     }
     __syncthreads();
     // 3. values (and keys)
-    for (uint32_t t = 0; t < nt; t++) {
-        const Pairs sp = pivot(t);
-        for (uint32_t j = tid; j < sp.nnz; j += nthreads) {
-            const uint2 kv = NARROW ? sp.raw(j) : sp[j];
-            const uint32_t idx = ranktab_index<NARROW>(T, kv.x, j >= sp.ns);
-            const uint2 w = T.word[idx >> 5];
-            const uint32_t slot = w.y + __popc(w.x & ((1u << (idx & 31)) - 1u));
-            if (NARROW) {
+    auto put = [&](uint2 kv, uint32_t j, const Pairs& sp, int t) {
+        const uint32_t idx = ranktab_index<NARROW>(T, kv.x, j >= sp.ns);
+        const uint2 w = T.word[idx >> 5];
+        const uint32_t slot = w.y + __popc(w.x & ((1u << (idx & 31)) - 1u));
+        if (NARROW) {
+            reinterpret_cast<uint32_t*>(&T.vals[slot])[t] = kv.y;
+        } else {
+            const uint32_t old = atomicCAS(&T.keys[slot], EMPTY, kv.x);
+            if (old == EMPTY || old == kv.x) {
                 reinterpret_cast<uint32_t*>(&T.vals[slot])[t] = kv.y;
-            } else {
-                const uint32_t old = atomicCAS(&T.keys[slot], EMPTY, kv.x);
-                if (old == EMPTY || old == kv.x) {
-                    reinterpret_cast<uint32_t*>(&T.vals[slot])[t] = kv.y;
-                } else { // another term of the group sits on this bit
-                    uint32_t at = EMPTY;
-                    for (uint32_t s = 0; s < RT_OVF; s++) {
-                        const uint32_t o = atomicCAS(&T.ovf_key[s], EMPTY, kv.x);
-                        if (o == EMPTY) atomicAdd(&scan[16], 1u);
-                        if (o == EMPTY || o == kv.x) { at = s; break; }
-                    }
-                    if (at != EMPTY) reinterpret_cast<uint32_t*>(&T.ovf_val[at])[t] = kv.y;
-                    else atomicAdd(&scan[16], RT_OVF + 1u);
+            } else { // another term of the group sits on this bit
+                uint32_t at = EMPTY;
+                for (uint32_t s = 0; s < RT_OVF; s++) {
+                    const uint32_t o = atomicCAS(&T.ovf_key[s], EMPTY, kv.x);
+                    if (o == EMPTY) atomicAdd(&scan[16], 1u);
+                    if (o == EMPTY || o == kv.x) { at = s; break; }
                 }
+                if (at != EMPTY) reinterpret_cast<uint32_t*>(&T.ovf_val[at])[t] = kv.y;
+                else atomicAdd(&scan[16], RT_OVF + 1u);
             }
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < RT_T; t++) {
+        if ((uint32_t)t < nt) {
+            const Pairs sp = pivot(t);
+#pragma unroll
+            for (int k = 0; k < RT_PV; k++) {
+                const uint32_t j = tid + k * nthreads;
+                if (j < sp.nnz) put(regs.kv[t][k], j, sp, t);
+            }
+            for (uint32_t j = tid + RT_PV * nthreads; j < sp.nnz; j += nthreads) put(sp.raw(j), j, sp, t);
         }
     }
     __syncthreads();
@@ -195,95 +238,173 @@ __device__ __forceinline__ float wave_sum4_dpp(const float acc[4], int lane, uin
     return z;
 }
 
-constexpr int RT_CHUNKS = 5; // 64-pair chunks of a streamed row kept in registers (320 pairs); longer rows loop
+constexpr int RT_CHUNKS = 3; // 64-pair chunks of a streamed row kept in registers (192 pairs); longer rows read the rest when they are probed
 
-struct RtRow { // raw pairs of a streamed row
-    uint2 kv[RT_CHUNKS];
+// Raw pairs of a streamed row in registers: lane l holds pairs l, l + 64, l + 128. Narrow keys are 16 bits wide:
+// the first two share a register.
+template <bool NARROW>
+struct RtRow;
+template <>
+struct RtRow<true> {
+    uint32_t v[RT_CHUNKS], k01, k2;
+    // tells the compiler that the keys may have changed: what is derived from them (bit index, masks) is then computed
+    // where it is used instead of once for all rows ahead of a loop, where it would occupy registers for the whole loop
+    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(k01), "+v"(k2)); }
+    __device__ __forceinline__ uint32_t key(int c) const { return c == 0 ? (k01 & 0xFFFFu) : c == 1 ? (k01 >> 16) : k2; }
+    __device__ __forceinline__ void set(int c, uint2 kv) {
+        v[c] = kv.y;
+        if (c == 0) k01 = kv.x;
+        else if (c == 1) k01 |= kv.x << 16;
+        else k2 = kv.x;
+    }
 };
-__device__ __forceinline__ void rt_row_load(RtRow& r, const Pairs& sp, int lane) {
+template <>
+struct RtRow<false> {
+    uint32_t v[RT_CHUNKS], k[RT_CHUNKS];
+    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(k[0]), "+v"(k[1]), "+v"(k[2])); }
+    __device__ __forceinline__ uint32_t key(int c) const { return k[c]; }
+    __device__ __forceinline__ void set(int c, uint2 kv) { v[c] = kv.y; k[c] = kv.x; }
+};
+template <bool NARROW>
+__device__ __forceinline__ void rt_row_load(RtRow<NARROW>& r, const Pairs& sp, int lane) {
 #pragma unroll
     for (int c = 0; c < RT_CHUNKS; c++) {
         const uint32_t j = c * WAVE + lane;
-        r.kv[c] = j < sp.nnz ? sp.raw(j) : make_uint2(0u, 0u);
+        r.set(c, j < sp.nnz ? sp.raw(j) : make_uint2(0u, 0u));
     }
 }
 
-// The streamed row `cur` (nnz pairs, ns of them SPLADE; sp gives the pairs beyond the register window) against
-// the table: acc[0..3] += per-pivot sums of this lane's pairs.
-template <bool NARROW>
-__device__ __forceinline__ void ranktab_probe_row(const RankTab& T, const RtRow& cur, const Pairs& sp, uint32_t n_ovf, float acc[4], int lane) {
-    const uint32_t nnz = sp.nnz, ns = sp.ns;
-    auto overflow = [&](uint32_t key, uint32_t val_bits, bool in) {
+// NB streamed rows against the table at once: acc[r][0..3] += per-pivot sums of this lane's pairs of row r.
+// All bitmap reads of the batch are issued before the first value read, all value reads before the first
+// multiply: the batch costs two LDS round trips whatever NB is. shape[r] = nnz | ns << 16 of row r (wave-uniform;
+// 0: the row is not there); tail(r) gives the Pairs of row r for the pairs beyond the register window.
+template <bool NARROW, int NB, typename TailFn>
+__device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow<NARROW> (&rows)[NB], const uint32_t (&shape)[NB], TailFn tail,
+                                                   uint32_t n_ovf, float (&acc)[NB][RT_T], int lane) {
+    auto overflow = [&](int r, uint32_t key, uint32_t val_bits, bool in) {
         for (uint32_t o = 0; o < n_ovf; o++) { // wave-uniform count, zero for narrow corpora
             if (in && T.ovf_key[o] == key) {
                 const float4 v = T.ovf_val[o];
                 const float val = __uint_as_float(val_bits);
-                acc[0] = fmaf(val, v.x, acc[0]);
-                acc[1] = fmaf(val, v.y, acc[1]);
-                acc[2] = fmaf(val, v.z, acc[2]);
-                acc[3] = fmaf(val, v.w, acc[3]);
+                acc[r][0] = fmaf(val, v.x, acc[r][0]);
+                acc[r][1] = fmaf(val, v.y, acc[r][1]);
+                acc[r][2] = fmaf(val, v.z, acc[r][2]);
+                acc[r][3] = fmaf(val, v.w, acc[r][3]);
             }
         }
     };
-    auto key_of = [&](uint2 kv, uint32_t j) -> uint32_t { return NARROW ? kv.x : kv.x; };
-    // the first three chunks as one batch: three bitmap reads, then three value reads
-    {
-        uint32_t idx[3];
-        uint2 w[3];
-        bool in[3];
+    uint32_t idx[NB][RT_CHUNKS];
+    uint2 w[NB][RT_CHUNKS];
 #pragma unroll
-        for (int c = 0; c < 3; c++) {
+    for (int r = 0; r < NB; r++) {
+        const uint32_t nnz = shape[r] & 0xFFFFu, ns = shape[r] >> 16;
+#pragma unroll
+        for (int c = 0; c < RT_CHUNKS; c++) {
             const uint32_t j = c * WAVE + lane;
-            in[c] = j < nnz;
-            idx[c] = ranktab_index<NARROW>(T, key_of(cur.kv[c], j), NARROW ? j >= ns : (int)cur.kv[c].x < 0);
-            w[c] = T.word[in[c] ? idx[c] >> 5 : 0u];
+            const uint32_t key = rows[r].key(c);
+            idx[r][c] = ranktab_index<NARROW>(T, key, NARROW ? j >= ns : (int)key < 0);
+            w[r][c] = T.word[j < nnz ? idx[r][c] >> 5 : 0u];
         }
-        asm volatile("" : "+v"(w[0].x), "+v"(w[1].x), "+v"(w[2].x));
-        RankProbe p[3];
-        float4 v[3];
-        bool ok[3];
+    }
 #pragma unroll
-        for (int c = 0; c < 3; c++) {
-            p[c] = ranktab_locate<NARROW>(T, w[c], idx[c], cur.kv[c].y, in[c]);
-            v[c] = T.vals[p[c].slot];
-            ok[c] = true;
-            if (!NARROW) ok[c] = p[c].mul == 0.f || T.keys[p[c].slot] == cur.kv[c].x;
+    for (int r = 0; r < NB; r++) asm volatile("" : "+v"(w[r][0].x), "+v"(w[r][1].x), "+v"(w[r][2].x));
+    RankProbe p[NB][RT_CHUNKS];
+    float4 v[NB][RT_CHUNKS];
+    bool ok[NB][RT_CHUNKS];
+#pragma unroll
+    for (int r = 0; r < NB; r++) {
+        const uint32_t nnz = shape[r] & 0xFFFFu;
+#pragma unroll
+        for (int c = 0; c < RT_CHUNKS; c++) {
+            const bool in = (uint32_t)(c * WAVE + lane) < nnz;
+            p[r][c] = ranktab_locate<NARROW>(T, w[r][c], idx[r][c], rows[r].v[c], in);
+            v[r][c] = T.vals[p[r][c].slot];
+            ok[r][c] = true;
+            if (!NARROW) ok[r][c] = p[r][c].mul == 0.f || T.keys[p[r][c].slot] == rows[r].key(c);
         }
-        asm volatile("" : "+v"(v[0].x), "+v"(v[1].x), "+v"(v[2].x));
+    }
 #pragma unroll
-        for (int c = 0; c < 3; c++) {
-            const float m = ok[c] ? p[c].mul : 0.f;
-            acc[0] = fmaf(m, v[c].x, acc[0]);
-            acc[1] = fmaf(m, v[c].y, acc[1]);
-            acc[2] = fmaf(m, v[c].z, acc[2]);
-            acc[3] = fmaf(m, v[c].w, acc[3]);
+    for (int r = 0; r < NB; r++) asm volatile("" : "+v"(v[r][0].x), "+v"(v[r][1].x), "+v"(v[r][2].x));
+#pragma unroll
+    for (int r = 0; r < NB; r++) {
+        const uint32_t nnz = shape[r] & 0xFFFFu;
+#pragma unroll
+        for (int c = 0; c < RT_CHUNKS; c++) {
+            const float m = ok[r][c] ? p[r][c].mul : 0.f;
+            acc[r][0] = fmaf(m, v[r][c].x, acc[r][0]);
+            acc[r][1] = fmaf(m, v[r][c].y, acc[r][1]);
+            acc[r][2] = fmaf(m, v[r][c].z, acc[r][2]);
+            acc[r][3] = fmaf(m, v[r][c].w, acc[r][3]);
         }
         if (!NARROW && n_ovf) {
 #pragma unroll
-            for (int c = 0; c < 3; c++) overflow(cur.kv[c].x, cur.kv[c].y, in[c] && !ok[c]);
+            for (int c = 0; c < RT_CHUNKS; c++) overflow(r, rows[r].key(c), rows[r].v[c], (uint32_t)(c * WAVE + lane) < nnz && !ok[r][c]);
         }
     }
-    auto one = [&](uint2 kv, uint32_t j, bool in) {
-        const uint32_t idx = ranktab_index<NARROW>(T, kv.x, NARROW ? j >= ns : (int)kv.x < 0);
-        const uint2 w = T.word[in ? idx >> 5 : 0u];
-        const RankProbe p = ranktab_locate<NARROW>(T, w, idx, kv.y, in);
-        const float4 v = T.vals[p.slot];
-        bool ok = true;
-        if (!NARROW) ok = p.mul == 0.f || T.keys[p.slot] == kv.x;
-        const float m = ok ? p.mul : 0.f;
-        acc[0] = fmaf(m, v.x, acc[0]);
-        acc[1] = fmaf(m, v.y, acc[1]);
-        acc[2] = fmaf(m, v.z, acc[2]);
-        acc[3] = fmaf(m, v.w, acc[3]);
-        if (!NARROW && n_ovf) overflow(kv.x, kv.y, in && !ok);
-    };
+    // rows longer than the register window
 #pragma unroll
-    for (int c = 3; c < RT_CHUNKS; c++)
-        if (c * WAVE < (int)nnz) one(cur.kv[c], c * WAVE + lane, (uint32_t)(c * WAVE + lane) < nnz); // wave-uniform branch
-    for (uint32_t j0 = RT_CHUNKS * WAVE; j0 < nnz; j0 += WAVE) { // rows longer than the register window
-        const uint32_t j = j0 + lane;
-        one(j < nnz ? sp.raw(j) : make_uint2(0u, 0u), j, j < nnz);
+    for (int r = 0; r < NB; r++) {
+        const uint32_t nnz = shape[r] & 0xFFFFu, ns = shape[r] >> 16;
+        if (nnz > RT_CHUNKS * WAVE) {
+            const Pairs sp = tail(r);
+            for (uint32_t j0 = RT_CHUNKS * WAVE; j0 < nnz; j0 += WAVE) {
+                const uint32_t j = j0 + lane;
+                const bool in = j < nnz;
+                const uint2 kv = in ? sp.raw(j) : make_uint2(0u, 0u);
+                const uint32_t ix = ranktab_index<NARROW>(T, kv.x, NARROW ? j >= ns : (int)kv.x < 0);
+                const uint2 ww = T.word[in ? ix >> 5 : 0u];
+                const RankProbe q = ranktab_locate<NARROW>(T, ww, ix, kv.y, in);
+                const float4 vv = T.vals[q.slot];
+                bool good = true;
+                if (!NARROW) good = q.mul == 0.f || T.keys[q.slot] == kv.x;
+                const float m = good ? q.mul : 0.f;
+                acc[r][0] = fmaf(m, vv.x, acc[r][0]);
+                acc[r][1] = fmaf(m, vv.y, acc[r][1]);
+                acc[r][2] = fmaf(m, vv.z, acc[r][2]);
+                acc[r][3] = fmaf(m, vv.w, acc[r][3]);
+                if (!NARROW && n_ovf) overflow(r, kv.x, kv.y, in && !good);
+            }
+        }
     }
+}
+
+// The wave totals of NB (2 or 4) streamed rows x 4 pivots from the per-lane accumulators of ranktab_probe_rows, with
+// NB - 1 + (NB == 2) cross-row exchanges for all of them: inside each 16-lane row the four pivot sums of a streamed
+// row are reduced as in wave_sum4_dpp (lane l keeps pivot t(l) = 2 * (l & 1) + ((l >> 1) & 1)); then the four
+// 16-lane rows of the wave share out the streamed rows between them. Returns the total of (*r_out, *t_out).
+template <int NB>
+__device__ __forceinline__ float wave_sum_rows(const float (&acc)[NB][RT_T], int lane, uint32_t* t_out, uint32_t* r_out) {
+    static_assert(NB == 2 || NB == 4, "two or four streamed rows");
+    float z[NB];
+    const bool odd = lane & 1, hi = lane & 2;
+#pragma unroll
+    for (int r = 0; r < NB; r++) {
+        const float keep0 = odd ? acc[r][2] : acc[r][0], keep1 = odd ? acc[r][3] : acc[r][1];
+        const float give0 = odd ? acc[r][0] : acc[r][2], give1 = odd ? acc[r][1] : acc[r][3];
+        const float x0 = keep0 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give0), 0xB1, 0xF, 0xF, false));
+        const float x1 = keep1 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give1), 0xB1, 0xF, 0xF, false));
+        const float keep = hi ? x1 : x0, give = hi ? x0 : x1;
+        float y = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give), 0x4E, 0xF, 0xF, false));
+        y += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, y), 0x124, 0xF, 0xF, false)); // row_ror:4
+        y += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, y), 0x128, 0xF, 0xF, false)); // row_ror:8
+        z[r] = y;
+    }
+    const bool q0 = lane & 16, q1 = lane & 32;
+    *t_out = 2u * (lane & 1) + ((lane >> 1) & 1);
+    if (NB == 4) {
+        const float keepA0 = q0 ? z[2] : z[0], giveA0 = q0 ? z[0] : z[2];
+        const float keepA1 = q0 ? z[NB - 1] : z[1], giveA1 = q0 ? z[1] : z[NB - 1];
+        const float xa = keepA0 + __shfl_xor(giveA0, 16, WAVE);
+        const float xb = keepA1 + __shfl_xor(giveA1, 16, WAVE);
+        const float keepB = q1 ? xb : xa, giveB = q1 ? xa : xb;
+        *r_out = 2u * ((lane >> 4) & 1) + ((lane >> 5) & 1);
+        return keepB + __shfl_xor(giveB, 32, WAVE);
+    }
+    const float keepA = q0 ? z[1] : z[0], giveA = q0 ? z[0] : z[1];
+    float x = keepA + __shfl_xor(giveA, 16, WAVE);
+    x += __shfl_xor(x, 32, WAVE);
+    *r_out = (lane >> 4) & 1;
+    return x;
 }
 
 #endif // __HIPCC__

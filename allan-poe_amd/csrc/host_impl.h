@@ -29,6 +29,9 @@ struct BuildOptions {
     // NN-Descent steps on a half-precision copy of the dense rows (what the reference stores), stored distances
     // recomputed from the fp32 rows before the prune. Off: every step reads fp32 rows.
     bool half_rows = false;
+    // 0: the reference's expansion step (index.cu:156-376). 1: the same pairs as a local join around the picked
+    // neighbour (rows gathered once per tile, dense part on the matrix cores). 2: the join, both endpoints updated.
+    int nnd_join = 0;
 };
 
 struct SearchOptions {

@@ -4,8 +4,10 @@
 // each neighbour v it picks: one pivot against many rows, every row gathered for one evaluation. Here the same
 // pairs are formed the other way round: all pickers of one v are the ROWS of a tile (32 at a time), N(v) and R(v)
 // are its COLUMNS (up to 128), every row of the tile is gathered once and meets every column:
-//   dense part   32 x 128 x 1024 contraction on the matrix cores (fp32 MFMA 32x32x2, one 32-column block per wave)
-//   sparse part  four picker rows at a time in an LDS rank table that the column rows probe (apoe_ranktab.h)
+//   dense part   32 x 128 x 1024 contraction on the matrix cores (fp32 MFMA 32x32x2; eight waves: four 32-column
+//                blocks x two halves of the dimensions)
+//   sparse part  four picker rows at a time in an LDS rank table that the column rows probe (apoe_ranktab.h); a
+//                wave keeps the pairs of its sixteen columns in registers, so a row is read from memory once per tile
 //   insertion    a pair closer than the row's last list entry (and not in that list) is offered to the row node
 //                with a 64-bit atomicMin on slot hash(id) of its proposal row: (distance, id), the smallest wins;
 //                in symmetric mode the pair is offered to the column node as well (both endpoints, as the classic
@@ -26,11 +28,13 @@ namespace apoe {
 
 constexpr int JT_ROWS = 32;
 constexpr int JT_COLS = 128;
-constexpr int JT_THREADS = 256;
+constexpr int JT_THREADS = 512;
 constexpr int JT_STRIDE = JT_COLS + 1;
 constexpr int JT_SEEN = 512; // slots of the id set that removes repeated columns
 constexpr uint32_t JOIN_K = 64;
 constexpr int JOIN_PICKS = 4; // index.cu:157,171-181
+constexpr int JT_BATCH = 4;   // column rows a wave probes together
+constexpr int JT_OWN = JT_COLS / (JT_THREADS / WAVE); // columns of a tile that one wave owns: their pairs stay in its registers
 
 __device__ __forceinline__ uint32_t prop_slot(uint32_t id, uint32_t P) { return (uint32_t)(mix64(id) >> 40) & (P - 1); }
 
@@ -126,32 +130,44 @@ struct JoinLds {
     }
 };
 
-// acc = <rows, cols> over all 1024 dimensions for the 32 x 32 block of row ids `ra` (nr of them) and column ids
+// acc = <rows, cols> over the 8-float blocks [b_begin, b_end) of the dimensions for the 32 x 32 block of row ids `ra` (nr of them) and column ids
 // `cb` (nc of them); operand layout as gram_dense_tile. Rows / columns beyond the counts repeat the last one.
-__device__ __forceinline__ floatx16 join_dense_block(const CorpusView& C, const uint32_t* ra, uint32_t nr, const uint32_t* cb, uint32_t nc, int lane) {
+__device__ __forceinline__ floatx16 join_dense_block(const CorpusView& C, const uint32_t* ra, uint32_t nr, const uint32_t* cb, uint32_t nc, int lane,
+                                                     int b_begin, int b_end) {
     floatx16 acc;
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[v] = 0.f;
     const uint32_t ia = min((uint32_t)(lane & 31), nr - 1), ib = min((uint32_t)(lane & 31), nc - 1);
     const float4* pa = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ra[ia]]) * 16) + (lane >> 5);
     const float4* pb = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[cb[ib]]) * 16) + (lane >> 5);
-    for (int b = 0; b < DIM / 8; b += 4) {
-        float4 a[4], bb[4];
+    // operands of the next four 8-float blocks are requested before the current four are multiplied
+    constexpr int NB = 4;
+    float4 a[2][NB], bb[2][NB];
 #pragma unroll
-        for (int u = 0; u < 4; u++) { a[u] = pa[2 * (b + u)]; bb[u] = pb[2 * (b + u)]; }
+    for (int u = 0; u < NB; u++) { a[0][u] = pa[2 * (b_begin + u)]; bb[0][u] = pb[2 * (b_begin + u)]; }
+#pragma unroll 1
+    for (int b = b_begin; b < b_end; b += 2 * NB) {
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].x, bb[u].x, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].y, bb[u].y, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].z, bb[u].z, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].w, bb[u].w, acc, 0, 0, 0);
+        for (int half = 0; half < 2; half++) {
+            const int nb = b + (half + 1) * NB; // first block of the batch after this one
+            if (nb < b_end) {
+#pragma unroll
+                for (int u = 0; u < NB; u++) { a[half ^ 1][u] = pa[2 * (nb + u)]; bb[half ^ 1][u] = pb[2 * (nb + u)]; }
+            }
+#pragma unroll
+            for (int u = 0; u < NB; u++) {
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[half][u].x, bb[half][u].x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[half][u].y, bb[half][u].y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[half][u].z, bb[half][u].z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[half][u].w, bb[half][u].w, acc, 0, 0, 0);
+            }
         }
     }
     return acc;
 }
 
 template <bool NARROW>
-__global__ __launch_bounds__(JT_THREADS) void join_tile_kernel(JoinArgs a) {
+__global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void join_tile_kernel(JoinArgs a) {
     a.C.narrow = NARROW ? 1u : 0u;
     extern __shared__ __align__(16) char smem[];
     const JoinLds L(a.index_bits, a.slot_cap, NARROW);
@@ -218,52 +234,88 @@ __global__ __launch_bounds__(JT_THREADS) void join_tile_kernel(JoinArgs a) {
             __builtin_amdgcn_wave_barrier();
             lst[rank] = mine;
         }
-        // dense part: wave w owns the 32-column block w
-        if ((uint32_t)(wave * 32) < M) {
-            const uint32_t nc = min(32u, M - wave * 32);
-            const floatx16 acc = join_dense_block(a.C, row_id, R, col_id + wave * 32, nc, lane);
+        // dense part: wave w takes the 32-column block (w & 3) over half (w >> 2) of the dimensions; the second half is
+        // added after a barrier
+        {
+            const int blk = wave & 3, part = wave >> 2;
+            const bool active = (uint32_t)(blk * 32) < M;
+            floatx16 acc;
+            if (active) acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, part * (DIM / 16), (part + 1) * (DIM / 16));
+            auto store = [&](bool add) {
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int i = 8 * (e / 4) + 4 * (lane >> 5) + (e % 4), j = lane & 31;
-                G[i * JT_STRIDE + wave * 32 + j] = a.dense_mul * acc[e];
-            }
+                for (int e = 0; e < 16; e++) {
+                    const int i = 8 * (e / 4) + 4 * (lane >> 5) + (e % 4), j = lane & 31;
+                    float* at = &G[i * JT_STRIDE + blk * 32 + j];
+                    *at = add ? *at + a.dense_mul * acc[e] : a.dense_mul * acc[e];
+                }
+            };
+            if (active && part == 0) store(false);
+            __syncthreads();
+            if (active && part == 1) store(true);
         }
         __syncthreads();
-        // sparse part: groups of four rows in the rank table, every column probes it once per group
+        // sparse part: groups of four rows in the rank table, every column probes it once per group. The pairs of a
+        // group's rows are requested while the group before it is probed; the pairs of a wave's columns stay in its
+        // registers for the whole tile: a build and the probes find their operands there.
+        auto row_pairs = [&](uint32_t i) { Pairs p = gram_row(a.C, rowptr, rownnz, i); p.narrow = NARROW ? 1u : 0u; return p; };
+        auto col_pairs = [&](uint32_t b) { Pairs p = gram_row(a.C, rowptr + JT_ROWS, rownnz + JT_ROWS, b); p.narrow = NARROW ? 1u : 0u; return p; };
         uint32_t a0 = 0;
+        PivotRegs pv;
+        ranktab_pivots_load(pv, [&](uint32_t t) { return row_pairs(a0 + t); }, min((uint32_t)RT_T, R - a0), tid, JT_THREADS);
+        // the wave's columns wave, wave + NW, ...: read once per tile, probed once per group; their shapes
+        // (nnz | ns << 16) are wave-uniform and stay in scalar registers
+        RtRow<NARROW> own[JT_OWN];
+        uint32_t own_shape[JT_OWN];
+#pragma unroll
+        for (int k = 0; k < JT_OWN; k++) {
+            const uint32_t b = wave + k * NW;
+            own_shape[k] = 0;
+            if (b < M) {
+                own_shape[k] = uniform(rownnz[JT_ROWS + b]);
+                rt_row_load(own[k], col_pairs(b), lane);
+            }
+        }
         while (a0 < R) {
             uint32_t nt = min((uint32_t)RT_T, R - a0);
             uint32_t built;
             while (true) {
-                built = ranktab_build<NARROW>(T, [&](uint32_t t) { Pairs p = gram_row(a.C, rowptr, rownnz, a0 + t); p.narrow = NARROW ? 1u : 0u; return p; }, nt, scan, tid, JT_THREADS);
+                built = ranktab_build<NARROW>(T, [&](uint32_t t) { return row_pairs(a0 + t); }, pv, nt, scan, tid, JT_THREADS);
                 if (built != EMPTY || nt == 1) break;
-                nt = (nt + 1) / 2;
+                nt = (nt + 1) / 2; // the registers hold the first pivots of the group whatever nt is
             }
+            const uint32_t a1 = a0 + nt;
+            if (a1 < R) ranktab_pivots_load(pv, [&](uint32_t t) { return row_pairs(a1 + t); }, min((uint32_t)RT_T, R - a1), tid, JT_THREADS);
             if (built == EMPTY) { // one row alone does not fit: its sparse part is missing, the host is told
                 if (tid == 0) atomicAdd(a.work + 3, 1ull);
-                a0 += nt;
+                a0 = a1;
                 continue;
             }
             const uint32_t n_ovf = NARROW ? 0u : uniform(min(scan[16], (uint32_t)RT_OVF));
-            uint32_t b = wave;
-            RtRow cur;
-            Pairs sp_cur;
-            if (b < M) { sp_cur = gram_row(a.C, rowptr + JT_ROWS, rownnz + JT_ROWS, b); sp_cur.narrow = NARROW ? 1u : 0u; rt_row_load(cur, sp_cur, lane); }
-            while (b < M) {
-                const uint32_t bn = b + NW;
-                RtRow nxt;
-                Pairs sp_nxt = sp_cur;
-                if (bn < M) { sp_nxt = gram_row(a.C, rowptr + JT_ROWS, rownnz + JT_ROWS, bn); sp_nxt.narrow = NARROW ? 1u : 0u; rt_row_load(nxt, sp_nxt, lane); }
-                float acc[RT_T] = {0.f, 0.f, 0.f, 0.f};
-                ranktab_probe_row<NARROW>(T, cur, sp_cur, n_ovf, acc, lane);
-                uint32_t t;
-                const float z = wave_sum4_dpp(acc, lane, &t);
-                if (lane < RT_T && t < nt) G[(a0 + t) * JT_STRIDE + b] += z;
-                cur = nxt;
-                sp_cur = sp_nxt;
-                b = bn;
+#pragma unroll
+            for (int q = 0; q < JT_OWN / JT_BATCH; q++) {
+                const uint32_t b0 = wave + q * JT_BATCH * NW;
+                if (b0 < M) { // wave-uniform
+                    float acc[JT_BATCH][RT_T];
+                    RtRow<NARROW> rows[JT_BATCH];
+                    uint32_t shape[JT_BATCH];
+#pragma unroll
+                    for (int k = 0; k < JT_BATCH; k++) {
+                        rows[k] = own[q * JT_BATCH + k];
+                        rows[k].touch();
+                        shape[k] = own_shape[q * JT_BATCH + k];
+                        asm volatile("" : "+s"(shape[k])); // as touch(): the lane masks of a row are made where they are used
+#pragma unroll
+                        for (int t = 0; t < RT_T; t++) acc[k][t] = 0.f;
+                    }
+                    ranktab_probe_rows<NARROW, JT_BATCH>(T, rows, shape, [&](int k) { return col_pairs(b0 + k * NW); }, n_ovf, acc, lane);
+                    uint32_t t, r;
+                    const float z = wave_sum_rows<JT_BATCH>(acc, lane, &t, &r);
+                    const uint32_t b = b0 + r * NW;
+                    if ((lane & 15) < RT_T && t < nt && b < M) G[(a0 + t) * JT_STRIDE + b] += z;
+                }
+                __builtin_amdgcn_sched_barrier(0); // one batch at a time: the scheduler must not pile up the reads of all of them
             }
-            a0 += nt;
+            a0 = a1;
             __syncthreads();
         }
         // proposals
