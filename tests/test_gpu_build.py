@@ -189,25 +189,44 @@ def test_entry_points_match_oracle(pruned):
     assert np.array_equal(pruned["entry"], O.entry_points(pruned["norms"], 32))
 
 
-def test_gpu_built_index_recall(gpu_world):
-    """Whole GPU build; recall@10 of search on it within 0.5 points of the oracle-built index."""
+def _mean_recall(graphs, ctx, gc, gq, truth, cands):
     import apoe
-    import oracle as O
     from parity import recall_at_k
+    out = []
+    for g in graphs:
+        ids, _, _ = apoe.search(ctx, gc, gq, g, (1.0, 1.0, 1.0), cands)
+        out.append(recall_at_k(ids, truth, 10))
+    return float(np.mean(out)), out
+
+
+@pytest.mark.parametrize("join", [0, 1])
+def test_gpu_built_index_recall(gpu_world, join):
+    """Whole GPU build (expansion step and local join): recall@10 of the search on it within 0.5 points of the
+    oracle-built index. Both builds start from random lists (and the GPU's expansion step races, as the reference's
+    does), so each side is the mean over three seeds, measured on 2 000 queries against exact brute force."""
+    import apoe
+    import apoe_synth as S
+    import oracle as O
     w = gpu_world
-    graph, ms = apoe.build_graph(w["ctx"], w["gc"], K=64, iters=8, degree=32, dense_scale=7.0, seed=5)
-    w3 = (1.0, 1.0, 1.0)
-    truth, _ = O.bruteforce_topk(w["C"], w["Q"], w3, 10)
-    ids_g, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], graph, w3, 128)
-    ids_c, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], w3, 128)
-    r_g, r_c = recall_at_k(ids_g, truth, 10), recall_at_k(ids_c, truth, 10)
-    print(f"recall@10 cands=128: gpu-built {r_g:.4f}, oracle-built {r_c:.4f}, gpu build {ms:.1f} ms")
-    # both builds race (so does the reference's) and each one's recall moves by half a point between runs:
-    # 0.950-0.961 for the GPU build, 0.944-0.954 for the oracle's over two dozen runs
-    assert r_g >= r_c - 0.01
-    rows, entry = graph.download()
+    if w["gc"].pair_bytes() == 8:
+        pytest.skip("one pair format is enough here: the build kernels are compared per format in the tests above")
+    q_arrays = S.to_numpy(S.queries(2000, seed=412))
+    Q = O.HybridSet(*q_arrays)
+    gq = apoe.Queries(w["ctx"], *q_arrays)
+    truth, _ = O.bruteforce_topk(w["C"], Q, (1.0, 1.0, 1.0), 10)
+    seeds = (5, 6, 7)
+    g_gpu = [apoe.build_graph(w["ctx"], w["gc"], K=64, iters=8, degree=32, dense_scale=7.0, seed=s, join=join)[0] for s in seeds]
+    g_orc = [apoe.Graph(w["ctx"], *O.build_index(w["C"], dense_scale=7.0, K=64, iters=8, d=32, seed=s)) for s in seeds]
+    for cands in (64, 128):
+        r_g, all_g = _mean_recall(g_gpu, w["ctx"], w["gc"], gq, truth, cands)
+        r_c, all_c = _mean_recall(g_orc, w["ctx"], w["gc"], gq, truth, cands)
+        print(f"join={join} cands={cands}: recall@10 gpu-built {r_g:.4f} {np.round(all_g, 4)}, oracle-built {r_c:.4f} {np.round(all_c, 4)}")
+        assert r_g >= r_c - 0.005
+    rows, entry = g_gpu[0].download()
     assert rows.shape == (w["C"].n, 40) and len(entry) == 32
-    graph.close()
+    for g in g_gpu + g_orc:
+        g.close()
+    gq.close()
 
 
 def test_prune_k128_sequential_kernel_matches_oracle(gpu_world):

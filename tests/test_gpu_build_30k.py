@@ -1,0 +1,70 @@
+"""Build parity where list quality starts to drop: 30 000 docs (kNN-list recall of a 10-step build is well below 1
+here). Recall@10 of the search on the GPU-built index (expansion step and local join, mean over three seeds) against
+the index the oracle builds with the reference's algorithm, on 2 000 queries and exact brute force; and the K-NN lists
+of both against exact lists of a node sample."""
+import numpy as np
+import pytest
+
+from parity import recall_at_k
+
+pytestmark = pytest.mark.gpu
+
+N, NQ = 30_000, 2_000
+
+
+@pytest.fixture(scope="module")
+def world30k(gpu_ctx):
+    import torch
+    import apoe
+    import apoe_synth as S
+    import apoe_bruteforce as B
+    import oracle as O
+    corpus = S.corpus(N, seed=201, device="cuda:0")
+    queries = S.queries(NQ, seed=202, device="cuda:0")
+    gc, gq = apoe.Corpus(gpu_ctx, *corpus), apoe.Queries(gpu_ctx, *queries)
+    truth, _ = B.hybrid_topk(corpus, queries, (1.0, 1.0, 1.0), 10)
+    samp = torch.arange(0, N, 15, device="cuda:0")
+    exact, _ = B.hybrid_topk(corpus, B.rows_as_queries(corpus, samp), (49.0, 1.0, 1.0), 64, self_ids=samp.cpu().numpy())
+    C = O.HybridSet(*S.to_numpy(corpus))
+    rows, entry, knn_ids, _ = O.build_index(C, dense_scale=7.0, K=64, iters=10, d=32, seed=5, return_knn=True)
+    yield dict(ctx=gpu_ctx, gc=gc, gq=gq, truth=truth, samp=samp.cpu().numpy(), exact=exact, o_rows=rows, o_entry=entry, o_knn=knn_ids)
+    gq.close()
+    gc.close()
+
+
+def _knn_recall(ids, truth, k):
+    return float(np.mean([len(set(ids[i, :k].tolist()) & set(truth[i, :k].tolist())) / k for i in range(len(truth))]))
+
+
+@pytest.mark.parametrize("join", [0, 1, 2])
+def test_build_recall_within_half_a_point_of_the_oracle_build(world30k, join):
+    import apoe
+    w = world30k
+    og = apoe.Graph(w["ctx"], w["o_rows"], w["o_entry"])
+    lists, graphs = [], []
+    for seed in (5, 6, 7):
+        knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+        knn.set_join(join)
+        knn.init(seed)
+        for it in range(10):
+            knn.iterate(last=(it == 9))
+        knn.merge_reverse()
+        lists.append(_knn_recall(knn.download()[0][w["samp"]], w["exact"], 10))
+        knn.prune(32)
+        graphs.append(knn.finalize())
+        knn.close()
+    l_o = _knn_recall(w["o_knn"][w["samp"]], w["exact"], 10)
+    print(f"join={join}: K-NN list recall@10 gpu {np.round(lists, 4)} oracle {l_o:.4f}")
+    assert np.mean(lists) >= l_o - 0.005
+    for cands in (128, 512):
+        r_g = []
+        for g in graphs:
+            ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], g, (1.0, 1.0, 1.0), cands)
+            r_g.append(recall_at_k(ids, w["truth"], 10))
+        ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], og, (1.0, 1.0, 1.0), cands)
+        r_o = recall_at_k(ids, w["truth"], 10)
+        print(f"join={join} cands={cands}: search recall@10 gpu-built {np.round(r_g, 4)} mean {np.mean(r_g):.4f}, oracle-built {r_o:.4f}")
+        assert np.mean(r_g) >= r_o - 0.005
+    for g in graphs:
+        g.close()
+    og.close()

@@ -1,12 +1,7 @@
 """The whole path at 100 000 docs (degree 32, K = 64, 10 NN-Descent steps, cands 128): the oracle checks a
 sample, the rest is checked through properties that do not depend on the size."""
-import os
-import sys
-
 import numpy as np
 import pytest
-
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))  # bench.py's torch ground truth
 
 from parity import assert_dist_close, assert_topk_match, recall_at_k
 
@@ -96,10 +91,10 @@ def test_sample_matches_oracle_on_the_gpu_built_graph(world):
 def test_recall_grows_with_the_pool_and_beats_a_random_graph(world):
     import torch
     import apoe
-    from bench import ground_truth
+    import apoe_bruteforce as B
     w = world
     nq = 500
-    truth, _ = ground_truth(torch, w["corpus"], w["queries"], (1.0, 1.0, 1.0), 10, nq)
+    truth, _ = B.hybrid_topk(w["corpus"], w["queries"], (1.0, 1.0, 1.0), 10, nq=nq)
     rec = []
     for cands in (32, 128, 512):
         ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], w["graph"], (1, 1, 1), cands, q_count=nq)
