@@ -89,6 +89,10 @@ struct apoe_ctx {
     // a device allocation each. One search at a time per context.
     apoe::DevBuf<char> search_ws;
     char* static_ws = nullptr; // this GPU's copy of the static workspace of apoe_search_noalloc
+    // Upload pipeline for large pageable host arrays: two pinned staging buffers that host threads fill while the
+    // copy engine drains the other one (created on first use, kept until the context is destroyed).
+    void* pinned[2] = {nullptr, nullptr};
+    hipEvent_t pinned_done[2] = {nullptr, nullptr};
     int search_workspace(size_t bytes, char** out) {
         if (search_ws.n < bytes) APOE_TRY(search_ws.alloc(bytes));
         *out = search_ws.p;

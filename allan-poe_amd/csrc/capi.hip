@@ -2,8 +2,10 @@
 // wrappers that stage caller memory and call the kernel launchers.
 #include <algorithm>
 #include <cmath>
+#include <cstring>
 #include <memory>
 #include <numeric>
+#include <thread>
 
 #include "apoe_internal.h"
 
@@ -30,8 +32,61 @@ static bool is_device_ptr(const void* p) {
     return attr.type == hipMemoryTypeDevice;
 }
 
+constexpr size_t STREAM_CHUNK = 32u << 20;     // bytes per pinned staging buffer
+constexpr size_t STREAM_MIN = 4 * STREAM_CHUNK; // smaller uploads go through the plain copy
+
+static int host_copy_threads() {
+    const unsigned hw = std::thread::hardware_concurrency();
+    return (int)std::min(8u, std::max(1u, hw / 2));
+}
+
+// Pageable host memory -> device through the two pinned buffers: while the copy engine moves chunk i out of one buffer,
+// host threads fill the other with chunk i + 1 (the reference copies whole arrays with blocking cudaMemcpy from pageable
+// memory, index.cu:842-877, query.cu:1901-1980).
+static int stream_in(apoe_ctx* ctx, char* dst_dev, const char* src_host, size_t bytes) {
+    for (int b = 0; b < 2; b++) {
+        if (!ctx->pinned[b]) APOE_HIP(hipHostMalloc(&ctx->pinned[b], STREAM_CHUNK, hipHostMallocDefault));
+        if (!ctx->pinned_done[b]) APOE_HIP(hipEventCreateWithFlags(&ctx->pinned_done[b], hipEventDisableTiming));
+    }
+    const int nt = host_copy_threads();
+    bool used[2] = {false, false};
+    size_t i = 0;
+    for (size_t off = 0; off < bytes; off += STREAM_CHUNK, i++) {
+        const int b = (int)(i & 1);
+        const size_t len = std::min(STREAM_CHUNK, bytes - off);
+        if (used[b]) APOE_HIP(hipEventSynchronize(ctx->pinned_done[b])); // the copy that last read this buffer has finished
+        char* stage = static_cast<char*>(ctx->pinned[b]);
+        if (nt == 1) {
+            std::memcpy(stage, src_host + off, len);
+        } else {
+            std::thread workers[8];
+            const size_t part = ((len + nt - 1) / nt + 4095) & ~(size_t)4095;
+            int started = 0;
+            for (int t = 0; t < nt; t++) {
+                const size_t p0 = (size_t)t * part;
+                if (p0 >= len) break;
+                const size_t pl = std::min(part, len - p0);
+                workers[started++] = std::thread([=]() { std::memcpy(stage + p0, src_host + off + p0, pl); });
+            }
+            for (int t = 0; t < started; t++) workers[t].join();
+        }
+        APOE_HIP(hipMemcpyAsync(dst_dev + off, stage, len, hipMemcpyHostToDevice, ctx->stream));
+        APOE_HIP(hipEventRecord(ctx->pinned_done[b], ctx->stream));
+        used[b] = true;
+    }
+    APOE_HIP(hipStreamSynchronize(ctx->stream));
+    return APOE_OK;
+}
+
 int copy_in(apoe_ctx* ctx, void* dst_dev, const void* src_any, size_t bytes) {
     if (bytes == 0) return APOE_OK;
+    if (bytes >= STREAM_MIN) {
+        hipPointerAttribute_t attr;
+        const hipError_t e = hipPointerGetAttributes(&attr, src_any);
+        if (e != hipSuccess) (void)hipGetLastError(); // plain host memory is reported as an error
+        const bool pageable = e != hipSuccess || attr.type == hipMemoryTypeUnregistered;
+        if (pageable) return stream_in(ctx, static_cast<char*>(dst_dev), static_cast<const char*>(src_any), bytes);
+    }
     APOE_HIP(hipMemcpyAsync(dst_dev, src_any, bytes, hipMemcpyDefault, ctx->stream));
     APOE_HIP(hipStreamSynchronize(ctx->stream));
     return APOE_OK;
@@ -126,6 +181,10 @@ void apoe_ctx_destroy(apoe_ctx* ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    for (int b = 0; b < 2; b++) {
+        if (ctx->pinned_done[b]) (void)hipEventDestroy(ctx->pinned_done[b]);
+        if (ctx->pinned[b]) (void)hipHostFree(ctx->pinned[b]);
+    }
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }

@@ -1,6 +1,9 @@
 #!/usr/bin/env python3
 """Headline benchmark: search QPS at recall@10 >= 0.95 and index build seconds on a
 synthetic hybrid corpus (dense 1024-d + SPLADE-like CSR + BM25-like CSR), one MI355X.
+When no pool of the sweep reaches the recall target the line says so in `metric`,
+`config.recall_target_met` and `config.qps_at_recall_target` (null), and `value` is the
+rate at the largest configured pool (256).
 
 A "step" is one pass of the beam-search kernel over the whole query batch, inputs
 already resident in HBM. The JSON line also carries the roofline of the search kernel
@@ -22,63 +25,15 @@ sys.path.insert(0, os.path.join(ROOT, "allan-poe_amd"))
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per search launch from FETCH_SIZE + WRITE_SIZE counter runs (rocprofv3 --pmc,
-# scaled by what the counters read for a 1 GiB copy), keyed by the workload they were taken on:
-# (docs, degree, queries, cands, variant). Other workloads report null.
-MEASURED_TRAFFIC = {
-    (1000000, 48, 10000, 512, 0): 331965225494,
-}
-# The same for the launches that read every dense row (variant | 0x100).
-MEASURED_TRAFFIC_FULL = {
-    (1000000, 48, 10000, 512, 0): 910016881459,
-}
+# HBM bytes per search launch, RECORDED from FETCH_SIZE + WRITE_SIZE counter runs (rocprofv3 --pmc, scaled by what the
+# counters read for a 1 GiB copy) and not measured by this script: keyed by the workload they were taken on
+# (docs, degree, queries, cands, variant, NN-Descent step) with the profiles/ file that holds the run. Any other
+# workload reports null.
+RECORDED_TRAFFIC = {}
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
-
-
-def ground_truth(torch, corpus, queries, w3, k, nq, chunk=4096):
-    """Exact hybrid top-k of the first nq queries, by torch on the GPU (checker only).
-    dense: matmul; sparse: gather of a dense [2*vocab, nq] query-term matrix."""
-    import apoe_synth as S
-    dense, s_off, s_idx, s_val, b_off, b_idx, b_val = corpus
-    qd, qs_off, qs_idx, qs_val, qb_off, qb_idx, qb_val = queries
-    dev = dense.device
-    n = dense.shape[0]
-    V = S.VOCAB
-    Qt = torch.zeros(2 * V, nq, device=dev)
-    for off, idx, val, base, w in ((qs_off, qs_idx, qs_val, 0, w3[1]), (qb_off, qb_idx, qb_val, V, w3[2])):
-        if w < 1e-5:
-            continue
-        cnt = (off[1:nq + 1] - off[:nq]).long()
-        rows = torch.repeat_interleave(torch.arange(nq, device=dev), cnt)
-        e = int(off[nq])
-        Qt[idx[:e].long() + base, rows] = val[:e] * w
-    qdw = qd[:nq] * w3[0]
-    best_d = torch.full((nq, k), float("inf"), device=dev)
-    best_i = torch.zeros((nq, k), dtype=torch.long, device=dev)
-    for r0 in range(0, n, chunk):
-        r1 = min(n, r0 + chunk)
-        ip = torch.zeros(r1 - r0, nq, device=dev)
-        if w3[0] >= 1e-5:
-            ip += dense[r0:r1] @ qdw.T
-        for off, idx, val, base, w in ((s_off, s_idx, s_val, 0, w3[1]), (b_off, b_idx, b_val, V, w3[2])):
-            if w < 1e-5:
-                continue
-            e0, e1 = int(off[r0]), int(off[r1])
-            if e1 == e0:
-                continue
-            cnt = (off[r0 + 1:r1 + 1] - off[r0:r1]).long()
-            rows = torch.repeat_interleave(torch.arange(r1 - r0, device=dev), cnt)
-            contrib = Qt.index_select(0, idx[e0:e1].long() + base) * val[e0:e1, None]
-            ip.index_add_(0, rows, contrib)
-        dist = (1.0 - ip).T  # [nq, chunk]
-        cat_d = torch.cat([best_d, dist], 1)
-        cat_i = torch.cat([best_i, torch.arange(r0, r1, device=dev).expand(nq, -1)], 1)
-        best_d, sel = torch.topk(cat_d, k, dim=1, largest=False)
-        best_i = torch.gather(cat_i, 1, sel)
-    return best_i.cpu().numpy(), best_d.cpu().numpy()
 
 
 def recall_at_k(found, truth, k):
@@ -86,6 +41,25 @@ def recall_at_k(found, truth, k):
     for f, t in zip(found, truth):
         hit += len(set(f[:k].tolist()) & set(t[:k].tolist()))
     return hit / (len(truth) * k)
+
+
+def build_index(apoe, ctx, gc, args, join, keep_lists=False):
+    """NN-Descent + reverse merge + prune + final rows; returns (graph, timings dict, K-NN ids or None)."""
+    t0 = time.time()
+    knn = apoe.Knn(ctx, gc, args.nnd_k, 7.0)
+    knn.set_join(join)
+    knn.init(1)
+    for it in range(args.nnd_iters):
+        knn.iterate(last=(it == args.nnd_iters - 1))
+    nnd_ms = knn.elapsed_ms()
+    evals, rows = knn.counters()
+    knn.merge_reverse()
+    lists = knn.download()[0] if keep_lists else None
+    knn.prune(args.degree)
+    graph = knn.finalize()
+    total_ms = knn.elapsed_ms()
+    knn.close()
+    return graph, dict(nnd_ms=nnd_ms, total_ms=total_ms, wall_s=time.time() - t0, evaluations=evals, rows_read=rows), lists
 
 
 def main():
@@ -98,15 +72,19 @@ def main():
     ap.add_argument("--degree", type=int, default=48)
     ap.add_argument("--nnd-k", type=int, default=64)
     ap.add_argument("--nnd-iters", type=int, default=10)
-    ap.add_argument("--cands", type=str, default="64,128,256,512")
+    ap.add_argument("--join", type=int, default=1, help="NN-Descent step of the index the searches run on: 0 the reference's expansion step, "
+                    "1 the local join around the picked neighbour (same pairs), 2 the join that updates both endpoints")
+    ap.add_argument("--cands", type=str, default="64,128,256,512,1024,2048",
+                    help="pool sizes of the recall sweep; 64,128,256 are the configured ones, the larger ones look for the recall target")
     ap.add_argument("--truth-queries", type=int, default=1000)
     ap.add_argument("--cpu-queries", type=int, default=10000)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-membench", action="store_true", help="do not run bench/membench for roofline.random_read_ceiling")
+    ap.add_argument("--no-sweeps", action="store_true", help="skip the query-time weight sweep and the knowledge-graph search (about 10 s)")
     ap.add_argument("--extras", action="store_true",
-                    help="also time the other search paths at cands=128: the query-time weight sweep, the knowledge-graph search "
-                         "(200k entities, 1-3 entities per query, kg_weight 40) and the keyword-filter search (rarest BM25 term of each query)")
+                    help="also time: the keyword-filter search, a four times longer batch, the corpus handed over as host buffers, "
+                         "the half-precision walks and build")
     ap.add_argument("--calibrate", action="store_true",
                     help="apply the reference's query-time weight calibration to the 1/1/1 weights (off: the metric is literally 1/1/1)")
     ap.add_argument("--copy-calib", action="store_true",
@@ -118,6 +96,7 @@ def main():
     import numpy as np
     import torch
     import apoe
+    import apoe_bruteforce as B
     import apoe_synth as S
 
     if not torch.cuda.is_available():
@@ -136,35 +115,53 @@ def main():
     gq = apoe.Queries(ctx, *queries)
     log(f"[bench] packed corpus: {gc.bytes() / 1e9:.2f} GB of records in {time.time() - t0:.2f}s")
 
-    # ---- index build (NN-Descent + reverse merge + RNG-IP prune + final rows) ----
-    t0 = time.time()
-    knn = apoe.Knn(ctx, gc, args.nnd_k, 7.0)
-    knn.init(1)
-    for it in range(args.nnd_iters):
-        knn.iterate(last=(it == args.nnd_iters - 1))
-    nnd_ms = knn.elapsed_ms()
-    nnd_evals, nnd_dense = knn.counters()
-    knn.merge_reverse()
-    knn.prune(args.degree)
-    graph = knn.finalize()
-    build_gpu_ms = knn.elapsed_ms()
-    knn.close()
-    build_wall = time.time() - t0
+    # ---- index build (NN-Descent + reverse merge + RNG-IP prune + final rows), with both NN-Descent steps ----
     mean_pairs = (corpus[2].numel() + corpus[5].numel()) / args.docs
-    nnd_bytes = nnd_dense * 4096 + nnd_evals * (gc.pair_bytes() * mean_pairs + 12)
-    log(f"[bench] build: {build_gpu_ms / 1e3:.2f}s GPU time ({build_wall:.2f}s wall); NN-Descent {nnd_ms / 1e3:.2f}s, "
-        f"{nnd_evals / 1e9:.2f}G evaluations, {nnd_dense / 1e9:.2f}G dense rows, {nnd_bytes / (nnd_ms / 1e3) / 1e12:.2f} TB/s algorithmic")
+    row_bytes = 4096 + gc.pair_bytes() * mean_pairs + 12
+    builds = {}
+    graph = None
+    lists = None
+    for join in sorted({0, args.join}):
+        g, tm, ls = build_index(apoe, ctx, gc, args, join, keep_lists=True)
+        if join == 0:
+            # expansion step: an evaluation reads pairs + descriptor, and the dense row when the bound does not settle it
+            tm["algo_bytes"] = tm["rows_read"] * 4096 + tm["evaluations"] * (gc.pair_bytes() * mean_pairs + 12)
+        else:
+            # join: every row of a tile is read once, in full
+            tm["algo_bytes"] = tm["rows_read"] * row_bytes
+        builds[join] = tm
+        log(f"[bench] build (NN-Descent step {join}): {tm['total_ms'] / 1e3:.2f}s GPU time ({tm['wall_s']:.2f}s wall); NN-Descent {tm['nnd_ms'] / 1e3:.2f}s, "
+            f"{tm['evaluations'] / 1e9:.2f}G pair evaluations, {tm['rows_read'] / 1e9:.3f}G rows read, {tm['algo_bytes'] / (tm['nnd_ms'] / 1e3) / 1e12:.2f} TB/s algorithmic")
+        if join == args.join:
+            graph, lists = g, ls
+        else:
+            builds[join]["lists"] = ls
+            g.close()
+    # K-NN list quality of both builds against exact lists of a node sample (brute force by torch)
+    gsamp = torch.Generator(device="cpu")
+    gsamp.manual_seed(7)
+    samp = torch.sort(torch.randperm(args.docs, generator=gsamp)[:1000])[0].to(dev)
+    exact, _ = B.hybrid_topk(corpus, B.rows_as_queries(corpus, samp), (49.0, 1.0, 1.0), 10, self_ids=samp.cpu().numpy())
+    samp_np = samp.cpu().numpy()
+    for join, tm in builds.items():
+        ls = tm.pop("lists", None)
+        ls = lists if ls is None else ls
+        tm["knn_list_recall_at_10"] = float(np.mean([len(set(ls[samp_np[i], :10].tolist()) & set(exact[i].tolist())) / 10 for i in range(len(samp_np))]))
+        log(f"[bench] NN-Descent step {join}: K-NN list recall@10 on 1000 sampled nodes {tm['knn_list_recall_at_10']:.4f}")
+    del lists
+    bt = builds[args.join]
 
     # ---- effective weights and exact ground truth on a query subset ----
     w3 = apoe.calibrate_weights(ctx, gc, gq, (1.0, 1.0, 1.0)) if args.calibrate else (1.0, 1.0, 1.0)
     nq_truth = min(args.truth_queries, args.queries)
     t0 = time.time()
-    truth, _ = ground_truth(torch, corpus, queries, w3, 10, nq_truth)
+    truth, _ = B.hybrid_topk(corpus, queries, w3, 10, nq=nq_truth)
     log(f"[bench] effective weights dense/sparse/bm25 = {w3}; ground truth for {nq_truth} queries in {time.time() - t0:.1f}s")
 
-    # ---- cands sweep: recall, then timed steps ----
+    # ---- pool sweep: recall and one launch each ----
     sweep = []
     for cands in [int(c) for c in args.cands.split(",")]:
+        apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant)
         ids, dist, st = apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant)
         rec = recall_at_k(ids[:nq_truth], truth, 10)
         sweep.append(dict(cands=cands, recall=rec, ms=st.kernel_ms, qps=args.queries / (st.kernel_ms / 1e3),
@@ -173,8 +170,10 @@ def main():
             f"{sweep[-1]['gbs']:.0f} GB/s algorithmic, {st.evaluations / args.queries:.0f} evals/query, "
             f"{st.dense_rows / max(st.evaluations, 1):.2f} of them read the dense row")
     ok = [s for s in sweep if s["recall"] >= 0.95]
-    # the smallest pool that reaches the recall target; if none does, the largest pool tried
-    pick = ok[0] if ok else sweep[-1]
+    # the smallest pool that reaches the recall target; if none does, the largest configured pool (256) stands in and the
+    # line says so: `value` is then NOT a rate at the target
+    configured = [s for s in sweep if s["cands"] <= 256] or sweep
+    pick = ok[0] if ok else configured[-1]
     cands = pick["cands"]
 
     out_ids = torch.empty((args.queries, cands), dtype=torch.int32, device=dev)
@@ -203,24 +202,47 @@ def main():
             full_ms.append(stf.kernel_ms)
             full_bytes = stf.algo_bytes
     full_avg = sum(full_ms) / len(full_ms)
+    key = (args.docs, args.degree, args.queries, cands, args.variant, args.join)
+    rec_traffic = RECORDED_TRAFFIC.get(key) if not args.calibrate else None
     full_eval = {"kernel_ms": full_avg, "qps": args.queries / (full_avg / 1e3), "achieved": full_bytes / (full_avg / 1e3) / 1e9,
                  "frac": full_bytes / (full_avg / 1e3) / 1e9 / HBM_PEAK_GBS, "algo_bytes_per_launch": full_bytes,
-                 "traffic": MEASURED_TRAFFIC_FULL.get((args.docs, args.degree, args.queries, cands, args.variant))
-                 if not args.calibrate else None}
+                 "traffic": rec_traffic["every_dense_row_read"] if rec_traffic else None}
     log(f"[bench] timed: {avg_kernel_ms:.2f} ms/launch, {achieved:.0f} GB/s algorithmic; every dense row read: {full_avg:.2f} ms, "
         f"{full_eval['achieved']:.0f} GB/s")
+
+    # ---- the other searches of the configured workloads: query-time weight sweep without rebuild, knowledge graph ----
+    weight_sweep, kg_search = None, None
+    if not args.no_sweeps:
+        weight_sweep = []
+        for wx in ((1.0, 0.0, 0.0), (0.0, 1.0, 0.0), (0.0, 0.0, 1.0), (1.0, 1.0, 1.0), (1.0, 0.5, 2.0)):
+            tx, _ = B.hybrid_topk(corpus, queries, wx, 10, nq=nq_truth)
+            for ec in (64, 128, 256):
+                apoe.search(ctx, gc, gq, graph, wx, ec)
+                ids_x, _, sx = apoe.search(ctx, gc, gq, graph, wx, ec)
+                weight_sweep.append(dict(weights=wx, cands=ec, kernel_ms=sx.kernel_ms, qps=args.queries / (sx.kernel_ms / 1e3),
+                                         recall_at_10=recall_at_k(ids_x[:nq_truth], tx, 10), algo_gbs=sx.algo_bytes / (sx.kernel_ms / 1e3) / 1e9))
+                log(f"[bench] weights {wx} cands {ec}: {sx.kernel_ms:.2f} ms, recall {weight_sweep[-1]['recall_at_10']:.4f}")
+        kg = S.knowledge_graph(200_000, args.docs, args.queries, device=dev)
+        gkg = apoe.KnowledgeGraph(ctx, *kg)
+        apoe.search(ctx, gc, gq, graph, w3, 128, kg=gkg, kg_weight=40.0)
+        ids_k, _, sk = apoe.search(ctx, gc, gq, graph, w3, 128, kg=gkg, kg_weight=40.0)
+        # documents of the query's own entities among the top 10: what the logical edges bring in
+        q2e_off, q2e_idx, e2d_off, e2d_idx = kg[4].long(), kg[5].long(), kg[2].long(), kg[3].long()
+        hits = 0
+        for qi in range(nq_truth):
+            ents = q2e_idx[q2e_off[qi]:q2e_off[qi + 1]]
+            docs = torch.cat([e2d_idx[e2d_off[e]:e2d_off[e + 1]] for e in ents.tolist()]).tolist()
+            hits += len(set(docs) & set(ids_k[qi, :10].tolist())) > 0
+        kg_search = dict(entities=200_000, cands=128, kg_weight=40.0, kernel_ms=sk.kernel_ms, qps=args.queries / (sk.kernel_ms / 1e3),
+                         evaluations=int(sk.evaluations), algo_gbs=sk.algo_bytes / (sk.kernel_ms / 1e3) / 1e9,
+                         queries_with_an_entity_document_in_top10=hits / nq_truth)
+        log(f"[bench] KG search cands 128: {sk.kernel_ms:.2f} ms, entity document in the top 10 for {hits / nq_truth:.3f} of the queries")
+        gkg.close()
 
     extras = None
     if args.extras:
         extras = {}
         ec = 128
-        for wx in ((1.0, 0.0, 0.0), (0.0, 1.0, 0.0), (0.0, 0.0, 1.0), (1.0, 1.0, 1.0), (1.0, 0.5, 2.0)):
-            tx, _ = ground_truth(torch, corpus, queries, wx, 10, nq_truth)
-            apoe.search(ctx, gc, gq, graph, wx, ec, out_ids=None)
-            ids_x, _, sx = apoe.search(ctx, gc, gq, graph, wx, ec)
-            extras[f"weights {wx}"] = dict(kernel_ms=sx.kernel_ms, qps=args.queries / (sx.kernel_ms / 1e3), recall_at_10=recall_at_k(ids_x[:nq_truth], tx, 10),
-                                           algo_gbs=sx.algo_bytes / (sx.kernel_ms / 1e3) / 1e9)
-            log(f"[bench] extras: weights {wx} cands {ec}: {sx.kernel_ms:.2f} ms, recall {extras[f'weights {wx}']['recall_at_10']:.4f}")
         # the host boundary: the same corpus handed over as host (pageable) buffers, H2D included
         host = S.to_numpy(corpus)
         th = time.perf_counter()
@@ -250,11 +272,11 @@ def main():
             apoe.search(ctx, gc, gq, graph, hw, hc, variant=0x200 | args.variant)
             ids_h, _, sh = apoe.search(ctx, gc, gq, graph, hw, hc, variant=0x200 | args.variant)
             ids_d, _, sd = apoe.search(ctx, gc, gq, graph, hw, hc, variant=args.variant)
-            key = f"half-precision rows, weights {hw}, cands {hc}"
-            extras[key] = dict(kernel_ms=sh.kernel_ms, default_kernel_ms=sd.kernel_ms, same_top10=float((ids_h[:, :10] == ids_d[:, :10]).mean()),
-                               algo_gbs=sh.algo_bytes / (sh.kernel_ms / 1e3) / 1e9)
-            log(f"[bench] extras: {key}: {sh.kernel_ms:.2f} ms (fp32 rows {sd.kernel_ms:.2f} ms), top-10 ids equal at {extras[key]['same_top10']:.4f}")
-        # the build with NN-Descent steps on the half-precision rows (stored distances recomputed in fp32 before the prune)
+            key_h = f"half-precision rows, weights {hw}, cands {hc}"
+            extras[key_h] = dict(kernel_ms=sh.kernel_ms, default_kernel_ms=sd.kernel_ms, same_top10=float((ids_h[:, :10] == ids_d[:, :10]).mean()),
+                                 algo_gbs=sh.algo_bytes / (sh.kernel_ms / 1e3) / 1e9)
+            log(f"[bench] extras: {key_h}: {sh.kernel_ms:.2f} ms (fp32 rows {sd.kernel_ms:.2f} ms), top-10 ids equal at {extras[key_h]['same_top10']:.4f}")
+        # the build with NN-Descent (expansion) steps on the half-precision rows (stored distances recomputed in fp32 before the prune)
         knn_h = apoe.Knn(ctx, gc, args.nnd_k, 7.0)
         knn_h.use_half_rows()
         knn_h.init(20251125)
@@ -267,20 +289,11 @@ def main():
         build_h_ms = knn_h.elapsed_ms()
         knn_h.close()
         ids_gh, _, _ = apoe.search(ctx, gc, gq, graph_h, w3, ec)
-        ids_gf, _, _ = apoe.search(ctx, gc, gq, graph, w3, ec)
         extras["build with half-precision rows"] = dict(build_seconds_gpu=build_h_ms / 1e3, nnd_seconds_gpu=nnd_h_ms / 1e3,
-                                                        recall_at_10=recall_at_k(ids_gh[:nq_truth], truth, 10),
-                                                        recall_at_10_fp32_build=recall_at_k(ids_gf[:nq_truth], truth, 10))
+                                                        recall_at_10=recall_at_k(ids_gh[:nq_truth], truth, 10))
         log(f"[bench] extras: build with half-precision rows: {build_h_ms / 1e3:.2f}s (NN-Descent {nnd_h_ms / 1e3:.2f}s); recall@10 at cands {ec}: "
-            f"{extras['build with half-precision rows']['recall_at_10']:.4f} (fp32 build {extras['build with half-precision rows']['recall_at_10_fp32_build']:.4f})")
+            f"{extras['build with half-precision rows']['recall_at_10']:.4f}")
         graph_h.close()
-        kg = S.knowledge_graph(200_000, args.docs, args.queries, device=dev)
-        gkg = apoe.KnowledgeGraph(ctx, *kg)
-        apoe.search(ctx, gc, gq, graph, w3, ec, kg=gkg, kg_weight=40.0)
-        _, _, sk = apoe.search(ctx, gc, gq, graph, w3, ec, kg=gkg, kg_weight=40.0)
-        extras["knowledge graph, kg_weight 40"] = dict(kernel_ms=sk.kernel_ms, qps=args.queries / (sk.kernel_ms / 1e3), evaluations=int(sk.evaluations),
-                                                       algo_gbs=sk.algo_bytes / (sk.kernel_ms / 1e3) / 1e9)
-        log(f"[bench] extras: KG search cands {ec}: {sk.kernel_ms:.2f} ms")
         # keyword filter: flag the rarest BM25 term of each query (by document frequency)
         qb_off, qb_idx = queries[4].long(), queries[5].long()
         df = torch.bincount(corpus[5].long(), minlength=S.VOCAB)
@@ -333,8 +346,14 @@ def main():
                           f"{cpu_s:.1f}s; top-10 ids equal to the GPU's at {agree:.4f} of positions")
         log(f"[bench] cpu oracle: {cpu['value']:.0f} QPS on {threads} threads; top-10 agreement {agree:.4f}")
 
+    if ok:
+        metric = "search QPS @ recall@10>=0.95 (index build seconds in config)"
+    else:
+        best = max(sweep, key=lambda s: s["recall"])
+        metric = (f"search QPS at cands={cands}, recall@10 {pick['recall']:.3f}: the recall@10>=0.95 point of the configured metric is NOT reached on this corpus "
+                  f"(best {best['recall']:.3f} at cands {best['cands']}); index build seconds in config")
     result = {
-        "metric": "search QPS @ recall@10>=0.95 (index build seconds in config)",
+        "metric": metric,
         "value": args.queries / (ms_per_step / 1e3),
         "unit": "queries/s",
         "n_gpus": 1,
@@ -353,21 +372,33 @@ def main():
             "cands": cands,
             "recall_at_10": pick["recall"],
             "recall_target_met": bool(ok),
-            "build_seconds_gpu": build_gpu_ms / 1e3,
-            "build_seconds_wall": build_wall,
+            "qps_at_recall_target": (args.queries / (ms_per_step / 1e3)) if ok else None,
+            "build_seconds_gpu": bt["total_ms"] / 1e3,
+            "build_seconds_wall": bt["wall_s"],
+            "nnd_step": {0: "expansion (the reference's step)", 1: "local join around the picked neighbour", 2: "local join, both endpoints updated"}[args.join],
             "nnd_k": args.nnd_k,
             "nnd_iters": args.nnd_iters,
-            "nnd_seconds_gpu": nnd_ms / 1e3,
-            "nnd_evaluations": nnd_evals,
-            "nnd_dense_rows": nnd_dense,
-            "nnd_algo_gbs": nnd_bytes / (nnd_ms / 1e3) / 1e9,
+            "nnd_seconds_gpu": bt["nnd_ms"] / 1e3,
+            "nnd_pair_evaluations": bt["evaluations"],
+            "nnd_rows_read": bt["rows_read"],
+            "nnd_algo_gbs": bt["algo_bytes"] / (bt["nnd_ms"] / 1e3) / 1e9,
+            "knn_list_recall_at_10": bt["knn_list_recall_at_10"],
+            **({"build_with_the_reference_expansion_step": {
+                "build_seconds_gpu": builds[0]["total_ms"] / 1e3, "nnd_seconds_gpu": builds[0]["nnd_ms"] / 1e3, "nnd_pair_evaluations": builds[0]["evaluations"],
+                "nnd_dense_rows_read": builds[0]["rows_read"], "nnd_algo_gbs": builds[0]["algo_bytes"] / (builds[0]["nnd_ms"] / 1e3) / 1e9,
+                "knn_list_recall_at_10": builds[0]["knn_list_recall_at_10"]}} if args.join != 0 else {}),
             "cands_sweep": sweep,
             "kernel_ms": avg_kernel_ms,
+            **({"weight_sweep_without_rebuild": weight_sweep} if weight_sweep else {}),
+            **({"knowledge_graph_search": kg_search} if kg_search else {}),
             **({"extras": extras} if extras else {}),
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC.get((args.docs, args.degree, args.queries, cands, args.variant)) if not args.calibrate else None,
+                     # HBM bytes per launch from rocprofv3 counter runs recorded in profiles/ (not measured in this run): null for any other workload
+                     "traffic": rec_traffic["default"] if rec_traffic else None,
+                     "traffic_source": rec_traffic["source"] if rec_traffic else None,
                      "kernel": "search_kernel", "algo_bytes_per_launch": algo_bytes,
+                     "at_recall_target": bool(ok),
                      "mode": "dense row read only when the sparse part plus the bound of the dense part can enter the pool",
                      # the same evaluations priced as the reference prices them (every evaluation reads its dense row), over the
                      # default mode's time: what a kernel without the bound would have to sustain to be as fast
