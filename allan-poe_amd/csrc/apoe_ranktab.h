@@ -4,7 +4,7 @@
 //
 //   word[w] = (bits, count of set bits in words before w)      one ds_read_b64 per look-up
 //   slot of a term = count + popcount(bits below its bit)      no hashing, no probe loop, no key compare
-//   vals[slot] = one value per pivot of the group (zero where the pivot lacks the term): one ds_read_b128
+//   vals[slot] = one value per pivot of the group (zero where the pivot lacks the term): two ds_read_b128
 //
 // A corpus in the narrow pair format (term ids below 65536, the path known from the position in the row)
 // maps a term to bit (term | path * span) with span = the power of two above the largest term id: distinct
@@ -19,7 +19,7 @@ namespace apoe {
 
 #ifdef __HIPCC__
 
-constexpr int RT_T = 4;     // pivots per table: one float4 per term
+constexpr int RT_T = 8;     // pivots per table: two float4 per term
 constexpr int RT_OVF = 32;  // overflow entries (wide corpora only)
 
 struct RankTabLds { // byte offsets inside the table region
@@ -39,7 +39,7 @@ struct RankTabLds { // byte offsets inside the table region
 struct RankTab {
     uint2* word;      // [index_bits / 32]
     uint32_t* keys;   // [slot_cap], wide only
-    float4* vals;     // [slot_cap]
+    float4* vals;     // [slot_cap][RT_T / 4]
     uint32_t* ovf_key;
     float4* ovf_val;
     uint32_t index_bits, slot_cap;
@@ -68,10 +68,10 @@ __device__ __forceinline__ uint32_t ranktab_index(const RankTab& T, uint32_t key
     return ((k * 0x9E3779B1u) >> 12) & (T.index_bits - 1);
 }
 
-// The pairs of the pivots of one group, spread over the threads of the block: thread i holds pairs i and
-// i + nthreads of every pivot (rows with more pairs read the rest when the table is built). Loaded ahead of
+// The pairs of the pivots of one group, spread over the threads of the block: thread i holds pair i of every
+// pivot (rows with more pairs than the block has threads read the rest when the table is built). Loaded ahead of
 // time, while the previous group is still being probed, so that a build does not wait for memory.
-constexpr int RT_PV = 2;
+constexpr int RT_PV = 1;
 struct PivotRegs {
     uint2 kv[RT_T][RT_PV]; // raw pairs
 };
@@ -155,12 +155,11 @@ __device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivo
             before += __popc(T.word[w].x);
         }
     }
-    for (uint32_t s = tid; s < total; s += nthreads) {
-        T.vals[s] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (!NARROW) T.keys[s] = EMPTY;
-    }
+    for (uint32_t s = tid; s < total * (RT_T / 4); s += nthreads) T.vals[s] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (!NARROW) {
-        for (uint32_t s = tid; s < RT_OVF; s += nthreads) { T.ovf_key[s] = EMPTY; T.ovf_val[s] = make_float4(0.f, 0.f, 0.f, 0.f); }
+        for (uint32_t s = tid; s < total; s += nthreads) T.keys[s] = EMPTY;
+        for (uint32_t s = tid; s < RT_OVF; s += nthreads) T.ovf_key[s] = EMPTY;
+        for (uint32_t s = tid; s < RT_OVF * (RT_T / 4); s += nthreads) T.ovf_val[s] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     __syncthreads();
     // 3. values (and keys)
@@ -169,11 +168,11 @@ __device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivo
         const uint2 w = T.word[idx >> 5];
         const uint32_t slot = w.y + __popc(w.x & ((1u << (idx & 31)) - 1u));
         if (NARROW) {
-            reinterpret_cast<uint32_t*>(&T.vals[slot])[t] = kv.y;
+            reinterpret_cast<uint32_t*>(T.vals)[slot * RT_T + t] = kv.y;
         } else {
             const uint32_t old = atomicCAS(&T.keys[slot], EMPTY, kv.x);
             if (old == EMPTY || old == kv.x) {
-                reinterpret_cast<uint32_t*>(&T.vals[slot])[t] = kv.y;
+                reinterpret_cast<uint32_t*>(T.vals)[slot * RT_T + t] = kv.y;
             } else { // another term of the group sits on this bit
                 uint32_t at = EMPTY;
                 for (uint32_t s = 0; s < RT_OVF; s++) {
@@ -181,7 +180,7 @@ __device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivo
                     if (o == EMPTY) atomicAdd(&scan[16], 1u);
                     if (o == EMPTY || o == kv.x) { at = s; break; }
                 }
-                if (at != EMPTY) reinterpret_cast<uint32_t*>(&T.ovf_val[at])[t] = kv.y;
+                if (at != EMPTY) reinterpret_cast<uint32_t*>(T.ovf_val)[at * RT_T + t] = kv.y;
                 else atomicAdd(&scan[16], RT_OVF + 1u);
             }
         }
@@ -274,23 +273,26 @@ __device__ __forceinline__ void rt_row_load(RtRow<NARROW>& r, const Pairs& sp, i
     }
 }
 
-// NB streamed rows against the table at once: acc[r][0..3] += per-pivot sums of this lane's pairs of row r.
+// NB streamed rows against the table at once: acc[r][0..7] += per-pivot sums of this lane's pairs of row r.
 // All bitmap reads of the batch are issued before the first value read, all value reads before the first
 // multiply: the batch costs two LDS round trips whatever NB is. shape[r] = nnz | ns << 16 of row r (wave-uniform;
 // 0: the row is not there); tail(r) gives the Pairs of row r for the pairs beyond the register window.
 template <bool NARROW, int NB, typename TailFn>
 __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow<NARROW> (&rows)[NB], const uint32_t (&shape)[NB], TailFn tail,
                                                    uint32_t n_ovf, float (&acc)[NB][RT_T], int lane) {
+    auto add8 = [&](int r, float m, const float4& lo, const float4& hi) {
+        acc[r][0] = fmaf(m, lo.x, acc[r][0]);
+        acc[r][1] = fmaf(m, lo.y, acc[r][1]);
+        acc[r][2] = fmaf(m, lo.z, acc[r][2]);
+        acc[r][3] = fmaf(m, lo.w, acc[r][3]);
+        acc[r][4] = fmaf(m, hi.x, acc[r][4]);
+        acc[r][5] = fmaf(m, hi.y, acc[r][5]);
+        acc[r][6] = fmaf(m, hi.z, acc[r][6]);
+        acc[r][7] = fmaf(m, hi.w, acc[r][7]);
+    };
     auto overflow = [&](int r, uint32_t key, uint32_t val_bits, bool in) {
         for (uint32_t o = 0; o < n_ovf; o++) { // wave-uniform count, zero for narrow corpora
-            if (in && T.ovf_key[o] == key) {
-                const float4 v = T.ovf_val[o];
-                const float val = __uint_as_float(val_bits);
-                acc[r][0] = fmaf(val, v.x, acc[r][0]);
-                acc[r][1] = fmaf(val, v.y, acc[r][1]);
-                acc[r][2] = fmaf(val, v.z, acc[r][2]);
-                acc[r][3] = fmaf(val, v.w, acc[r][3]);
-            }
+            if (in && T.ovf_key[o] == key) add8(r, __uint_as_float(val_bits), T.ovf_val[2 * o], T.ovf_val[2 * o + 1]);
         }
     };
     uint32_t idx[NB][RT_CHUNKS];
@@ -309,7 +311,7 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
 #pragma unroll
     for (int r = 0; r < NB; r++) asm volatile("" : "+v"(w[r][0].x), "+v"(w[r][1].x), "+v"(w[r][2].x));
     RankProbe p[NB][RT_CHUNKS];
-    float4 v[NB][RT_CHUNKS];
+    float4 lo[NB][RT_CHUNKS], hi[NB][RT_CHUNKS];
     bool ok[NB][RT_CHUNKS];
 #pragma unroll
     for (int r = 0; r < NB; r++) {
@@ -318,24 +320,19 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
         for (int c = 0; c < RT_CHUNKS; c++) {
             const bool in = (uint32_t)(c * WAVE + lane) < nnz;
             p[r][c] = ranktab_locate<NARROW>(T, w[r][c], idx[r][c], rows[r].v[c], in);
-            v[r][c] = T.vals[p[r][c].slot];
+            lo[r][c] = T.vals[2 * p[r][c].slot];
+            hi[r][c] = T.vals[2 * p[r][c].slot + 1];
             ok[r][c] = true;
             if (!NARROW) ok[r][c] = p[r][c].mul == 0.f || T.keys[p[r][c].slot] == rows[r].key(c);
         }
     }
 #pragma unroll
-    for (int r = 0; r < NB; r++) asm volatile("" : "+v"(v[r][0].x), "+v"(v[r][1].x), "+v"(v[r][2].x));
+    for (int r = 0; r < NB; r++) asm volatile("" : "+v"(lo[r][0].x), "+v"(lo[r][1].x), "+v"(lo[r][2].x), "+v"(hi[r][0].x), "+v"(hi[r][1].x), "+v"(hi[r][2].x));
 #pragma unroll
     for (int r = 0; r < NB; r++) {
         const uint32_t nnz = shape[r] & 0xFFFFu;
 #pragma unroll
-        for (int c = 0; c < RT_CHUNKS; c++) {
-            const float m = ok[r][c] ? p[r][c].mul : 0.f;
-            acc[r][0] = fmaf(m, v[r][c].x, acc[r][0]);
-            acc[r][1] = fmaf(m, v[r][c].y, acc[r][1]);
-            acc[r][2] = fmaf(m, v[r][c].z, acc[r][2]);
-            acc[r][3] = fmaf(m, v[r][c].w, acc[r][3]);
-        }
+        for (int c = 0; c < RT_CHUNKS; c++) add8(r, ok[r][c] ? p[r][c].mul : 0.f, lo[r][c], hi[r][c]);
         if (!NARROW && n_ovf) {
 #pragma unroll
             for (int c = 0; c < RT_CHUNKS; c++) overflow(r, rows[r].key(c), rows[r].v[c], (uint32_t)(c * WAVE + lane) < nnz && !ok[r][c]);
@@ -354,57 +351,48 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
                 const uint32_t ix = ranktab_index<NARROW>(T, kv.x, NARROW ? j >= ns : (int)kv.x < 0);
                 const uint2 ww = T.word[in ? ix >> 5 : 0u];
                 const RankProbe q = ranktab_locate<NARROW>(T, ww, ix, kv.y, in);
-                const float4 vv = T.vals[q.slot];
+                const float4 vl = T.vals[2 * q.slot], vh = T.vals[2 * q.slot + 1];
                 bool good = true;
                 if (!NARROW) good = q.mul == 0.f || T.keys[q.slot] == kv.x;
-                const float m = good ? q.mul : 0.f;
-                acc[r][0] = fmaf(m, vv.x, acc[r][0]);
-                acc[r][1] = fmaf(m, vv.y, acc[r][1]);
-                acc[r][2] = fmaf(m, vv.z, acc[r][2]);
-                acc[r][3] = fmaf(m, vv.w, acc[r][3]);
+                add8(r, good ? q.mul : 0.f, vl, vh);
                 if (!NARROW && n_ovf) overflow(r, kv.x, kv.y, in && !good);
             }
         }
     }
 }
 
-// The wave totals of NB (2 or 4) streamed rows x 4 pivots from the per-lane accumulators of ranktab_probe_rows, with
-// NB - 1 + (NB == 2) cross-row exchanges for all of them: inside each 16-lane row the four pivot sums of a streamed
-// row are reduced as in wave_sum4_dpp (lane l keeps pivot t(l) = 2 * (l & 1) + ((l >> 1) & 1)); then the four
-// 16-lane rows of the wave share out the streamed rows between them. Returns the total of (*r_out, *t_out).
-template <int NB>
-__device__ __forceinline__ float wave_sum_rows(const float (&acc)[NB][RT_T], int lane, uint32_t* t_out, uint32_t* r_out) {
-    static_assert(NB == 2 || NB == 4, "two or four streamed rows");
-    float z[NB];
+// The wave totals of 2 streamed rows x 8 pivots from the per-lane accumulators of ranktab_probe_rows<., 2>. The two
+// halves of the pivots (0-3, 4-7) of each row are reduced inside every 16-lane row of the wave like four sums at once
+// (two exchange-and-add steps inside each quad leave lane l with pivot t(l) = 2 * (l & 1) + ((l >> 1) & 1) of its half,
+// then two rotations inside the 16 lanes); the four 16-lane rows of the wave then share out the four (streamed row,
+// half) combinations between them with three cross-row exchanges. Returns the total of streamed row *r_out, pivot *t_out.
+__device__ __forceinline__ float wave_sum_2x8(const float (&acc)[2][RT_T], int lane, uint32_t* t_out, uint32_t* r_out) {
+    float z[4]; // (row 0, low half), (row 0, high half), (row 1, low), (row 1, high)
     const bool odd = lane & 1, hi = lane & 2;
 #pragma unroll
-    for (int r = 0; r < NB; r++) {
-        const float keep0 = odd ? acc[r][2] : acc[r][0], keep1 = odd ? acc[r][3] : acc[r][1];
-        const float give0 = odd ? acc[r][0] : acc[r][2], give1 = odd ? acc[r][1] : acc[r][3];
+    for (int k = 0; k < 4; k++) {
+        const float* a = &acc[k >> 1][4 * (k & 1)];
+        const float keep0 = odd ? a[2] : a[0], keep1 = odd ? a[3] : a[1];
+        const float give0 = odd ? a[0] : a[2], give1 = odd ? a[1] : a[3];
         const float x0 = keep0 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give0), 0xB1, 0xF, 0xF, false));
         const float x1 = keep1 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give1), 0xB1, 0xF, 0xF, false));
         const float keep = hi ? x1 : x0, give = hi ? x0 : x1;
         float y = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give), 0x4E, 0xF, 0xF, false));
         y += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, y), 0x124, 0xF, 0xF, false)); // row_ror:4
         y += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, y), 0x128, 0xF, 0xF, false)); // row_ror:8
-        z[r] = y;
+        z[k] = y;
     }
     const bool q0 = lane & 16, q1 = lane & 32;
-    *t_out = 2u * (lane & 1) + ((lane >> 1) & 1);
-    if (NB == 4) {
-        const float keepA0 = q0 ? z[2] : z[0], giveA0 = q0 ? z[0] : z[2];
-        const float keepA1 = q0 ? z[NB - 1] : z[1], giveA1 = q0 ? z[1] : z[NB - 1];
-        const float xa = keepA0 + __shfl_xor(giveA0, 16, WAVE);
-        const float xb = keepA1 + __shfl_xor(giveA1, 16, WAVE);
-        const float keepB = q1 ? xb : xa, giveB = q1 ? xa : xb;
-        *r_out = 2u * ((lane >> 4) & 1) + ((lane >> 5) & 1);
-        return keepB + __shfl_xor(giveB, 32, WAVE);
-    }
-    const float keepA = q0 ? z[1] : z[0], giveA = q0 ? z[0] : z[1];
-    float x = keepA + __shfl_xor(giveA, 16, WAVE);
-    x += __shfl_xor(x, 32, WAVE);
-    *r_out = (lane >> 4) & 1;
-    return x;
+    const float keepA0 = q0 ? z[2] : z[0], giveA0 = q0 ? z[0] : z[2];
+    const float keepA1 = q0 ? z[3] : z[1], giveA1 = q0 ? z[1] : z[3];
+    const float xa = keepA0 + __shfl_xor(giveA0, 16, WAVE);
+    const float xb = keepA1 + __shfl_xor(giveA1, 16, WAVE);
+    const float keepB = q1 ? xb : xa, giveB = q1 ? xa : xb;
+    // 16-lane row q of the wave now holds combination k(q) = 2 * (q & 1) + (q >> 1): streamed row k >> 1, half k & 1
+    const uint32_t k = 2u * ((lane >> 4) & 1) + ((lane >> 5) & 1);
+    *r_out = k >> 1;
+    *t_out = 4u * (k & 1) + 2u * (lane & 1) + ((lane >> 1) & 1);
+    return keepB + __shfl_xor(giveB, 32, WAVE);
 }
 
 #endif // __HIPCC__

@@ -6,7 +6,7 @@
 // are its COLUMNS (up to 128), every row of the tile is gathered once and meets every column:
 //   dense part   32 x 128 x 1024 contraction on the matrix cores (fp32 MFMA 32x32x2; eight waves: four 32-column
 //                blocks x two halves of the dimensions)
-//   sparse part  four picker rows at a time in an LDS rank table that the column rows probe (apoe_ranktab.h); a
+//   sparse part  eight picker rows at a time in an LDS rank table that the column rows probe (apoe_ranktab.h); a
 //                wave keeps the pairs of its sixteen columns in registers, so a row is read from memory once per tile
 //   insertion    a pair closer than the row's last list entry (and not in that list) is offered to the row node
 //                with a 64-bit atomicMin on slot hash(id) of its proposal row: (distance, id), the smallest wins;
@@ -33,7 +33,7 @@ constexpr int JT_STRIDE = JT_COLS + 1;
 constexpr int JT_SEEN = 512; // slots of the id set that removes repeated columns
 constexpr uint32_t JOIN_K = 64;
 constexpr int JOIN_PICKS = 4; // index.cu:157,171-181
-constexpr int JT_BATCH = 4;   // column rows a wave probes together
+constexpr int JT_BATCH = 2;   // column rows a wave probes together
 constexpr int JT_OWN = JT_COLS / (JT_THREADS / WAVE); // columns of a tile that one wave owns: their pairs stay in its registers
 
 __device__ __forceinline__ uint32_t prop_slot(uint32_t id, uint32_t P) { return (uint32_t)(mix64(id) >> 40) & (P - 1); }
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
             if (active && part == 1) store(true);
         }
         __syncthreads();
-        // sparse part: groups of four rows in the rank table, every column probes it once per group. The pairs of a
+        // sparse part: groups of eight rows in the rank table, every column probes it once per group. The pairs of a
         // group's rows are requested while the group before it is probed; the pairs of a wave's columns stay in its
         // registers for the whole tile: a build and the probes find their operands there.
         auto row_pairs = [&](uint32_t i) { Pairs p = gram_row(a.C, rowptr, rownnz, i); p.narrow = NARROW ? 1u : 0u; return p; };
@@ -309,9 +309,9 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
                     }
                     ranktab_probe_rows<NARROW, JT_BATCH>(T, rows, shape, [&](int k) { return col_pairs(b0 + k * NW); }, n_ovf, acc, lane);
                     uint32_t t, r;
-                    const float z = wave_sum_rows<JT_BATCH>(acc, lane, &t, &r);
+                    const float z = wave_sum_2x8(acc, lane, &t, &r);
                     const uint32_t b = b0 + r * NW;
-                    if ((lane & 15) < RT_T && t < nt && b < M) G[(a0 + t) * JT_STRIDE + b] += z;
+                    if ((lane & 15) < 4 && t < nt && b < M) G[(a0 + t) * JT_STRIDE + b] += z;
                 }
                 __builtin_amdgcn_sched_barrier(0); // one batch at a time: the scheduler must not pile up the reads of all of them
             }
@@ -407,7 +407,7 @@ static void join_table_shape(const apoe_corpus* c, uint32_t* index_bits, uint32_
     *span = next_pow2(std::max(c->max_term + 1, 1024u));
     *index_bits = c->narrow ? 2 * *span : 65536u;
     const uint32_t want = RT_T * (c->max_nnz_s + c->max_nnz_b);
-    *slot_cap = std::min<uint32_t>(std::max<uint32_t>((want + 63) & ~63u, 256u), 2560u);
+    *slot_cap = std::min<uint32_t>(std::max<uint32_t>((want + 63) & ~63u, 256u), 2304u);
 }
 
 int join_alloc(apoe_knn* g) {
@@ -439,7 +439,7 @@ int launch_nnd_join_iterate(apoe_knn* g) {
     uint32_t index_bits, slot_cap, span;
     join_table_shape(g->corpus, &index_bits, &slot_cap, &span);
     const JoinLds L(index_bits, slot_cap, g->corpus->narrow);
-    APOE_REQUIRE(L.total <= 96 * 1024, "the local-join tile needs %u bytes of LDS", L.total);
+    APOE_REQUIRE(L.total <= 150 * 1024, "the local-join tile needs %u bytes of LDS", L.total);
 
     APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), st)); // [0] inserted; [2], [3] accumulate over the build
     fill_u32_kernel2<<<1024, 256, 0, st>>>(g->pick_cnt.p, (uint64_t)n + 1, 0u);
