@@ -402,13 +402,15 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
         }
     }
     // hybrid Gram matrix of the m rows
-    // waves 0-3 take the first half of the dimensions of the four tiles, waves 4-7 (if there) the second half
+    // waves 0-3 take the first half of the dimensions of the tiles, waves 4-7 (if there) the second half. Only the
+    // upper triangle of G is used (the sparse part is added there and the lower triangle is mirrored from it at the
+    // end), so the lower left tile is not computed: its two row blocks would be read a third time for nothing.
     {
         constexpr int NWAVES = NT / WAVE, PARTS = NWAVES >= 8 ? 2 : 1, BLOCKS = DIM / 8;
         const int part = wave >> 2;
         bool active = false;
         floatx16 acc;
-        if (m > 0 && part < PARTS) acc = gram_dense_tile(C, nb_id, m, wave & 3, lane, part * (BLOCKS / PARTS), (part + 1) * (BLOCKS / PARTS), active);
+        if (m > 0 && part < PARTS && (wave & 3) != 2) acc = gram_dense_tile(C, nb_id, m, wave & 3, lane, part * (BLOCKS / PARTS), (part + 1) * (BLOCKS / PARTS), active);
         if (active && part == 0) gram_dense_store(G, wave & 3, lane, acc, dense_mul, false);
         __syncthreads();
         if (active && part == 1) gram_dense_store(G, wave & 3, lane, acc, dense_mul, true);
