@@ -160,11 +160,17 @@ def main():
 
     # ---- pool sweep: recall and one launch each ----
     sweep = []
+
+    def iter_cap(c):
+        # the reference stops a walk after 1000 expansions (query.cu:7 MAX_ITER), fewer than a pool above 512 has entries:
+        # the larger pools of the sweep get four expansions per entry so that the pool, not the cap, ends the walk
+        return 0 if c <= 512 else 4 * c
+
     for cands in [int(c) for c in args.cands.split(",")]:
-        apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant)
-        ids, dist, st = apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant)
+        apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant, max_iter=iter_cap(cands))
+        ids, dist, st = apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant, max_iter=iter_cap(cands))
         rec = recall_at_k(ids[:nq_truth], truth, 10)
-        sweep.append(dict(cands=cands, recall=rec, ms=st.kernel_ms, qps=args.queries / (st.kernel_ms / 1e3),
+        sweep.append(dict(cands=cands, max_iter=iter_cap(cands) or 1000, recall=rec, ms=st.kernel_ms, qps=args.queries / (st.kernel_ms / 1e3),
                           gbs=st.algo_bytes / (st.kernel_ms / 1e3) / 1e9))
         log(f"[bench] cands={cands}: recall@10={rec:.4f} kernel {st.kernel_ms:.2f} ms -> {sweep[-1]['qps']:.0f} QPS, "
             f"{sweep[-1]['gbs']:.0f} GB/s algorithmic, {st.evaluations / args.queries:.0f} evals/query, "
@@ -179,13 +185,13 @@ def main():
     out_ids = torch.empty((args.queries, cands), dtype=torch.int32, device=dev)
     out_dist = torch.empty((args.queries, cands), dtype=torch.float32, device=dev)
     for _ in range(args.warmup):
-        apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant, out_ids=out_ids, out_dist=out_dist)
+        apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant, out_ids=out_ids, out_dist=out_dist, max_iter=iter_cap(cands))
     torch.cuda.synchronize()
     ctx.synchronize()
     kernel_ms, algo_bytes = [], 0
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        _, _, st = apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant, out_ids=out_ids, out_dist=out_dist)
+        _, _, st = apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant, out_ids=out_ids, out_dist=out_dist, max_iter=iter_cap(cands))
         kernel_ms.append(st.kernel_ms)
         algo_bytes = st.algo_bytes
     ctx.synchronize()
@@ -197,7 +203,7 @@ def main():
     # the same launch with the dense row of every candidate read (no bound test): same results, more bytes
     full_ms, full_bytes = [], 0
     for i in range(args.warmup + args.steps):
-        _, _, stf = apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant | 0x100, out_ids=out_ids, out_dist=out_dist)
+        _, _, stf = apoe.search(ctx, gc, gq, graph, w3, cands, variant=args.variant | 0x100, out_ids=out_ids, out_dist=out_dist, max_iter=iter_cap(cands))
         if i >= args.warmup:
             full_ms.append(stf.kernel_ms)
             full_bytes = stf.algo_bytes
@@ -338,7 +344,7 @@ def main():
         rows, entry = graph.download()
         threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
         t0 = time.perf_counter()
-        oid, odist, _ = O.search(C_, Q_, rows, entry, w3, cands, threads=threads)
+        oid, odist, _ = O.search(C_, Q_, rows, entry, w3, cands, max_iter=iter_cap(cands) or 1000, threads=threads)
         cpu_s = time.perf_counter() - t0
         agree = float(np.mean(oid[:, :10] == out_ids[:ncpu, :10].cpu().numpy().view(np.uint32)))
         cpu = dict(value=ncpu / cpu_s, unit="queries/s", cores=threads, kind="port",
