@@ -90,38 +90,24 @@ __device__ __forceinline__ void ranktab_pivots_load(PivotRegs& r, PivotFn pivot,
     }
 }
 
-// Builds the table of pivots [0, nt) (nt <= RT_T); pivot(t) gives the Pairs of pivot t, `regs` its first pairs
-// (ranktab_pivots_load). All threads of the block call it (the block size is a multiple of 64, at most 1024);
-// `scan` is LDS scratch of 20 words. Returns the number of distinct terms, or EMPTY if they exceed the slot
-// capacity or the overflow list (the table is then unusable: the caller retries with fewer pivots). Ends with
-// a barrier: the table is ready on return.
-template <bool NARROW, typename PivotFn>
-__device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivot, const PivotRegs& regs, uint32_t nt, uint32_t* scan, int tid,
-                                                  int nthreads) {
+// Builds the table from the pairs that `each` hands out: each(f) calls f(raw pair, is BM25, pivot index t < RT_T)
+// for every pair of the group that this thread is responsible for, and must hand out the same pairs every time it is
+// called (it is called twice: bits, then values). All threads of the block call this (the block size is a multiple
+// of 64, at most 1024); `scan` is LDS scratch of 20 words. Returns the number of distinct terms, or EMPTY if they
+// exceed the slot capacity or the overflow list (the table is then unusable: the caller retries with fewer pivots).
+// Ends with a barrier: the table is ready on return.
+template <bool NARROW, typename EachFn>
+__device__ __forceinline__ uint32_t ranktab_build_each(const RankTab& T, EachFn each, uint32_t* scan, int tid, int nthreads) {
     const uint32_t W = T.index_bits / 32;
     const int lane = tid & (WAVE - 1), wave = tid / WAVE, nwaves = nthreads / WAVE;
     for (uint32_t w = tid; w < W; w += nthreads) T.word[w] = make_uint2(0u, 0u);
     if (tid == 0) scan[16] = 0; // overflow count
     __syncthreads();
     // 1. bits
-#pragma unroll
-    for (int t = 0; t < RT_T; t++) {
-        if ((uint32_t)t < nt) {
-            const Pairs sp = pivot(t);
-#pragma unroll
-            for (int k = 0; k < RT_PV; k++) {
-                const uint32_t j = tid + k * nthreads;
-                if (j < sp.nnz) {
-                    const uint32_t idx = ranktab_index<NARROW>(T, regs.kv[t][k].x, j >= sp.ns);
-                    atomicOr(&T.word[idx >> 5].x, 1u << (idx & 31));
-                }
-            }
-            for (uint32_t j = tid + RT_PV * nthreads; j < sp.nnz; j += nthreads) {
-                const uint32_t idx = ranktab_index<NARROW>(T, sp.raw(j).x, j >= sp.ns);
-                atomicOr(&T.word[idx >> 5].x, 1u << (idx & 31));
-            }
-        }
-    }
+    each([&](uint2 kv, bool bm25, int) {
+        const uint32_t idx = ranktab_index<NARROW>(T, kv.x, bm25);
+        atomicOr(&T.word[idx >> 5].x, 1u << (idx & 31));
+    });
     __syncthreads();
     // 2. running counts: thread i owns the words [i * per, (i + 1) * per)
     const uint32_t per = (W + nthreads - 1) / nthreads;
@@ -163,8 +149,8 @@ __device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivo
     }
     __syncthreads();
     // 3. values (and keys)
-    auto put = [&](uint2 kv, uint32_t j, const Pairs& sp, int t) {
-        const uint32_t idx = ranktab_index<NARROW>(T, kv.x, j >= sp.ns);
+    each([&](uint2 kv, bool bm25, int t) {
+        const uint32_t idx = ranktab_index<NARROW>(T, kv.x, bm25);
         const uint2 w = T.word[idx >> 5];
         const uint32_t slot = w.y + __popc(w.x & ((1u << (idx & 31)) - 1u));
         if (NARROW) {
@@ -184,22 +170,35 @@ __device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivo
                 else atomicAdd(&scan[16], RT_OVF + 1u);
             }
         }
-    };
-#pragma unroll
-    for (int t = 0; t < RT_T; t++) {
-        if ((uint32_t)t < nt) {
-            const Pairs sp = pivot(t);
-#pragma unroll
-            for (int k = 0; k < RT_PV; k++) {
-                const uint32_t j = tid + k * nthreads;
-                if (j < sp.nnz) put(regs.kv[t][k], j, sp, t);
-            }
-            for (uint32_t j = tid + RT_PV * nthreads; j < sp.nnz; j += nthreads) put(sp.raw(j), j, sp, t);
-        }
-    }
+    });
     __syncthreads();
-    if (!NARROW && scan[16] > RT_OVF) return EMPTY;
+    if (!NARROW) { // every thread reads the count before any thread can start the next build, which clears it
+        const uint32_t ov = scan[16];
+        __syncthreads();
+        if (ov > RT_OVF) return EMPTY;
+    }
     return total;
+}
+
+// The table of pivots [0, nt) (nt <= RT_T) whose pairs are spread over the threads of the block: pivot(t) gives the
+// Pairs of pivot t, `regs` its first pairs (ranktab_pivots_load).
+template <bool NARROW, typename PivotFn>
+__device__ __forceinline__ uint32_t ranktab_build(const RankTab& T, PivotFn pivot, const PivotRegs& regs, uint32_t nt, uint32_t* scan, int tid,
+                                                  int nthreads) {
+    return ranktab_build_each<NARROW>(T, [&](auto f) {
+#pragma unroll
+        for (int t = 0; t < RT_T; t++) {
+            if ((uint32_t)t < nt) {
+                const Pairs sp = pivot(t);
+#pragma unroll
+                for (int k = 0; k < RT_PV; k++) {
+                    const uint32_t j = tid + k * nthreads;
+                    if (j < sp.nnz) f(regs.kv[t][k], j >= sp.ns, t);
+                }
+                for (uint32_t j = tid + RT_PV * nthreads; j < sp.nnz; j += nthreads) f(sp.raw(j), j >= sp.ns, t);
+            }
+        }
+    }, scan, tid, nthreads);
 }
 
 // One pair against the table: acc[t] += value * (pivot t's value of the term). `in` = the lane holds a pair.
@@ -237,33 +236,46 @@ __device__ __forceinline__ float wave_sum4_dpp(const float acc[4], int lane, uin
     return z;
 }
 
-constexpr int RT_CHUNKS = 3; // 64-pair chunks of a streamed row kept in registers (192 pairs); longer rows read the rest when they are probed
+constexpr int RT_CHUNKS = 4; // 64-pair chunks of a streamed row kept in registers (256 pairs); longer rows read the rest when they are probed
 
-// Raw pairs of a streamed row in registers: lane l holds pairs l, l + 64, l + 128. Narrow keys are 16 bits wide:
-// the first two share a register.
+// Raw pairs of a streamed row in registers: lane l holds pairs l, l + 64, l + 128, l + 192. Narrow keys are 16 bits
+// wide: two share a register.
 template <bool NARROW>
 struct RtRow;
 template <>
 struct RtRow<true> {
-    uint32_t v[RT_CHUNKS], k01, k2;
+    uint32_t v[RT_CHUNKS], k2[RT_CHUNKS / 2];
     // tells the compiler that the keys may have changed: what is derived from them (bit index, masks) is then computed
     // where it is used instead of once for all rows ahead of a loop, where it would occupy registers for the whole loop
-    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(k01), "+v"(k2)); }
-    __device__ __forceinline__ uint32_t key(int c) const { return c == 0 ? (k01 & 0xFFFFu) : c == 1 ? (k01 >> 16) : k2; }
+    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(k2[0]), "+v"(k2[1])); }
+    __device__ __forceinline__ uint32_t key(int c) const { return (c & 1) ? (k2[c >> 1] >> 16) : (k2[c >> 1] & 0xFFFFu); }
     __device__ __forceinline__ void set(int c, uint2 kv) {
         v[c] = kv.y;
-        if (c == 0) k01 = kv.x;
-        else if (c == 1) k01 |= kv.x << 16;
-        else k2 = kv.x;
+        if (c & 1) k2[c >> 1] |= kv.x << 16;
+        else k2[c >> 1] = kv.x;
     }
 };
 template <>
 struct RtRow<false> {
     uint32_t v[RT_CHUNKS], k[RT_CHUNKS];
-    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(k[0]), "+v"(k[1]), "+v"(k[2])); }
+    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3])); }
     __device__ __forceinline__ uint32_t key(int c) const { return k[c]; }
     __device__ __forceinline__ void set(int c, uint2 kv) { v[c] = kv.y; k[c] = kv.x; }
 };
+// dst = take ? src : dst, member by member (a wave-uniform choice between rows that stay in registers)
+__device__ __forceinline__ void rt_row_select(RtRow<true>& dst, const RtRow<true>& src, bool take) {
+#pragma unroll
+    for (int c = 0; c < RT_CHUNKS; c++) dst.v[c] = take ? src.v[c] : dst.v[c];
+#pragma unroll
+    for (int c = 0; c < RT_CHUNKS / 2; c++) dst.k2[c] = take ? src.k2[c] : dst.k2[c];
+}
+__device__ __forceinline__ void rt_row_select(RtRow<false>& dst, const RtRow<false>& src, bool take) {
+#pragma unroll
+    for (int c = 0; c < RT_CHUNKS; c++) {
+        dst.v[c] = take ? src.v[c] : dst.v[c];
+        dst.k[c] = take ? src.k[c] : dst.k[c];
+    }
+}
 template <bool NARROW>
 __device__ __forceinline__ void rt_row_load(RtRow<NARROW>& r, const Pairs& sp, int lane) {
 #pragma unroll
@@ -273,13 +285,33 @@ __device__ __forceinline__ void rt_row_load(RtRow<NARROW>& r, const Pairs& sp, i
     }
 }
 
+// The table of a group whose pivots are held one per wave, in registers: this wave's row `pr` (shape = nnz | ns << 16)
+// becomes pivot t when `mine` is set (wave-uniform); `tail` = the Pairs of that row, read for the pairs beyond the
+// register window only. Everything else as ranktab_build_each.
+template <bool NARROW>
+__device__ __forceinline__ uint32_t ranktab_build_rows(const RankTab& T, const RtRow<NARROW>& pr, uint32_t shape, bool mine, int t, const Pairs& tail,
+                                                       uint32_t* scan, int tid, int nthreads) {
+    const int lane = tid & (WAVE - 1);
+    const uint32_t nnz = mine ? shape & 0xFFFFu : 0u, ns = shape >> 16;
+    return ranktab_build_each<NARROW>(T, [&](auto f) {
+#pragma unroll
+        for (int c = 0; c < RT_CHUNKS; c++) {
+            const uint32_t j = c * WAVE + lane;
+            if (j < nnz) f(make_uint2(pr.key(c), pr.v[c]), NARROW ? j >= ns : false, t);
+        }
+        for (uint32_t j = RT_CHUNKS * WAVE + lane; j < nnz; j += WAVE) f(tail.raw(j), j >= ns, t);
+    }, scan, tid, nthreads);
+}
+
 // NB streamed rows against the table at once: acc[r][0..7] += per-pivot sums of this lane's pairs of row r.
-// All bitmap reads of the batch are issued before the first value read, all value reads before the first
-// multiply: the batch costs two LDS round trips whatever NB is. shape[r] = nnz | ns << 16 of row r (wave-uniform;
+// All bitmap reads of the batch are issued before the first value read; the value reads follow in two halves (chunks
+// 0-1, then 2-3 of every row), each issued whole before its multiplies: three LDS round trips per batch whatever NB
+// is, and at most NB x 2 x 8 value registers in flight. shape[r] = nnz | ns << 16 of row r (wave-uniform;
 // 0: the row is not there); tail(r) gives the Pairs of row r for the pairs beyond the register window.
 template <bool NARROW, int NB, typename TailFn>
 __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow<NARROW> (&rows)[NB], const uint32_t (&shape)[NB], TailFn tail,
                                                    uint32_t n_ovf, float (&acc)[NB][RT_T], int lane) {
+    static_assert(RT_CHUNKS % 2 == 0, "the value reads go out in two halves");
     auto add8 = [&](int r, float m, const float4& lo, const float4& hi) {
         acc[r][0] = fmaf(m, lo.x, acc[r][0]);
         acc[r][1] = fmaf(m, lo.y, acc[r][1]);
@@ -295,47 +327,48 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
             if (in && T.ovf_key[o] == key) add8(r, __uint_as_float(val_bits), T.ovf_val[2 * o], T.ovf_val[2 * o + 1]);
         }
     };
-    uint32_t idx[NB][RT_CHUNKS];
+    auto index_of = [&](int r, int c) {
+        const uint32_t key = rows[r].key(c);
+        return ranktab_index<NARROW>(T, key, NARROW ? (uint32_t)(c * WAVE + lane) >= (shape[r] >> 16) : (int)key < 0);
+    };
     uint2 w[NB][RT_CHUNKS];
 #pragma unroll
     for (int r = 0; r < NB; r++) {
-        const uint32_t nnz = shape[r] & 0xFFFFu, ns = shape[r] >> 16;
-#pragma unroll
-        for (int c = 0; c < RT_CHUNKS; c++) {
-            const uint32_t j = c * WAVE + lane;
-            const uint32_t key = rows[r].key(c);
-            idx[r][c] = ranktab_index<NARROW>(T, key, NARROW ? j >= ns : (int)key < 0);
-            w[r][c] = T.word[j < nnz ? idx[r][c] >> 5 : 0u];
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < NB; r++) asm volatile("" : "+v"(w[r][0].x), "+v"(w[r][1].x), "+v"(w[r][2].x));
-    RankProbe p[NB][RT_CHUNKS];
-    float4 lo[NB][RT_CHUNKS], hi[NB][RT_CHUNKS];
-    bool ok[NB][RT_CHUNKS];
-#pragma unroll
-    for (int r = 0; r < NB; r++) {
         const uint32_t nnz = shape[r] & 0xFFFFu;
 #pragma unroll
-        for (int c = 0; c < RT_CHUNKS; c++) {
-            const bool in = (uint32_t)(c * WAVE + lane) < nnz;
-            p[r][c] = ranktab_locate<NARROW>(T, w[r][c], idx[r][c], rows[r].v[c], in);
-            lo[r][c] = T.vals[2 * p[r][c].slot];
-            hi[r][c] = T.vals[2 * p[r][c].slot + 1];
-            ok[r][c] = true;
-            if (!NARROW) ok[r][c] = p[r][c].mul == 0.f || T.keys[p[r][c].slot] == rows[r].key(c);
-        }
+        for (int c = 0; c < RT_CHUNKS; c++) w[r][c] = T.word[(uint32_t)(c * WAVE + lane) < nnz ? index_of(r, c) >> 5 : 0u];
     }
 #pragma unroll
-    for (int r = 0; r < NB; r++) asm volatile("" : "+v"(lo[r][0].x), "+v"(lo[r][1].x), "+v"(lo[r][2].x), "+v"(hi[r][0].x), "+v"(hi[r][1].x), "+v"(hi[r][2].x));
+    for (int r = 0; r < NB; r++) asm volatile("" : "+v"(w[r][0].x), "+v"(w[r][1].x), "+v"(w[r][2].x), "+v"(w[r][3].x));
 #pragma unroll
-    for (int r = 0; r < NB; r++) {
-        const uint32_t nnz = shape[r] & 0xFFFFu;
+    for (int h = 0; h < RT_CHUNKS; h += 2) {
+        RankProbe p[NB][2];
+        float4 lo[NB][2], hi[NB][2];
+        bool ok[NB][2];
 #pragma unroll
-        for (int c = 0; c < RT_CHUNKS; c++) add8(r, ok[r][c] ? p[r][c].mul : 0.f, lo[r][c], hi[r][c]);
-        if (!NARROW && n_ovf) {
+        for (int r = 0; r < NB; r++) {
+            const uint32_t nnz = shape[r] & 0xFFFFu;
 #pragma unroll
-            for (int c = 0; c < RT_CHUNKS; c++) overflow(r, rows[r].key(c), rows[r].v[c], (uint32_t)(c * WAVE + lane) < nnz && !ok[r][c]);
+            for (int c = 0; c < 2; c++) {
+                const bool in = (uint32_t)((h + c) * WAVE + lane) < nnz;
+                p[r][c] = ranktab_locate<NARROW>(T, w[r][h + c], index_of(r, h + c), rows[r].v[h + c], in);
+                lo[r][c] = T.vals[2 * p[r][c].slot];
+                hi[r][c] = T.vals[2 * p[r][c].slot + 1];
+                ok[r][c] = true;
+                if (!NARROW) ok[r][c] = p[r][c].mul == 0.f || T.keys[p[r][c].slot] == rows[r].key(h + c);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < NB; r++) asm volatile("" : "+v"(lo[r][0].x), "+v"(lo[r][1].x), "+v"(hi[r][0].x), "+v"(hi[r][1].x));
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const uint32_t nnz = shape[r] & 0xFFFFu;
+#pragma unroll
+            for (int c = 0; c < 2; c++) add8(r, ok[r][c] ? p[r][c].mul : 0.f, lo[r][c], hi[r][c]);
+            if (!NARROW && n_ovf) {
+#pragma unroll
+                for (int c = 0; c < 2; c++) overflow(r, rows[r].key(h + c), rows[r].v[h + c], (uint32_t)((h + c) * WAVE + lane) < nnz && !ok[r][c]);
+            }
         }
     }
     // rows longer than the register window
@@ -393,6 +426,32 @@ __device__ __forceinline__ float wave_sum_2x8(const float (&acc)[2][RT_T], int l
     *r_out = k >> 1;
     *t_out = 4u * (k & 1) + 2u * (lane & 1) + ((lane >> 1) & 1);
     return keepB + __shfl_xor(giveB, 32, WAVE);
+}
+
+// The wave totals of one streamed row x 8 pivots from the per-lane accumulators of ranktab_probe_rows<., 1>: as
+// wave_sum_2x8 with two (low half, high half) instead of four combinations. Returns the total of pivot *t_out.
+__device__ __forceinline__ float wave_sum_1x8(const float (&acc)[RT_T], int lane, uint32_t* t_out) {
+    float z[2];
+    const bool odd = lane & 1, hi = lane & 2;
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const float* a = &acc[4 * k];
+        const float keep0 = odd ? a[2] : a[0], keep1 = odd ? a[3] : a[1];
+        const float give0 = odd ? a[0] : a[2], give1 = odd ? a[1] : a[3];
+        const float x0 = keep0 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give0), 0xB1, 0xF, 0xF, false));
+        const float x1 = keep1 + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give1), 0xB1, 0xF, 0xF, false));
+        const float keep = hi ? x1 : x0, give = hi ? x0 : x1;
+        float y = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, give), 0x4E, 0xF, 0xF, false));
+        y += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, y), 0x124, 0xF, 0xF, false)); // row_ror:4
+        y += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, y), 0x128, 0xF, 0xF, false)); // row_ror:8
+        z[k] = y;
+    }
+    const bool q0 = lane & 16;
+    const float keep = q0 ? z[1] : z[0], give = q0 ? z[0] : z[1];
+    float x = keep + __shfl_xor(give, 16, WAVE);
+    x += __shfl_xor(x, 32, WAVE);
+    *t_out = 4u * ((lane >> 4) & 1) + 2u * (lane & 1) + ((lane >> 1) & 1);
+    return x;
 }
 
 #endif // __HIPCC__

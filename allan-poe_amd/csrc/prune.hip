@@ -10,6 +10,7 @@
 #include <cmath>
 
 #include "apoe_internal.h"
+#include "apoe_ranktab.h"
 
 namespace apoe {
 
@@ -240,19 +241,26 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
 
 // ---- gather-once form of the prune (K = 64) ----
 
+#ifdef APOE_PRUNE_TIMING
+#define TICK(k) do { if (tid == 0) { const unsigned long long t1_ = wall_clock64(); atomicAdd(&apoe_prune_ticks[k], t1_ - t0_); t0_ = t1_; } } while (0)
+#else
+#define TICK(k)
+#endif
 constexpr int GRAM_THREADS = 512; // 8 waves share one node's tables: more lookups in flight per byte of LDS
 
 struct GramPruneLds {
     uint32_t G, tabs, ovf_cnt, rowptr, rownnz, umap, R, F, idmap, nb_id, nb_dist, nrm, det, order, sel_gi, sel_live, sel_kw, o_fwd, o_det, o_kw, ctl, total;
-    // union_slots != 0: the table region holds one union table (apoe_gram.h) instead of tgroup pivot tables
-    __host__ __device__ GramPruneLds(uint32_t term_slots, uint32_t tgroup, uint32_t umap_slots, uint32_t map_slots, uint32_t words,
-                                     uint32_t union_slots) {
+    // union_slots != 0: the table region holds one union table (apoe_gram.h) instead of tgroup pivot tables;
+    // rank_slots != 0: it holds a rank table (apoe_ranktab.h) of rank_bits index bits instead
+    __host__ __device__ __forceinline__ GramPruneLds(uint32_t term_slots, uint32_t tgroup, uint32_t umap_slots, uint32_t map_slots, uint32_t words,
+                                     uint32_t union_slots, uint32_t rank_bits = 0, uint32_t rank_slots = 0, bool narrow = true) {
         uint32_t o = 0;
         G = o; o += GRAM_ROWS * GRAM_STRIDE * 4;
         o = (o + 15) & ~15u;
-        tabs = o; o += union_slots ? GramUnionLds(union_slots).total : tgroup * (term_slots + GRAM_OVF) * 8;
+        tabs = o; o += rank_slots ? RankTabLds(rank_bits, rank_slots, narrow).total
+                           : union_slots ? GramUnionLds(union_slots).total : tgroup * (term_slots + GRAM_OVF) * 8;
         o = (o + 15) & ~15u;
-        ovf_cnt = o; o += 8 * 4;
+        ovf_cnt = o; o += 24 * 4; // also the scratch of the rank table's running counts
         rowptr = o; o += GRAM_ROWS * 8;
         rownnz = o; o += GRAM_ROWS * 4;
         umap = o; o += umap_slots * 8;
@@ -275,22 +283,99 @@ struct GramPruneLds {
     }
 };
 
+// Sparse part of the Gram matrix with the rows in registers (K = 64, eight waves): wave w owns rows w, w + 8, ...
+// (own[k] = row w + 8k, shape nnz | ns << 16, 0 where the row does not exist), loaded once. The pivots are taken
+// eight at a time, one per wave (group g = rows 8g .. 8g + 7: every wave scatters ITS row own[g] into the rank
+// table, apoe_ranktab.h), and every wave then probes the table with its own rows of index >= 8g, two per batch:
+// no global memory access in the whole phase but for rows longer than the register window. G[p][b] += <p, b>
+// for p < b. A group whose distinct terms exceed the table is done in passes of 4, 2 or 1 pivots.
+constexpr int GR_OWN = GRAM_ROWS / 8;
+template <bool NARROW>
+__device__ __forceinline__ void gram_sparse_rank(const CorpusView& C, uint32_t m, float* G, const RankTab& T, uint32_t* scan,
+                                                 const unsigned long long* rowptr, const uint32_t* rownnz, const RtRow<NARROW> (&own)[GR_OWN],
+                                                 const uint32_t (&own_shape)[GR_OWN], uint32_t* fail, int tid, int nthreads) {
+    const int wave = (int)uniform(tid / WAVE), lane = tid & (WAVE - 1);
+    auto row_pairs = [&](uint32_t i) { Pairs p = gram_row(C, rowptr, rownnz, i); p.narrow = NARROW ? 1u : 0u; return p; };
+    const uint32_t ng = m >= 2 ? (m - 2) / 8 + 1 : 0; // the last row is never a pivot
+    uint32_t shape_lanes = 0; // lane k holds own_shape[k]: a wave-uniform pick by index without an indexed array
+#pragma unroll
+    for (int k = 0; k < GR_OWN; k++) shape_lanes = lane == k ? own_shape[k] : shape_lanes;
+#ifdef APOE_PRUNE_TIMING
+    unsigned long long g0_ = wall_clock64();
+#endif
+    for (uint32_t g = 0; g < ng; g++) {
+        // this wave's pivot of the group: own[g], picked with wave-uniform selects so that own[] stays in registers
+        RtRow<NARROW> pr = own[0];
+#pragma unroll
+        for (int k = 1; k < GR_OWN; k++) rt_row_select(pr, own[k], g == (uint32_t)k);
+        const uint32_t pshape = (uint32_t)__builtin_amdgcn_readlane((int)shape_lanes, (int)g);
+        const uint32_t prow = 8 * g + wave;
+        const Pairs ptail = row_pairs(min(prow, m - 1));
+        uint32_t lo = 0, cnt = 8;
+        while (lo < 8) {
+            const bool mine = (uint32_t)wave >= lo && (uint32_t)wave < lo + cnt && prow < m;
+            const uint32_t built = ranktab_build_rows<NARROW>(T, pr, pshape, mine, wave - (int)lo, ptail, scan, tid, nthreads);
+            GTICK(8);
+            if (built == EMPTY) {
+                if (cnt == 1) { // one row alone does not fit: the caller falls back
+                    if (tid == 0) *fail = 1;
+                    lo += 1;
+                } else {
+                    cnt >>= 1;
+                }
+                continue;
+            }
+            const uint32_t n_ovf = NARROW ? 0u : uniform(min(scan[16], (uint32_t)RT_OVF));
+#pragma unroll
+            for (int k = 0; k < GR_OWN; k++) {
+                if ((uint32_t)k >= g && own_shape[k] != 0) { // wave-uniform: rows of earlier groups have met these pivots as pivots themselves
+                    float acc[1][RT_T];
+                    RtRow<NARROW> rows[1];
+                    uint32_t shape[1];
+                    rows[0] = own[k];
+                    rows[0].touch();
+                    shape[0] = own_shape[k];
+                    asm volatile("" : "+s"(shape[0]));
+#pragma unroll
+                    for (int t = 0; t < RT_T; t++) acc[0][t] = 0.f;
+                    ranktab_probe_rows<NARROW, 1>(T, rows, shape, [&](int) { return row_pairs(wave + 8 * k); }, n_ovf, acc, lane);
+                    uint32_t t;
+                    const float z = wave_sum_1x8(acc[0], lane, &t);
+                    const uint32_t b = wave + 8 * k, p = 8 * g + lo + t;
+                    if ((lane & 15) < 4 && (lane & 32) == 0 && t < cnt && p < b) G[p * GRAM_STRIDE + b] += z;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            lo += cnt;
+            GTICK(9);
+            __syncthreads(); // the table is rebuilt next
+            GTICK(10);
+        }
+    }
+    for (uint32_t t = tid; t < m * m; t += nthreads) {
+        const uint32_t i = t / m, j = t % m;
+        if (i > j) G[i * GRAM_STRIDE + j] = G[j * GRAM_STRIDE + i];
+    }
+    __syncthreads();
+}
+
 // Same result as prune_kernel, different traffic: the node's <= 64 neighbour rows are read
 // once, their hybrid Gram matrix is built in LDS (dense part on the matrix cores), every
 // row's overlap with the centre node's BM25 terms becomes a bit mask, and the sequential
 // RNG-IP selection with its keyword flags then runs on LDS only:
 //   <c,s> = G[c][s];   flag(c,s) = (R[s] & ~R[c]) != 0   with R[x] = bm25(x) ∩ bm25(u).
 template <int NT, bool NARROW>
-__global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dense_mul, const float* __restrict__ norms,
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void prune_gram_kernel(CorpusView C, float dense_mul, const float* __restrict__ norms,
                                                                 const uint32_t* __restrict__ ids, const float* __restrict__ dist,
                                                                 uint32_t d, uint32_t* fwd, uint32_t* det_out, uint32_t* cnt_out,
                                                                 uint32_t* kw_out, uint32_t term_slots, uint32_t tgroup,
                                                                 uint32_t umap_slots, uint32_t map_slots, uint32_t words,
-                                                                uint32_t union_slots, unsigned long long* gfail) {
+                                                                uint32_t union_slots, uint32_t rank_bits, uint32_t rank_slots,
+                                                                uint32_t rank_span, unsigned long long* gfail) {
     constexpr uint32_t K = GRAM_ROWS;
     C.narrow = NARROW ? 1u : 0u; // the pair format as a compile-time constant: no branch at the loads
     extern __shared__ __align__(16) char smem[];
-    const GramPruneLds L(term_slots, tgroup, umap_slots, map_slots, words, union_slots);
+    const GramPruneLds L(term_slots, tgroup, umap_slots, map_slots, words, union_slots, rank_bits, rank_slots, NARROW);
     float* G = reinterpret_cast<float*>(smem + L.G);
     uint2* tabs = reinterpret_cast<uint2*>(smem + L.tabs);
     uint32_t* ovf_cnt = reinterpret_cast<uint32_t*>(smem + L.ovf_cnt);
@@ -313,7 +398,7 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     uint32_t* o_kw = reinterpret_cast<uint32_t*>(smem + L.o_kw);
     volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
 
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const int tid = threadIdx.x, wave = (int)uniform(tid / WAVE), lane = lane_id();
     const uint32_t u = blockIdx.x, umask = umap_slots - 1, mmask = map_slots - 1;
     const size_t base = (size_t)u * K;
     const uint64_t lane_lt = (1ull << lane) - 1;
@@ -324,6 +409,9 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     for (uint32_t i = tid; i < K; i += NT) det[i] = 0;
     for (uint32_t i = tid; i < K * 2; i += NT) F[i] = 0;
     if (tid < 16) ctl[tid] = 0;
+#ifdef APOE_PRUNE_TIMING
+    unsigned long long t0_ = wall_clock64();
+#endif
     __syncthreads();
 
     if (wave == 0) {
@@ -355,8 +443,11 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
         }
     }
     __syncthreads();
-    const uint32_t m = ctl[PC_M];
+    const uint32_t m = uniform(ctl[PC_M]);
+    TICK(0);
 
+    const bool rank = rank_slots != 0; // the sparse part runs on the rank table with the rows held in registers
+    if (rank) gram_rows_gather(C, nb_id, m, rowptr, rownnz, tid, NT);
     // (a) detour counts (as prune_kernel)
     for (uint32_t i = tid; i < m; i += NT) {
         const uint32_t key = nb_id[i];
@@ -369,7 +460,16 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
         }
     }
     // R[r] = bits of u's BM25 terms that row r holds too: one wave per row, lanes over its BM25 pairs
-    for (uint32_t r = wave; r < m; r += NT / WAVE) {
+    auto mark = [&](uint32_t r, uint32_t key) {
+        uint32_t h = term_hash(key, umask);
+        while (true) {
+            const uint2 e = umap[h];
+            if (e.x == key) { atomicOr(&R[r * words + (e.y >> 5)], 1u << (e.y & 31)); break; }
+            if (e.x == EMPTY) break;
+            h = (h + 1) & umask;
+        }
+    };
+    for (uint32_t r = wave; r < (rank ? 0u : m); r += NT / WAVE) {
         const uint64_t dr = C.desc[nb_id[r]];
         const Pairs sp = record_pairs(C, dr);
         const uint32_t ns = desc_nnz_s(dr), nb = desc_nnz_b(dr);
@@ -385,6 +485,21 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
         }
     }
     __syncthreads();
+    // this wave's rows w, w + 8, ...: requested now, used from the keyword masks on
+    static_assert(NT / WAVE == 8 || NT / WAVE == 4, "rows are dealt out to eight waves");
+    RtRow<NARROW> own[GR_OWN];
+    uint32_t own_shape[GR_OWN];
+#pragma unroll
+    for (int k = 0; k < GR_OWN; k++) {
+        const uint32_t b = wave + 8 * k;
+        own_shape[k] = 0;
+        if (rank && b < m) {
+            own_shape[k] = uniform(rownnz[b]);
+            Pairs sp = gram_row(C, rowptr, rownnz, b);
+            sp.narrow = NARROW ? 1u : 0u;
+            rt_row_load(own[k], sp, lane);
+        }
+    }
     for (uint32_t t = tid; t < m * K; t += NT) {
         const uint32_t r = t / K, j = t % K;
         const size_t at = (size_t)nb_id[r] * K + j;
@@ -399,6 +514,26 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
             }
             if (e.x == EMPTY) break;
             h = (h + 1) & mmask;
+        }
+    }
+    __syncthreads();
+    TICK(1);
+    if (rank) {
+#pragma unroll
+        for (int k = 0; k < GR_OWN; k++) {
+            const uint32_t nnz = own_shape[k] & 0xFFFFu, ns = own_shape[k] >> 16, r = wave + 8 * k;
+            if (nnz > ns) { // wave-uniform: the row has BM25 pairs
+#pragma unroll
+                for (int c = 0; c < RT_CHUNKS; c++) {
+                    const uint32_t j = c * WAVE + lane;
+                    if (j >= ns && j < nnz) mark(r, own[k].key(c) | (NARROW ? 0x80000000u : 0u));
+                }
+                if (nnz > RT_CHUNKS * WAVE) {
+                    Pairs sp = gram_row(C, rowptr, rownnz, r);
+                    sp.narrow = NARROW ? 1u : 0u;
+                    for (uint32_t j = max(ns, (uint32_t)(RT_CHUNKS * WAVE)) + lane; j < nnz; j += WAVE) mark(r, sp.key(j));
+                }
+            }
         }
     }
     // hybrid Gram matrix of the m rows
@@ -416,9 +551,14 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
         if (active && part == 1) gram_dense_store(G, wave & 3, lane, acc, dense_mul, true);
     }
     __syncthreads();
-    if (union_slots) gram_sparse_union(C, nb_id, m, G, reinterpret_cast<char*>(tabs), union_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
+    TICK(2);
+    if (rank) {
+        const RankTab T = ranktab_at(reinterpret_cast<char*>(tabs), rank_bits, rank_slots, rank_span, NARROW);
+        gram_sparse_rank<NARROW>(C, m, G, T, ovf_cnt, rowptr, rownnz, own, own_shape, (uint32_t*)&ctl[PC_FAIL], tid, NT);
+    } else if (union_slots) gram_sparse_union(C, nb_id, m, G, reinterpret_cast<char*>(tabs), union_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else if (tgroup == 8) gram_sparse_64<8>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else gram_sparse_64<4>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
+    TICK(3);
     // (b) stable order by detour count
     for (uint32_t i = tid; i < m; i += NT) {
         const uint32_t key = (det[i] << 16) | i;
@@ -437,6 +577,7 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     }
     __syncthreads();
 
+    TICK(4);
     // (c)+(d) sequential selection on the Gram matrix: wave 0, lane i keeps selected member i in registers
     if (wave == 0 && m > 0) {
         uint32_t n_sel = 1;
@@ -485,6 +626,7 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
             for (uint32_t j = nkw; j < APOE_KW_CAND; j++) o_kw[1 + j] = 0;
         }
     }
+    TICK(5);
     if (m == 0 && tid == 0) {
         for (uint32_t j = 0; j < d; j++) { o_fwd[j] = u; o_det[j] = EMPTY; }
         for (uint32_t j = 0; j <= APOE_KW_CAND; j++) o_kw[j] = 0;
@@ -498,7 +640,8 @@ __global__ __launch_bounds__(NT) void prune_gram_kernel(CorpusView C, float dens
     for (uint32_t i = tid; i < 1 + APOE_KW_CAND; i += NT) kw_out[(size_t)u * (1 + APOE_KW_CAND) + i] = o_kw[i];
     if (tid == 0) {
         cnt_out[u] = ctl[PC_CNT];
-        if (ctl[PC_FAIL]) atomicOr(gfail, 1ull); // an overflow list was too short: the host redoes the prune with prune_kernel
+        if (ctl[PC_FAIL]) atomicOr(gfail, 1ull);
+        TICK(6); // an overflow list was too short: the host redoes the prune with prune_kernel
     }
 }
 
@@ -629,14 +772,32 @@ int launch_prune(apoe_knn* g, uint32_t degree) {
     const double mean_nnz = g->n ? (double)g->corpus->total_pairs / g->n : 0.0;
     uint32_t union_slots = std::max(next_pow2((uint32_t)std::ceil(2.5 * GU_T * mean_nnz)), std::max(512u, gram_slots));
     if (GramPruneLds(gram_slots, tgroup, uset_slots, map_slots, words, union_slots).total > lds_budget) union_slots = 0;
-    const GramPruneLds GL(gram_slots, tgroup, uset_slots, map_slots, words, union_slots);
+    // rank table for eight pivots when its bitmap leaves room for the values of at least the longest row (and then as many
+    // slots as the budget allows, up to eight rows' worth): the sparse part then runs with the rows held in registers
+    const bool narrow = g->corpus->narrow;
+    const uint32_t rank_span = next_pow2(std::max(g->corpus->max_term + 1, 1024u));
+    const uint32_t rank_bits = narrow ? 2 * rank_span : 65536u;
+    uint32_t rank_slots = 0;
+    {
+        const uint32_t longest = g->corpus->max_nnz_s + g->corpus->max_nnz_b;
+        const uint32_t fixed = GramPruneLds(gram_slots, tgroup, uset_slots, map_slots, words, 0, rank_bits, 64, narrow).total -
+                               RankTabLds(rank_bits, 64, narrow).total + RankTabLds(rank_bits, 0, narrow).total;
+        const uint32_t per_slot = RT_T * 4 + (narrow ? 0 : 4);
+        if (fixed + 64 < lds_budget) {
+            uint32_t fit = ((lds_budget - fixed - 64) / per_slot) & ~63u;
+            fit = std::min(fit, (RT_T * longest + 63) & ~63u);
+            if (fit >= std::max(longest, 64u)) rank_slots = fit;
+        }
+        if (getenv("APOE_PRUNE_NO_RANK")) rank_slots = 0;
+    }
+    const GramPruneLds GL(gram_slots, tgroup, uset_slots, map_slots, words, union_slots, rank_bits, rank_slots, narrow);
     if (g->K == GRAM_ROWS && GL.total <= lds_budget && !g->force_sequential_prune) {
         APOE_HIP(hipMemsetAsync(g->counter.p + 1, 0, sizeof(unsigned long long), ctx->stream));
         auto kernel = g->corpus->narrow ? &prune_gram_kernel<GRAM_THREADS, true> : &prune_gram_kernel<GRAM_THREADS, false>;
         APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GL.total));
         kernel<<<g->n, GRAM_THREADS, GL.total, ctx->stream>>>(g->corpus->view(), g->dense_scale * g->dense_scale, g->norms.p, g->ids.p, g->dist.p, degree,
                                                               g->fwd.p, g->det.p, g->cnt.p, g->kw.p, gram_slots, tgroup, uset_slots, map_slots, words,
-                                                              union_slots, g->counter.p + 1);
+                                                              union_slots, rank_bits, rank_slots, rank_span, g->counter.p + 1);
         APOE_HIP(hipGetLastError());
         unsigned long long failed = 0;
         APOE_HIP(hipMemcpyAsync(&failed, g->counter.p + 1, sizeof(failed), hipMemcpyDeviceToHost, ctx->stream));
@@ -687,6 +848,14 @@ int launch_final_graph(apoe_knn* g, uint32_t* rows_dev) {
 using namespace apoe;
 
 extern "C" {
+#ifdef APOE_PRUNE_TIMING
+int apoe_debug_prune_ticks(unsigned long long* out16) {
+    hipMemcpyFromSymbol(out16, HIP_SYMBOL(apoe::apoe_prune_ticks), 16 * 8);
+    unsigned long long z[16] = {0};
+    hipMemcpyToSymbol(HIP_SYMBOL(apoe::apoe_prune_ticks), z, 16 * 8);
+    return 0;
+}
+#endif
 
 int apoe_prune(apoe_knn* g, uint32_t degree) {
     APOE_REQUIRE(g, "null argument");
