@@ -29,6 +29,7 @@ constexpr int GRAM_STRIDE = GRAM_ROWS + 1; // odd stride: column reads do not co
 // accumulator register v of lane l is C[8 * (v / 4) + 4 * (l / 32) + v % 4][l % 32].
 // A lane therefore streams ITS row: float4 number (2 * block + l / 32) of every 8-float block,
 // and the four components go into four consecutive MFMAs (the k order inside the sum is free).
+template <bool DIAG>
 __device__ __forceinline__ floatx16 gram_dense_tile(const CorpusView& C, const uint32_t* ids, uint32_t m, int tile, int lane, int b_begin,
                                                     int b_end, bool& active) {
     const int ti = tile >> 1, tj = tile & 1;
@@ -40,30 +41,34 @@ __device__ __forceinline__ floatx16 gram_dense_tile(const CorpusView& C, const u
     const uint32_t ra = min((uint32_t)(ti * 32 + (lane & 31)), m - 1), rb = min((uint32_t)(tj * 32 + (lane & 31)), m - 1);
     const float4* pa = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[ra]]) * 16) + (lane >> 5);
     const float4* pb = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[rb]]) * 16) + (lane >> 5);
-    if (ti == tj) {
-        for (int b = b_begin; b < b_end; b += 4) {
-            float4 a[4];
+    // operands of the next batch of 8-float blocks are requested before the current batch is multiplied; a diagonal
+    // tile (DIAG: ti == tj) reads one operand only and takes batches twice as long for the same registers
+    constexpr int NB = 4, NBB = DIAG ? 1 : NB;
+    float4 a[2][NB], bb[2][NBB];
 #pragma unroll
-            for (int u = 0; u < 4; u++) a[u] = pa[2 * (b + u)];
+    for (int u = 0; u < NB; u++) {
+        a[0][u] = pa[2 * (b_begin + u)];
+        if (!DIAG) bb[0][u] = pb[2 * (b_begin + u)];
+    }
+#pragma unroll 1
+    for (int b = b_begin; b < b_end; b += 2 * NB) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].x, a[u].x, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].y, a[u].y, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].z, a[u].z, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].w, a[u].w, acc, 0, 0, 0);
+        for (int half = 0; half < 2; half++) {
+            const int nb = b + (half + 1) * NB; // first block of the batch after this one
+            if (nb < b_end) {
+#pragma unroll
+                for (int u = 0; u < NB; u++) {
+                    a[half ^ 1][u] = pa[2 * (nb + u)];
+                    if (!DIAG) bb[half ^ 1][u] = pb[2 * (nb + u)];
+                }
             }
-        }
-    } else {
-        for (int b = b_begin; b < b_end; b += 4) {
-            float4 a[4], bb[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) { a[u] = pa[2 * (b + u)]; bb[u] = pb[2 * (b + u)]; }
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].x, bb[u].x, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].y, bb[u].y, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].z, bb[u].z, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].w, bb[u].w, acc, 0, 0, 0);
+            for (int u = 0; u < NB; u++) {
+                const float4 x = a[half][u], y = DIAG ? a[half][u] : bb[half][DIAG ? 0 : u];
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, y.x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, y.y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, y.z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, y.w, acc, 0, 0, 0);
             }
         }
     }

@@ -236,10 +236,11 @@ __device__ __forceinline__ float wave_sum4_dpp(const float acc[4], int lane, uin
     return z;
 }
 
-constexpr int RT_CHUNKS = 4; // 64-pair chunks of a streamed row kept in registers (256 pairs); longer rows read the rest when they are probed
+constexpr int RT_CHUNKS = 4; // pairs of a streamed row per lane kept in registers (256 pairs a row); longer rows read the rest when they are probed
 
-// Raw pairs of a streamed row in registers: lane l holds pairs l, l + 64, l + 128, l + 192. Narrow keys are 16 bits
-// wide: two share a register.
+// Raw pairs of a streamed row in registers: lane l holds the four consecutive pairs 4l .. 4l + 3 (one 16-byte load of
+// values and one 8-byte load of terms per lane and narrow row). Narrow keys are 16 bits wide: two share a register.
+__device__ __forceinline__ uint32_t rt_pair(int c, int lane) { return (uint32_t)(RT_CHUNKS * lane + c); }
 template <bool NARROW>
 struct RtRow;
 template <>
@@ -276,12 +277,23 @@ __device__ __forceinline__ void rt_row_select(RtRow<false>& dst, const RtRow<fal
         dst.k[c] = take ? src.k[c] : dst.k[c];
     }
 }
-template <bool NARROW>
-__device__ __forceinline__ void rt_row_load(RtRow<NARROW>& r, const Pairs& sp, int lane) {
+__device__ __forceinline__ void rt_row_load(RtRow<true>& r, const Pairs& sp, int lane) {
+    static_assert(RT_CHUNKS == 4, "one uint4 of values and one uint2 of terms per lane");
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    uint2 k = make_uint2(0u, 0u);
+    if (rt_pair(0, lane) < sp.nnz) { // the arrays start on 128-byte boundaries and are padded to them: the last lane reads inside the record
+        v = reinterpret_cast<const uint4*>(sp.base)[lane];
+        k = reinterpret_cast<const uint2*>(sp.base + narrow_keys_offset(sp.nnz))[lane];
+    }
+    r.v[0] = v.x; r.v[1] = v.y; r.v[2] = v.z; r.v[3] = v.w;
+    r.k2[0] = k.x; r.k2[1] = k.y;
+}
+__device__ __forceinline__ void rt_row_load(RtRow<false>& r, const Pairs& sp, int lane) {
 #pragma unroll
-    for (int c = 0; c < RT_CHUNKS; c++) {
-        const uint32_t j = c * WAVE + lane;
-        r.set(c, j < sp.nnz ? sp.raw(j) : make_uint2(0u, 0u));
+    for (int c = 0; c < RT_CHUNKS; c += 2) {
+        uint4 kv = make_uint4(0u, 0u, 0u, 0u);
+        if (rt_pair(c, lane) < sp.nnz) kv = reinterpret_cast<const uint4*>(sp.base)[(RT_CHUNKS * lane + c) / 2]; // an odd count: the second pair is masked by its index
+        r.k[c] = kv.x; r.v[c] = kv.y; r.k[c + 1] = kv.z; r.v[c + 1] = kv.w;
     }
 }
 
@@ -296,7 +308,7 @@ __device__ __forceinline__ uint32_t ranktab_build_rows(const RankTab& T, const R
     return ranktab_build_each<NARROW>(T, [&](auto f) {
 #pragma unroll
         for (int c = 0; c < RT_CHUNKS; c++) {
-            const uint32_t j = c * WAVE + lane;
+            const uint32_t j = rt_pair(c, lane);
             if (j < nnz) f(make_uint2(pr.key(c), pr.v[c]), NARROW ? j >= ns : false, t);
         }
         for (uint32_t j = RT_CHUNKS * WAVE + lane; j < nnz; j += WAVE) f(tail.raw(j), j >= ns, t);
@@ -329,14 +341,14 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
     };
     auto index_of = [&](int r, int c) {
         const uint32_t key = rows[r].key(c);
-        return ranktab_index<NARROW>(T, key, NARROW ? (uint32_t)(c * WAVE + lane) >= (shape[r] >> 16) : (int)key < 0);
+        return ranktab_index<NARROW>(T, key, NARROW ? rt_pair(c, lane) >= (shape[r] >> 16) : (int)key < 0);
     };
     uint2 w[NB][RT_CHUNKS];
 #pragma unroll
     for (int r = 0; r < NB; r++) {
         const uint32_t nnz = shape[r] & 0xFFFFu;
 #pragma unroll
-        for (int c = 0; c < RT_CHUNKS; c++) w[r][c] = T.word[(uint32_t)(c * WAVE + lane) < nnz ? index_of(r, c) >> 5 : 0u];
+        for (int c = 0; c < RT_CHUNKS; c++) w[r][c] = T.word[rt_pair(c, lane) < nnz ? index_of(r, c) >> 5 : 0u];
     }
 #pragma unroll
     for (int r = 0; r < NB; r++) asm volatile("" : "+v"(w[r][0].x), "+v"(w[r][1].x), "+v"(w[r][2].x), "+v"(w[r][3].x));
@@ -350,7 +362,7 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
             const uint32_t nnz = shape[r] & 0xFFFFu;
 #pragma unroll
             for (int c = 0; c < 2; c++) {
-                const bool in = (uint32_t)((h + c) * WAVE + lane) < nnz;
+                const bool in = rt_pair(h + c, lane) < nnz;
                 p[r][c] = ranktab_locate<NARROW>(T, w[r][h + c], index_of(r, h + c), rows[r].v[h + c], in);
                 lo[r][c] = T.vals[2 * p[r][c].slot];
                 hi[r][c] = T.vals[2 * p[r][c].slot + 1];
@@ -367,7 +379,7 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
             for (int c = 0; c < 2; c++) add8(r, ok[r][c] ? p[r][c].mul : 0.f, lo[r][c], hi[r][c]);
             if (!NARROW && n_ovf) {
 #pragma unroll
-                for (int c = 0; c < 2; c++) overflow(r, rows[r].key(h + c), rows[r].v[h + c], (uint32_t)((h + c) * WAVE + lane) < nnz && !ok[r][c]);
+                for (int c = 0; c < 2; c++) overflow(r, rows[r].key(h + c), rows[r].v[h + c], rt_pair(h + c, lane) < nnz && !ok[r][c]);
             }
         }
     }

@@ -485,7 +485,55 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
     }
     __syncthreads();
-    // this wave's rows w, w + 8, ...: requested now, used from the keyword masks on
+    {   // all list entries of this thread are requested before the first one is looked up
+        constexpr uint32_t PER = K * K / NT;
+        uint32_t xs[PER];
+        float dxs[PER];
+#pragma unroll
+        for (uint32_t k = 0; k < PER; k++) {
+            const uint32_t t = tid + k * NT, r = t / K, j = t % K;
+            xs[k] = EMPTY;
+            dxs[k] = 0.f;
+            if (t < m * K) {
+                const size_t at = (size_t)nb_id[r] * K + j;
+                xs[k] = ids[at] & ~FLAG;
+                dxs[k] = dist[at];
+            }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < PER; k++) {
+            const uint32_t r = (tid + k * NT) / K, x = xs[k];
+            if (x == EMPTY) continue;
+            uint32_t h = term_hash(x, mmask);
+            while (true) {
+                const uint2 e = idmap[h];
+                if (e.x == x) {
+                    if (e.y > r && dxs[k] < nb_dist[e.y]) atomicAdd(&det[e.y], 1u);
+                    break;
+                }
+                if (e.x == EMPTY) break;
+                h = (h + 1) & mmask;
+            }
+        }
+    }
+    __syncthreads();
+    TICK(1);
+    // hybrid Gram matrix of the m rows. Only the upper triangle of G is used (the sparse part is added there and the
+    // lower triangle is mirrored from it at the end), so the lower left tile is not computed. The eight waves share
+    // the three tiles by the bytes they read: each diagonal tile (one operand) goes to two waves, half of the
+    // dimensions each, the upper right tile (two operands) to four waves, a quarter of the dimensions each. Partial
+    // sums are added into G in a fixed order (barriers between them): the result does not depend on timing.
+    constexpr int NWAVES = NT / WAVE, BLOCKS = DIM / 8;
+    static_assert(NWAVES == 8, "the dense tiles are dealt out to eight waves");
+    const int dtile = wave < 2 ? 0 : wave < 4 ? 3 : 1, dparts = wave < 4 ? 2 : 4, dpart = wave < 4 ? (wave & 1) : wave - 4;
+    bool dactive = false;
+    floatx16 dacc;
+    if (m > 0) {
+        if (wave < 4) dacc = gram_dense_tile<true>(C, nb_id, m, dtile, lane, dpart * (BLOCKS / dparts), (dpart + 1) * (BLOCKS / dparts), dactive);
+        else dacc = gram_dense_tile<false>(C, nb_id, m, dtile, lane, dpart * (BLOCKS / dparts), (dpart + 1) * (BLOCKS / dparts), dactive);
+    }
+    TICK(7);
+    // this wave's rows w, w + 8, ...: requested as soon as the wave's dense tile is done (its operands need the registers), used from the keyword masks on
     static_assert(NT / WAVE == 8 || NT / WAVE == 4, "rows are dealt out to eight waves");
     RtRow<NARROW> own[GR_OWN];
     uint32_t own_shape[GR_OWN];
@@ -500,33 +548,39 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             rt_row_load(own[k], sp, lane);
         }
     }
-    for (uint32_t t = tid; t < m * K; t += NT) {
-        const uint32_t r = t / K, j = t % K;
-        const size_t at = (size_t)nb_id[r] * K + j;
-        const uint32_t x = ids[at] & ~FLAG;
-        const float dx = dist[at];
-        uint32_t h = term_hash(x, mmask);
-        while (true) {
-            const uint2 e = idmap[h];
-            if (e.x == x) {
-                if (e.y > r && dx < nb_dist[e.y]) atomicAdd(&det[e.y], 1u);
-                break;
-            }
-            if (e.x == EMPTY) break;
-            h = (h + 1) & mmask;
-        }
+    // (b) stable order by detour count (LDS only: runs while the rows arrive)
+    for (uint32_t i = tid; i < m; i += NT) {
+        const uint32_t key = (det[i] << 16) | i;
+        uint32_t r = 0;
+        for (uint32_t j = 0; j < m; j++) r += ((det[j] << 16) | j) < key;
+        order[r] = i;
     }
-    __syncthreads();
-    TICK(1);
+    for (int ph = 0; ph < 4; ph++) {
+        if (dactive && dpart == ph) gram_dense_store(G, dtile, lane, dacc, dense_mul, ph != 0);
+        if (ph < 3) __syncthreads();
+    }
     if (rank) {
 #pragma unroll
         for (int k = 0; k < GR_OWN; k++) {
             const uint32_t nnz = own_shape[k] & 0xFFFFu, ns = own_shape[k] >> 16, r = wave + 8 * k;
             if (nnz > ns) { // wave-uniform: the row has BM25 pairs
+                // the first table slot of all four pairs is read before any is compared; the probe loop is for the
+                // pairs whose slot holds another term
+                uint32_t key[RT_CHUNKS], h[RT_CHUNKS];
+                uint2 e[RT_CHUNKS];
 #pragma unroll
                 for (int c = 0; c < RT_CHUNKS; c++) {
-                    const uint32_t j = c * WAVE + lane;
-                    if (j >= ns && j < nnz) mark(r, own[k].key(c) | (NARROW ? 0x80000000u : 0u));
+                    key[c] = own[k].key(c) | (NARROW ? 0x80000000u : 0u);
+                    h[c] = term_hash(key[c], umask);
+                    e[c] = umap[h[c]];
+                }
+#pragma unroll
+                for (int c = 0; c < RT_CHUNKS; c++) {
+                    const uint32_t j = rt_pair(c, lane);
+                    if (j >= ns && j < nnz) {
+                        if (e[c].x == key[c]) atomicOr(&R[r * words + (e[c].y >> 5)], 1u << (e[c].y & 31));
+                        else if (e[c].x != EMPTY) mark(r, key[c]);
+                    }
                 }
                 if (nnz > RT_CHUNKS * WAVE) {
                     Pairs sp = gram_row(C, rowptr, rownnz, r);
@@ -535,20 +589,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 }
             }
         }
-    }
-    // hybrid Gram matrix of the m rows
-    // waves 0-3 take the first half of the dimensions of the tiles, waves 4-7 (if there) the second half. Only the
-    // upper triangle of G is used (the sparse part is added there and the lower triangle is mirrored from it at the
-    // end), so the lower left tile is not computed: its two row blocks would be read a third time for nothing.
-    {
-        constexpr int NWAVES = NT / WAVE, PARTS = NWAVES >= 8 ? 2 : 1, BLOCKS = DIM / 8;
-        const int part = wave >> 2;
-        bool active = false;
-        floatx16 acc;
-        if (m > 0 && part < PARTS && (wave & 3) != 2) acc = gram_dense_tile(C, nb_id, m, wave & 3, lane, part * (BLOCKS / PARTS), (part + 1) * (BLOCKS / PARTS), active);
-        if (active && part == 0) gram_dense_store(G, wave & 3, lane, acc, dense_mul, false);
-        __syncthreads();
-        if (active && part == 1) gram_dense_store(G, wave & 3, lane, acc, dense_mul, true);
     }
     __syncthreads();
     TICK(2);
@@ -559,15 +599,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     else if (tgroup == 8) gram_sparse_64<8>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else gram_sparse_64<4>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     TICK(3);
-    // (b) stable order by detour count
-    for (uint32_t i = tid; i < m; i += NT) {
-        const uint32_t key = (det[i] << 16) | i;
-        uint32_t r = 0;
-        for (uint32_t j = 0; j < m; j++) r += ((det[j] << 16) | j) < key;
-        order[r] = i;
-    }
-    __syncthreads();
-
     // keyword flags of all pairs at once (index.cu:637,651-654): flag(c, s) = (R[s] & ~R[c]) != 0
     for (uint32_t p = tid; p < m * m; p += NT) {
         const uint32_t c = p / m, sidx = p % m;
@@ -578,23 +609,32 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     __syncthreads();
 
     TICK(4);
-    // (c)+(d) sequential selection on the Gram matrix: wave 0, lane i keeps selected member i in registers
+    // (c)+(d) sequential selection on the Gram matrix: wave 0, lane i keeps selected member i in registers and the
+    // candidate at position i of the order (its Gram row, norm and flag word are handed out with readlane); the Gram
+    // entries of step t + 1 are requested before step t is decided (the lane that would hold candidate t as a new
+    // member asks for its entry too), so a step waits for no memory
     if (wave == 0 && m > 0) {
+        const uint32_t ord = (uint32_t)lane < m ? order[lane] : order[0];
+        const float nrm_o = nrm[ord];
+        const uint32_t f_lo = F[ord * 2], f_hi = F[ord * 2 + 1];
+        const uint32_t id_o = nb_id[ord], det_o = det[ord];
         uint32_t n_sel = 1;
-        uint32_t my_gi = order[0], my_kw = 0;
+        uint32_t my_gi = (uint32_t)__builtin_amdgcn_readlane((int)ord, 0), my_kw = 0;
         bool my_live = lane == 0;
-        float my_nrm = nrm[my_gi];
+        float my_nrm = readlane_f32(nrm_o, 0);
+        float p_next = 0.f;
+        if (m > 1) p_next = G[(uint32_t)__builtin_amdgcn_readlane((int)ord, 1) * GRAM_STRIDE + my_gi];
         for (uint32_t t = 1; t < m; t++) {
-            const uint32_t c = uniform(order[t]);
-            const float norm_c = nrm[c];
-            const uint64_t fc = ((uint64_t)F[c * 2 + 1] << 32) | F[c * 2];
-            bool rej = false, noflag = false, tomb = false;
-            if ((uint32_t)lane < n_sel && my_live) {
-                const float p = G[c * GRAM_STRIDE + my_gi];
-                rej = norm_c < p;
-                tomb = my_nrm < p;
-                noflag = !((fc >> my_gi) & 1ull);
+            const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)ord, (int)t);
+            const float norm_c = readlane_f32(nrm_o, t);
+            const uint64_t fc = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)f_hi, (int)t) << 32) | (uint32_t)__builtin_amdgcn_readlane((int)f_lo, (int)t);
+            const float p = p_next;
+            if (t + 1 < m) {
+                const uint32_t cn = (uint32_t)__builtin_amdgcn_readlane((int)ord, (int)(t + 1));
+                p_next = G[cn * GRAM_STRIDE + ((uint32_t)lane == n_sel ? c : my_gi)];
             }
+            const bool act = (uint32_t)lane < n_sel && my_live;
+            const bool rej = act && norm_c < p, tomb = act && my_nrm < p, noflag = act && !((fc >> my_gi) & 1ull);
             const bool reject = __ballot(rej) != 0;
             const bool allflag = __ballot(noflag) == 0;
             if (tomb) my_live = false;
@@ -603,28 +643,30 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 n_sel++;
             }
         }
-        if ((uint32_t)lane < n_sel) { sel_gi[lane] = my_gi; sel_live[lane] = my_live ? 1u : 0u; sel_kw[lane] = my_kw; }
-        wave_fence_lds();
-        // (e) emit
-        if (lane == 0) {
-            uint32_t cnt = 0, nkw = 0;
-            for (uint32_t i = 0; i < n_sel; i++) {
-                if (!sel_live[i]) continue;
-                const uint32_t gi = sel_gi[i];
-                if (cnt < d) { o_fwd[cnt] = nb_id[gi]; o_det[cnt] = det[gi]; cnt++; }
-                else if (sel_kw[i] && nkw < APOE_KW_CAND) { o_kw[1 + nkw] = nb_id[gi]; nkw++; }
-            }
-            for (uint32_t t = 0; t < m && cnt < d; t++) {
-                const uint32_t cidv = nb_id[order[t]];
-                bool present = false;
-                for (uint32_t j = 0; j < cnt; j++) present |= o_fwd[j] == cidv;
-                if (!present) { o_fwd[cnt] = cidv; o_det[cnt] = det[order[t]]; cnt++; }
-            }
-            ctl[PC_CNT] = cnt;
-            for (; cnt < d; cnt++) { o_fwd[cnt] = u; o_det[cnt] = EMPTY; }
-            o_kw[0] = nkw;
-            for (uint32_t j = nkw; j < APOE_KW_CAND; j++) o_kw[1 + j] = 0;
+        // (e) emit: live members in selection order fill the row, flagged ones beyond d become keyword candidates
+        const bool live = (uint32_t)lane < n_sel && my_live;
+        const uint64_t lb = __ballot(live);
+        const uint32_t pos = __popcll(lb & lane_lt);
+        const uint32_t my_id = nb_id[my_gi], my_det = det[my_gi];
+        if (live && pos < d) { o_fwd[pos] = my_id; o_det[pos] = my_det; }
+        uint32_t cnt = min((uint32_t)__popcll(lb), d);
+        const bool kwc = live && pos >= d && my_kw;
+        const uint64_t kb = __ballot(kwc);
+        const uint32_t kpos = __popcll(kb & lane_lt);
+        if (kwc && kpos < APOE_KW_CAND) o_kw[1 + kpos] = my_id;
+        const uint32_t nkw = min((uint32_t)__popcll(kb), (uint32_t)APOE_KW_CAND);
+        if (cnt < d) { // fewer survivors than the row has slots: the remaining neighbours in order, each id once
+            bool add = (uint32_t)lane < m;
+            for (uint64_t rest = lb; rest; rest &= rest - 1) add = add && (uint32_t)__builtin_amdgcn_readlane((int)my_id, __builtin_ctzll(rest)) != id_o;
+            for (uint32_t t = 0; t + 1 < m; t++) add = add && !((uint32_t)lane > t && (uint32_t)__builtin_amdgcn_readlane((int)id_o, (int)t) == id_o);
+            const uint64_t ab = __ballot(add);
+            const uint32_t at = cnt + __popcll(ab & lane_lt);
+            if (add && at < d) { o_fwd[at] = id_o; o_det[at] = det_o; }
+            cnt = min(d, cnt + (uint32_t)__popcll(ab));
         }
+        if (lane == 0) { ctl[PC_CNT] = cnt; o_kw[0] = nkw; }
+        for (uint32_t j = cnt + lane; j < d; j += WAVE) { o_fwd[j] = u; o_det[j] = EMPTY; }
+        for (uint32_t j = nkw + lane; j < APOE_KW_CAND; j += WAVE) o_kw[1 + j] = 0;
     }
     TICK(5);
     if (m == 0 && tid == 0) {
