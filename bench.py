@@ -29,7 +29,10 @@ HBM_PEAK_GBS = 8000.0
 # counters read for a 1 GiB copy) and not measured by this script: keyed by the workload they were taken on
 # (docs, degree, queries, cands, variant, NN-Descent step) with the profiles/ file that holds the run. Any other
 # workload reports null.
-RECORDED_TRAFFIC = {}
+RECORDED_TRAFFIC = {
+    (1_000_000, 48, 10_000, 256, 0, 1): {"default": 1.881e11, "every_dense_row_read": 5.326e11,
+                                          "source": "profiles/bench_1Mdocs_degree48_cands256.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy)"},
+}
 
 
 def log(*a):
