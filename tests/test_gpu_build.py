@@ -229,6 +229,42 @@ def test_gpu_built_index_recall(gpu_world, join):
     gq.close()
 
 
+def test_prune_of_short_and_ragged_lists_matches_oracle(gpu_world):
+    """Lists with fewer than K usable entries (distance at the empty mark, or the node itself): 0, 1, 2, 7, 8, 9,
+    31, 33 and 63 neighbours. The gather-once prune deals rows out to its waves and takes pivots eight at a time,
+    so every count around those boundaries has to give the oracle's rows."""
+    import apoe
+    import oracle as O
+    w = gpu_world
+    n = w["C"].n
+    ids, dist = w["knn_ids"].copy(), w["knn_dist"].copy()
+    rng = np.random.default_rng(77)
+    counts = (0, 1, 2, 7, 8, 9, 31, 33, 63)
+    nodes = rng.choice(n, size=40 * len(counts), replace=False)
+    for i, u in enumerate(nodes):
+        m = counts[i % len(counts)]
+        if i % 2 == 0:
+            dist[u, m:] = apoe.INF_DIS          # the tail is empty
+        else:
+            ids[u, m:] = u                       # the tail names the node itself
+    knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+    knn.upload(ids, dist)
+    knn.prune(32)
+    g_fwd, g_det, g_cnt, g_kw = knn.prune_download()
+    knn.close()
+    c_fwd, c_det, c_cnt, c_kw = O.prune(w["C"], 7.0, O.norms(w["C"], 7.0), ids, dist, 32)
+    same = np.all(g_fwd[nodes] == c_fwd[nodes], axis=1)
+    assert same.mean() >= 0.99, f"{(~same).sum()} of {len(nodes)} short lists give other rows"
+    ok = nodes[same]
+    assert np.array_equal(g_det[ok], c_det[ok]) and np.array_equal(g_cnt[ok], c_cnt[ok])
+    assert np.all(g_kw[ok] == c_kw[ok], axis=1).mean() >= 0.99
+    for m in (0, 1):
+        sel = nodes[[i for i in range(len(nodes)) if counts[i % len(counts)] == m]]
+        assert np.all(g_cnt[sel] == m)
+    # the untouched nodes still see their neighbours' (now shorter) lists in the detour counts: the whole output agrees too
+    assert np.all(g_fwd == c_fwd, axis=1).mean() >= 0.995
+
+
 def test_prune_k128_sequential_kernel_matches_oracle(gpu_world):
     """K = 128 lists go through the table-probing prune kernel (the gather-once form is K = 64 only)."""
     import apoe
