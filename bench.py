@@ -248,6 +248,35 @@ def main():
         log(f"[bench] KG search cands 128: {sk.kernel_ms:.2f} ms, entity document in the top 10 for {hits / nq_truth:.3f} of the queries")
         gkg.close()
 
+    # ---- where the recall target IS reached: the same generators, build and search on smaller corpora ----
+    smaller = None
+    if not args.no_sweeps:
+        smaller = []
+        for n_small, deg_small in ((4_000, 32), (30_000, 32), (100_000, 32)):
+            if n_small >= args.docs:
+                continue
+            c_s = S.corpus(n_small, device=dev)
+            gc_s = apoe.Corpus(ctx, *c_s)
+            g_s, ms_s = apoe.build_graph(ctx, gc_s, K=args.nnd_k, iters=args.nnd_iters, degree=deg_small, seed=1, join=args.join)
+            t_s, _ = B.hybrid_topk(c_s, queries, (1.0, 1.0, 1.0), 10, nq=nq_truth)
+            row = dict(docs=n_small, degree=deg_small, build_seconds_gpu=ms_s / 1e3, sweep=[], qps_at_recall_target=None, cands_at_recall_target=None)
+            for ec in (64, 128, 256, 512, 1024, 2048):
+                if ec >= n_small:
+                    break
+                apoe.search(ctx, gc_s, gq, g_s, (1.0, 1.0, 1.0), ec, max_iter=iter_cap(ec))
+                ids_s, _, ss = apoe.search(ctx, gc_s, gq, g_s, (1.0, 1.0, 1.0), ec, max_iter=iter_cap(ec))
+                rec_s = recall_at_k(ids_s[:nq_truth], t_s, 10)
+                row["sweep"].append(dict(cands=ec, recall=rec_s, kernel_ms=ss.kernel_ms, qps=args.queries / (ss.kernel_ms / 1e3)))
+                if rec_s >= 0.95 and row["cands_at_recall_target"] is None:
+                    row["cands_at_recall_target"], row["qps_at_recall_target"] = ec, args.queries / (ss.kernel_ms / 1e3)
+                    break
+            smaller.append(row)
+            log(f"[bench] {n_small} docs, degree {deg_small}: " + ", ".join(f"cands {x['cands']} recall {x['recall']:.3f}" for x in row["sweep"]) +
+                (f" -> {row['qps_at_recall_target']:.0f} QPS at recall@10 >= 0.95" if row["qps_at_recall_target"] else " -> target not reached"))
+            g_s.close()
+            gc_s.close()
+            del c_s
+
     extras = None
     if args.extras:
         extras = {}
@@ -400,6 +429,7 @@ def main():
             "kernel_ms": avg_kernel_ms,
             **({"weight_sweep_without_rebuild": weight_sweep} if weight_sweep else {}),
             **({"knowledge_graph_search": kg_search} if kg_search else {}),
+            **({"same_generators_smaller_corpora": smaller} if smaller else {}),
             **({"extras": extras} if extras else {}),
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
