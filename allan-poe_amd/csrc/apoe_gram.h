@@ -75,6 +75,60 @@ __device__ __forceinline__ floatx16 gram_dense_tile(const CorpusView& C, const u
     return acc;
 }
 
+// The three tiles of the upper triangle at once, over the 8-float blocks [b_begin, b_end) of the rows: a wave reads
+// its slice of rows 0-31 (operand a) and of rows 32-63 (operand b) once and feeds a x a, a x b and b x b from the same
+// registers, so every dense row is read from memory exactly once per node (tile by tile each row block is read
+// twice). m <= 32: only a x a. Batches of NB blocks, the next batch requested before the current one is multiplied.
+template <int NB>
+__device__ __forceinline__ void gram_dense_upper(const CorpusView& C, const uint32_t* ids, uint32_t m, int lane, int b_begin, int b_end,
+                                                 floatx16& acc00, floatx16& acc01, floatx16& acc11) {
+#pragma unroll
+    for (int v = 0; v < 16; v++) { acc00[v] = 0.f; acc01[v] = 0.f; acc11[v] = 0.f; }
+    if (m == 0) return;
+    const bool has_b = m > 32;
+    const uint32_t ra = min((uint32_t)(lane & 31), m - 1), rb = min((uint32_t)(32 + (lane & 31)), m - 1);
+    const float4* pa = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[ra]]) * 16) + (lane >> 5);
+    const float4* pb = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[rb]]) * 16) + (lane >> 5);
+    float4 a[2][NB], bb[2][NB];
+#pragma unroll
+    for (int u = 0; u < NB; u++) {
+        a[0][u] = pa[2 * (b_begin + u)];
+        bb[0][u] = has_b ? pb[2 * (b_begin + u)] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll 1
+    for (int b = b_begin; b < b_end; b += 2 * NB) {
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int nb = b + (half + 1) * NB; // first block of the batch after this one
+            if (nb < b_end) {
+#pragma unroll
+                for (int u = 0; u < NB; u++) {
+                    a[half ^ 1][u] = pa[2 * (nb + u)];
+                    if (has_b) bb[half ^ 1][u] = pb[2 * (nb + u)];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < NB; u++) {
+                const float4 x = a[half][u], y = bb[half][u];
+                acc00 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, x.x, acc00, 0, 0, 0);
+                acc00 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, x.y, acc00, 0, 0, 0);
+                acc00 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, x.z, acc00, 0, 0, 0);
+                acc00 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, x.w, acc00, 0, 0, 0);
+                if (has_b) {
+                    acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, y.x, acc01, 0, 0, 0);
+                    acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, y.y, acc01, 0, 0, 0);
+                    acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, y.z, acc01, 0, 0, 0);
+                    acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, y.w, acc01, 0, 0, 0);
+                    acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.x, y.x, acc11, 0, 0, 0);
+                    acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.y, y.y, acc11, 0, 0, 0);
+                    acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.z, y.z, acc11, 0, 0, 0);
+                    acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.w, y.w, acc11, 0, 0, 0);
+                }
+            }
+        }
+    }
+}
+
 __device__ __forceinline__ void gram_dense_store(float* G, int tile, int lane, const floatx16& acc, float dense_mul, bool add) {
     const int ti = tile >> 1, tj = tile & 1;
 #pragma unroll

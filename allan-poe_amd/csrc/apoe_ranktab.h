@@ -4,7 +4,9 @@
 //
 //   word[w] = (bits, count of set bits in words before w)      one ds_read_b64 per look-up
 //   slot of a term = count + popcount(bits below its bit)      no hashing, no probe loop, no key compare
-//   vals[slot] = one value per pivot of the group (zero where the pivot lacks the term): two ds_read_b128
+//   vals[slot], vals[slot_cap + slot] = one value per pivot of the group (zero where the pivot lacks the term), pivots 0-3 and
+//   4-7 in two planes: two ds_read_b128 whose 64 lanes spread over all LDS banks (side by side, a read would touch every second
+//   16-byte unit only)
 //
 // A corpus in the narrow pair format (term ids below 65536, the path known from the position in the row)
 // maps a term to bit (term | path * span) with span = the power of two above the largest term id: distinct
@@ -39,7 +41,7 @@ struct RankTabLds { // byte offsets inside the table region
 struct RankTab {
     uint2* word;      // [index_bits / 32]
     uint32_t* keys;   // [slot_cap], wide only
-    float4* vals;     // [slot_cap][RT_T / 4]
+    float4* vals;     // [RT_T / 4][slot_cap]: plane h holds pivots 4h .. 4h + 3 of every slot
     uint32_t* ovf_key;
     float4* ovf_val;
     uint32_t index_bits, slot_cap;
@@ -109,12 +111,17 @@ __device__ __forceinline__ uint32_t ranktab_build_each(const RankTab& T, EachFn 
         atomicOr(&T.word[idx >> 5].x, 1u << (idx & 31));
     });
     __syncthreads();
-    // 2. running counts: thread i owns the words [i * per, (i + 1) * per)
-    const uint32_t per = (W + nthreads - 1) / nthreads;
+    // 2. running counts: thread i owns the words [i * per, (i + 1) * per), per even: read and written two words
+    // (16 bytes) at a time, which spreads a wave's accesses over half of the LDS banks instead of four of them
+    const uint32_t per = ((W + nthreads - 1) / nthreads + 1) & ~1u;
+    uint4* word2 = reinterpret_cast<uint4*>(T.word);
     uint32_t mine = 0;
-    for (uint32_t k = 0; k < per; k++) {
+    for (uint32_t k = 0; k < per; k += 2) {
         const uint32_t w = tid * per + k;
-        if (w < W) mine += __popc(T.word[w].x);
+        if (w < W) {
+            const uint4 two = word2[w >> 1];
+            mine += __popc(two.x) + __popc(two.z);
+        }
     }
     uint32_t incl = mine;
 #pragma unroll
@@ -134,14 +141,21 @@ __device__ __forceinline__ uint32_t ranktab_build_each(const RankTab& T, EachFn 
         __syncthreads();
         return EMPTY;
     }
-    for (uint32_t k = 0; k < per; k++) {
+    for (uint32_t k = 0; k < per; k += 2) {
         const uint32_t w = tid * per + k;
         if (w < W) {
-            T.word[w].y = before;
-            before += __popc(T.word[w].x);
+            uint4 two = word2[w >> 1];
+            two.y = before;
+            before += __popc(two.x);
+            two.w = before;
+            before += __popc(two.z);
+            word2[w >> 1] = two;
         }
     }
-    for (uint32_t s = tid; s < total * (RT_T / 4); s += nthreads) T.vals[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t s = tid; s < total; s += nthreads) {
+        T.vals[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+        T.vals[T.slot_cap + s] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     if (!NARROW) {
         for (uint32_t s = tid; s < total; s += nthreads) T.keys[s] = EMPTY;
         for (uint32_t s = tid; s < RT_OVF; s += nthreads) T.ovf_key[s] = EMPTY;
@@ -154,11 +168,11 @@ __device__ __forceinline__ uint32_t ranktab_build_each(const RankTab& T, EachFn 
         const uint2 w = T.word[idx >> 5];
         const uint32_t slot = w.y + __popc(w.x & ((1u << (idx & 31)) - 1u));
         if (NARROW) {
-            reinterpret_cast<uint32_t*>(T.vals)[slot * RT_T + t] = kv.y;
+            reinterpret_cast<uint32_t*>(T.vals)[((t >> 2) * T.slot_cap + slot) * 4 + (t & 3)] = kv.y;
         } else {
             const uint32_t old = atomicCAS(&T.keys[slot], EMPTY, kv.x);
             if (old == EMPTY || old == kv.x) {
-                reinterpret_cast<uint32_t*>(T.vals)[slot * RT_T + t] = kv.y;
+                reinterpret_cast<uint32_t*>(T.vals)[((t >> 2) * T.slot_cap + slot) * 4 + (t & 3)] = kv.y;
             } else { // another term of the group sits on this bit
                 uint32_t at = EMPTY;
                 for (uint32_t s = 0; s < RT_OVF; s++) {
@@ -364,8 +378,8 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
             for (int c = 0; c < 2; c++) {
                 const bool in = rt_pair(h + c, lane) < nnz;
                 p[r][c] = ranktab_locate<NARROW>(T, w[r][h + c], index_of(r, h + c), rows[r].v[h + c], in);
-                lo[r][c] = T.vals[2 * p[r][c].slot];
-                hi[r][c] = T.vals[2 * p[r][c].slot + 1];
+                lo[r][c] = T.vals[p[r][c].slot];
+                hi[r][c] = T.vals[T.slot_cap + p[r][c].slot];
                 ok[r][c] = true;
                 if (!NARROW) ok[r][c] = p[r][c].mul == 0.f || T.keys[p[r][c].slot] == rows[r].key(h + c);
             }
@@ -396,7 +410,7 @@ __device__ __forceinline__ void ranktab_probe_rows(const RankTab& T, const RtRow
                 const uint32_t ix = ranktab_index<NARROW>(T, kv.x, NARROW ? j >= ns : (int)kv.x < 0);
                 const uint2 ww = T.word[in ? ix >> 5 : 0u];
                 const RankProbe q = ranktab_locate<NARROW>(T, ww, ix, kv.y, in);
-                const float4 vl = T.vals[2 * q.slot], vh = T.vals[2 * q.slot + 1];
+                const float4 vl = T.vals[q.slot], vh = T.vals[T.slot_cap + q.slot];
                 bool good = true;
                 if (!NARROW) good = q.mul == 0.f || T.keys[q.slot] == kv.x;
                 add8(r, good ? q.mul : 0.f, vl, vh);

@@ -246,6 +246,9 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
 #else
 #define TICK(k)
 #endif
+#ifndef APOE_PRUNE_DENSE_NB
+#define APOE_PRUNE_DENSE_NB 2
+#endif
 constexpr int GRAM_THREADS = 512; // 8 waves share one node's tables: more lookups in flight per byte of LDS
 
 struct GramPruneLds {
@@ -519,19 +522,13 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     __syncthreads();
     TICK(1);
     // hybrid Gram matrix of the m rows. Only the upper triangle of G is used (the sparse part is added there and the
-    // lower triangle is mirrored from it at the end), so the lower left tile is not computed. The eight waves share
-    // the three tiles by the bytes they read: each diagonal tile (one operand) goes to two waves, half of the
-    // dimensions each, the upper right tile (two operands) to four waves, a quarter of the dimensions each. Partial
-    // sums are added into G in a fixed order (barriers between them): the result does not depend on timing.
+    // lower triangle is mirrored from it at the end). Every wave takes an eighth of the dimensions and computes the
+    // three upper tiles for it from one read of the rows; the partial tiles are added into G in a fixed order
+    // (barriers between them): the result does not depend on timing.
     constexpr int NWAVES = NT / WAVE, BLOCKS = DIM / 8;
-    static_assert(NWAVES == 8, "the dense tiles are dealt out to eight waves");
-    const int dtile = wave < 2 ? 0 : wave < 4 ? 3 : 1, dparts = wave < 4 ? 2 : 4, dpart = wave < 4 ? (wave & 1) : wave - 4;
-    bool dactive = false;
-    floatx16 dacc;
-    if (m > 0) {
-        if (wave < 4) dacc = gram_dense_tile<true>(C, nb_id, m, dtile, lane, dpart * (BLOCKS / dparts), (dpart + 1) * (BLOCKS / dparts), dactive);
-        else dacc = gram_dense_tile<false>(C, nb_id, m, dtile, lane, dpart * (BLOCKS / dparts), (dpart + 1) * (BLOCKS / dparts), dactive);
-    }
+    static_assert(NWAVES == 8, "dimensions and rows are dealt out to eight waves");
+    floatx16 dacc00, dacc01, dacc11;
+    gram_dense_upper<APOE_PRUNE_DENSE_NB>(C, nb_id, m, lane, wave * (BLOCKS / NWAVES), (wave + 1) * (BLOCKS / NWAVES), dacc00, dacc01, dacc11);
     TICK(7);
     // this wave's rows w, w + 8, ...: requested as soon as the wave's dense tile is done (its operands need the registers), used from the keyword masks on
     static_assert(NT / WAVE == 8 || NT / WAVE == 4, "rows are dealt out to eight waves");
@@ -555,9 +552,15 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (uint32_t j = 0; j < m; j++) r += ((det[j] << 16) | j) < key;
         order[r] = i;
     }
-    for (int ph = 0; ph < 4; ph++) {
-        if (dactive && dpart == ph) gram_dense_store(G, dtile, lane, dacc, dense_mul, ph != 0);
-        if (ph < 3) __syncthreads();
+    for (int ph = 0; ph < NWAVES; ph++) {
+        if (wave == ph && m > 0) {
+            gram_dense_store(G, 0, lane, dacc00, dense_mul, ph != 0);
+            if (m > 32) {
+                gram_dense_store(G, 1, lane, dacc01, dense_mul, ph != 0);
+                gram_dense_store(G, 3, lane, dacc11, dense_mul, ph != 0);
+            }
+        }
+        if (ph + 1 < NWAVES) __syncthreads();
     }
     if (rank) {
 #pragma unroll
