@@ -833,7 +833,6 @@ int launch_prune(apoe_knn* g, uint32_t degree) {
             fit = std::min(fit, (RT_T * longest + 63) & ~63u);
             if (fit >= std::max(longest, 64u)) rank_slots = fit;
         }
-        if (getenv("APOE_PRUNE_NO_RANK")) rank_slots = 0;
     }
     const GramPruneLds GL(gram_slots, tgroup, uset_slots, map_slots, words, union_slots, rank_bits, rank_slots, narrow);
     if (g->K == GRAM_ROWS && GL.total <= lds_budget && !g->force_sequential_prune) {
