@@ -62,13 +62,17 @@ def test_pair_distances_with_heavy_pivots_and_candidates(heavy_world):
     assert_dist_close(got, O.distance_pairs(w["C"], 7.0, a, b), "pairs with heavy rows")
 
 
-def test_nn_descent_stores_the_metric(heavy_world):
-    """Every stored distance is the metric of that pair: heavy pivots go through the overflow list of the
-    four-entry bucket table, heavy candidates through the loop over more than 192 pairs."""
+@pytest.mark.parametrize("join", [0, 1, 2])
+def test_nn_descent_stores_the_metric(heavy_world, join):
+    """Every stored distance is the metric of that pair. Expansion step: heavy pivots go through the overflow list of
+    the four-entry bucket table, heavy candidates through the loop over more than 192 pairs. Join tiles: a heavy row
+    among the pickers makes the rank table take its group in passes of fewer pivots, a heavy column is read beyond
+    the register window of 256 pairs."""
     import apoe
     import oracle as O
     w = heavy_world
     knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+    knn.set_join(join)
     knn.init(9)
     for it in range(4):
         knn.iterate(last=(it == 3))
