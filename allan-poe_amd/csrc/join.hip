@@ -234,13 +234,20 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
             __builtin_amdgcn_wave_barrier();
             lst[rank] = mine;
         }
-        // dense part: wave w takes the 32-column block (w & 3) over half (w >> 2) of the dimensions; the second half is
-        // added after a barrier
+        // dense part: the eight waves share the 32-column blocks that exist (1, 2 or 4 by the number of columns) and, for
+        // each block, equal parts of the dimensions (8, 4 or 2): no wave idles when a tile has few columns. The partial
+        // tiles are added into G in a fixed order, a barrier between them.
         {
-            const int blk = wave & 3, part = wave >> 2;
-            const bool active = (uint32_t)(blk * 32) < M;
+            const uint32_t nblk = M <= 32 ? 1u : M <= 64 ? 2u : 4u, parts = (uint32_t)NW / nblk;
+            const uint32_t blk = (uint32_t)wave % nblk, part = (uint32_t)wave / nblk;
+            const bool active = blk * 32 < M;
+            const uint32_t per = (DIM / 8) / parts; // 8-float blocks of the dimensions per part: 16, 32 or 64
             floatx16 acc;
-            if (active) acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, part * (DIM / 16), (part + 1) * (DIM / 16));
+            if (active) {
+                // the usual shape (more than 64 columns) with compile-time loop bounds
+                if (nblk == 4) acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, part ? DIM / 16 : 0, part ? DIM / 8 : DIM / 16);
+                else acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, (int)(part * per), (int)((part + 1) * per));
+            }
             auto store = [&](bool add) {
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
@@ -249,9 +256,10 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
                     *at = add ? *at + a.dense_mul * acc[e] : a.dense_mul * acc[e];
                 }
             };
-            if (active && part == 0) store(false);
-            __syncthreads();
-            if (active && part == 1) store(true);
+            for (uint32_t ph = 0; ph < parts; ph++) {
+                if (active && part == ph) store(ph != 0);
+                if (ph + 1 < parts) __syncthreads();
+            }
         }
         __syncthreads();
         // sparse part: groups of eight rows in the rank table, every column probes it once per group. The pairs of a
