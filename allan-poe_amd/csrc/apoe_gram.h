@@ -1,7 +1,8 @@
 // Hybrid Gram matrix of up to 64 documents, built once per workgroup in LDS:
 // dense part on the matrix cores (fp32 MFMA 32x32x2, one 32x32 tile per wave, rows read
 // straight from the packed records), sparse part by scattering a few pivot rows at a time
-// into LDS term tables that the later rows look their terms up in.
+// into LDS term tables that the later rows look their terms up in (the hashed tables below; the prune's
+// default is the rank table of apoe_ranktab.h with the rows held in registers, prune.hip).
 #pragma once
 
 #include "apoe_device.h"
@@ -21,60 +22,12 @@ __device__ unsigned long long apoe_prune_ticks[16];
 constexpr int GRAM_ROWS = 64;
 constexpr int GRAM_STRIDE = GRAM_ROWS + 1; // odd stride: column reads do not collide on LDS banks
 
-// G[i][j] (+)= dense_mul * <dense_i, dense_j> over the 8-float blocks [b_begin, b_end) of the rows, for
-// i, j < 64; rows >= m repeat row m-1 (their entries are never read). One call computes the 32x32
-// tile (tile >> 1, tile & 1); `add` says whether the tile's partial sum is stored or added (two
-// groups of four waves split the 1024 dimensions between them, the second group adds after a barrier).
+// Dense part of the Gram matrix on the matrix cores, fp32 in and out.
 // MFMA 32x32x2 operand layout: lane l feeds A[l % 32][l / 32] and B[l / 32][l % 32];
 // accumulator register v of lane l is C[8 * (v / 4) + 4 * (l / 32) + v % 4][l % 32].
 // A lane therefore streams ITS row: float4 number (2 * block + l / 32) of every 8-float block,
 // and the four components go into four consecutive MFMAs (the k order inside the sum is free).
-template <bool DIAG>
-__device__ __forceinline__ floatx16 gram_dense_tile(const CorpusView& C, const uint32_t* ids, uint32_t m, int tile, int lane, int b_begin,
-                                                    int b_end, bool& active) {
-    const int ti = tile >> 1, tj = tile & 1;
-    floatx16 acc;
-#pragma unroll
-    for (int v = 0; v < 16; v++) acc[v] = 0.f;
-    active = !((uint32_t)(ti * 32) >= m || (uint32_t)(tj * 32) >= m);
-    if (!active) return acc;
-    const uint32_t ra = min((uint32_t)(ti * 32 + (lane & 31)), m - 1), rb = min((uint32_t)(tj * 32 + (lane & 31)), m - 1);
-    const float4* pa = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[ra]]) * 16) + (lane >> 5);
-    const float4* pb = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ids[rb]]) * 16) + (lane >> 5);
-    // operands of the next batch of 8-float blocks are requested before the current batch is multiplied; a diagonal
-    // tile (DIAG: ti == tj) reads one operand only and takes batches twice as long for the same registers
-    constexpr int NB = 4, NBB = DIAG ? 1 : NB;
-    float4 a[2][NB], bb[2][NBB];
-#pragma unroll
-    for (int u = 0; u < NB; u++) {
-        a[0][u] = pa[2 * (b_begin + u)];
-        if (!DIAG) bb[0][u] = pb[2 * (b_begin + u)];
-    }
-#pragma unroll 1
-    for (int b = b_begin; b < b_end; b += 2 * NB) {
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int nb = b + (half + 1) * NB; // first block of the batch after this one
-            if (nb < b_end) {
-#pragma unroll
-                for (int u = 0; u < NB; u++) {
-                    a[half ^ 1][u] = pa[2 * (nb + u)];
-                    if (!DIAG) bb[half ^ 1][u] = pb[2 * (nb + u)];
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < NB; u++) {
-                const float4 x = a[half][u], y = DIAG ? a[half][u] : bb[half][DIAG ? 0 : u];
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, y.x, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, y.y, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, y.z, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, y.w, acc, 0, 0, 0);
-            }
-        }
-    }
-    return acc;
-}
-
+// Rows >= m repeat row m - 1 (their entries are never read).
 // The three tiles of the upper triangle at once, over the 8-float blocks [b_begin, b_end) of the rows: a wave reads
 // its slice of rows 0-31 (operand a) and of rows 32-63 (operand b) once and feeds a x a, a x b and b x b from the same
 // registers, so every dense row is read from memory exactly once per node (tile by tile each row block is read

@@ -4,8 +4,8 @@
 // each neighbour v it picks: one pivot against many rows, every row gathered for one evaluation. Here the same
 // pairs are formed the other way round: all pickers of one v are the ROWS of a tile (32 at a time), N(v) and R(v)
 // are its COLUMNS (up to 128), every row of the tile is gathered once and meets every column:
-//   dense part   32 x 128 x 1024 contraction on the matrix cores (fp32 MFMA 32x32x2; eight waves: four 32-column
-//                blocks x two halves of the dimensions)
+//   dense part   32 x 128 x 1024 contraction on the matrix cores (fp32 MFMA 32x32x2; eight waves: the 32-column
+//                blocks that exist x equal parts of the dimensions)
 //   sparse part  eight picker rows at a time in an LDS rank table that the column rows probe (apoe_ranktab.h); a
 //                wave keeps the pairs of its sixteen columns in registers, so a row is read from memory once per tile
 //   insertion    a pair closer than the row's last list entry (and not in that list) is offered to the row node
@@ -131,7 +131,7 @@ struct JoinLds {
 };
 
 // acc = <rows, cols> over the 8-float blocks [b_begin, b_end) of the dimensions for the 32 x 32 block of row ids `ra` (nr of them) and column ids
-// `cb` (nc of them); operand layout as gram_dense_tile. Rows / columns beyond the counts repeat the last one.
+// `cb` (nc of them); operand layout as gram_dense_upper (apoe_gram.h). Rows / columns beyond the counts repeat the last one.
 __device__ __forceinline__ floatx16 join_dense_block(const CorpusView& C, const uint32_t* ra, uint32_t nr, const uint32_t* cb, uint32_t nc, int lane,
                                                      int b_begin, int b_end) {
     floatx16 acc;
