@@ -742,25 +742,35 @@ __global__ __launch_bounds__(256) void final_rows_kernel(uint32_t n, uint32_t d,
     __builtin_amdgcn_wave_barrier();
     uint32_t fill = h;
     const uint32_t e0 = in_off[v], e1 = in_off[v + 1];
-    uint64_t last = 0;
-    bool first = true;
-    while (fill < 2 * h) {
-        // smallest key above the last one taken whose node is not in the first half
-        uint64_t best = ~0ull;
-        for (uint32_t e = e0 + lane; e < e1; e += WAVE) {
-            const uint64_t k = in_edges[e];
-            if (!first && k <= last) continue;
-            const uint32_t uu = (uint32_t)k;
-            bool present = false;
-            for (uint32_t j = 0; j < h; j++) present |= row[j] == uu;
-            if (!present && k < best) best = k;
+    {
+        // the h smallest (detour, source) keys among the in-edges whose source is not in the first half, in one pass:
+        // lanes 0 .. h-1 hold the best keys so far in ascending order; a chunk of 64 in-edges is tested against the
+        // largest of them first (after a few chunks almost no key passes: a node with 10^5 in-edges costs one load and
+        // one compare per 64 of them), the keys that pass are inserted one at a time
+        uint64_t best = ~0ull; // lane i: the i-th smallest key so far (lanes >= h unused)
+        for (uint32_t eb = e0; eb < e1; eb += WAVE) {
+            const uint32_t e = eb + lane;
+            uint64_t k = e < e1 ? in_edges[e] : ~0ull;
+            const uint64_t worst = readlane64(best, h - 1);
+            bool cand = k < worst;
+            if (__ballot(cand) == 0) continue;
+            if (cand) {
+                const uint32_t uu = (uint32_t)k;
+                bool present = false;
+                for (uint32_t j = 0; j < h; j++) present |= row[j] == uu;
+                cand = !present;
+            }
+            for (uint64_t rest = __ballot(cand); rest; rest &= rest - 1) {
+                const uint64_t x = readlane64(k, (uint32_t)__builtin_ctzll(rest));
+                const uint32_t pos = __popcll(__ballot(best < x)); // best is ascending: the lanes below pos keep their keys
+                if (pos >= h) continue;
+                const uint64_t up = __shfl_up(best, 1, WAVE);
+                best = (uint32_t)lane == pos ? x : (uint32_t)lane > pos ? up : best;
+            }
         }
-        best = wave_min64(best);
-        if (best == ~0ull) break;
-        if (lane == 0) row[fill] = (uint32_t)best;
-        fill++;
-        last = best;
-        first = false;
+        const uint32_t got = min((uint32_t)__popcll(__ballot(best != ~0ull && (uint32_t)lane < h)), h);
+        if ((uint32_t)lane < got) row[h + lane] = (uint32_t)best;
+        fill = h + got;
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
