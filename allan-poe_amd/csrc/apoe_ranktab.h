@@ -92,14 +92,13 @@ __device__ __forceinline__ void ranktab_pivots_load(PivotRegs& r, PivotFn pivot,
     }
 }
 
-// Builds the table from the pairs that `each` hands out: each(f) calls f(raw pair, is BM25, pivot index t < RT_T)
-// for every pair of the group that this thread is responsible for, and must hand out the same pairs every time it is
-// called (it is called twice: bits, then values). All threads of the block call this (the block size is a multiple
-// of 64, at most 1024); `scan` is LDS scratch of 20 words. Returns the number of distinct terms, or EMPTY if they
-// exceed the slot capacity or the overflow list (the table is then unusable: the caller retries with fewer pivots).
-// Ends with a barrier: the table is ready on return.
+// Bitmap and running counts of the terms that `each` hands out: each(f) calls f(raw pair, is BM25, pivot index) for
+// every pair that this thread is responsible for. All threads of the block call this (the block size is a multiple of
+// 64, at most 1024); `scan` is LDS scratch of 20 words. Returns the number of distinct terms. Does NOT end with a
+// barrier: the counts of other threads' words are readable after the caller's next one. With `cap` below the number
+// of distinct terms the counts are not written (the caller gives the table up).
 template <bool NARROW, typename EachFn>
-__device__ __forceinline__ uint32_t ranktab_build_each(const RankTab& T, EachFn each, uint32_t* scan, int tid, int nthreads) {
+__device__ __forceinline__ uint32_t ranktab_build_bits(const RankTab& T, EachFn each, uint32_t cap, uint32_t* scan, int tid, int nthreads) {
     const uint32_t W = T.index_bits / 32;
     const int lane = tid & (WAVE - 1), wave = tid / WAVE, nwaves = nthreads / WAVE;
     for (uint32_t w = tid; w < W; w += nthreads) T.word[w] = make_uint2(0u, 0u);
@@ -137,10 +136,7 @@ __device__ __forceinline__ uint32_t ranktab_build_each(const RankTab& T, EachFn 
         if (w < wave) before += s;
         total += s;
     }
-    if (total > T.slot_cap) {
-        __syncthreads();
-        return EMPTY;
-    }
+    if (total > cap) return total;
     for (uint32_t k = 0; k < per; k += 2) {
         const uint32_t w = tid * per + k;
         if (w < W) {
@@ -151,6 +147,25 @@ __device__ __forceinline__ uint32_t ranktab_build_each(const RankTab& T, EachFn 
             before += __popc(two.z);
             word2[w >> 1] = two;
         }
+    }
+    return total;
+}
+
+// Slot of a term in a table built by ranktab_build_bits, or EMPTY if the term is not in it (w = T.word[idx >> 5]).
+__device__ __forceinline__ uint32_t ranktab_slot(uint2 w, uint32_t idx) {
+    return ((w.x >> (idx & 31)) & 1u) ? w.y + __popc(w.x & ((1u << (idx & 31)) - 1u)) : EMPTY;
+}
+
+// Builds the table from the pairs that `each` hands out (as ranktab_build_bits; it is called twice: bits, then values, and
+// must hand out the same pairs both times). Returns the number of distinct terms, or EMPTY if they
+// exceed the slot capacity or the overflow list (the table is then unusable: the caller retries with fewer pivots).
+// Ends with a barrier: the table is ready on return.
+template <bool NARROW, typename EachFn>
+__device__ __forceinline__ uint32_t ranktab_build_each(const RankTab& T, EachFn each, uint32_t* scan, int tid, int nthreads) {
+    const uint32_t total = ranktab_build_bits<NARROW>(T, each, T.slot_cap, scan, tid, nthreads);
+    if (total > T.slot_cap) {
+        __syncthreads();
+        return EMPTY;
     }
     for (uint32_t s = tid; s < total; s += nthreads) {
         T.vals[s] = make_float4(0.f, 0.f, 0.f, 0.f);

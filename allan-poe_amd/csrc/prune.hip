@@ -430,7 +430,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
         if (lane == 0) ctl[PC_M] = __popcll(b);
     }
-    {   // u's BM25 terms -> index
+    if (!(NARROW && rank_slots != 0)) {   // u's BM25 terms -> index (the rank path of narrow corpora numbers them through the rank table)
         const uint64_t du = C.desc[u];
         const Pairs sp = record_pairs(C, du);
         const uint32_t ns = desc_nnz_s(du), nb = desc_nnz_b(du);
@@ -562,7 +562,50 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
         if (ph + 1 < NWAVES) __syncthreads();
     }
-    if (rank) {
+    if (rank && NARROW) {
+        // keyword masks through the rank table: u's BM25 terms alone go into the bitmap (no values), a term's slot -- its
+        // rank among them -- is its bit in the masks, and every wave looks the BM25 pairs of its rows up with one 8-byte
+        // read each: no hash collisions, no probe loop
+        const RankTab T = ranktab_at(reinterpret_cast<char*>(tabs), rank_bits, rank_slots, rank_span, NARROW);
+        const uint64_t du = C.desc[u];
+        const Pairs up = record_pairs(C, du);
+        const uint32_t ns_u = desc_nnz_s(du), nb_u = desc_nnz_b(du);
+        ranktab_build_bits<NARROW>(T, [&](auto f) {
+            for (uint32_t j = tid; j < nb_u; j += NT) f(up.raw(ns_u + j), true, 0);
+        }, ~0u, ovf_cnt, tid, NT);
+        __syncthreads();
+        auto mark_bit = [&](uint32_t r, uint2 w, uint32_t idx) {
+            const uint32_t e = ranktab_slot(w, idx);
+            if (e != EMPTY) atomicOr(&R[r * words + (e >> 5)], 1u << (e & 31));
+        };
+#pragma unroll
+        for (int k = 0; k < GR_OWN; k++) {
+            const uint32_t nnz = own_shape[k] & 0xFFFFu, ns = own_shape[k] >> 16, r = wave + 8 * k;
+            if (nnz > ns) { // wave-uniform: the row has BM25 pairs
+                uint32_t idx[RT_CHUNKS];
+                uint2 w[RT_CHUNKS];
+#pragma unroll
+                for (int c = 0; c < RT_CHUNKS; c++) {
+                    const uint32_t j = rt_pair(c, lane);
+                    idx[c] = ranktab_index<NARROW>(T, own[k].key(c), true);
+                    w[c] = T.word[j >= ns && j < nnz ? idx[c] >> 5 : 0u];
+                }
+#pragma unroll
+                for (int c = 0; c < RT_CHUNKS; c++) {
+                    const uint32_t j = rt_pair(c, lane);
+                    if (j >= ns && j < nnz) mark_bit(r, w[c], idx[c]);
+                }
+                if (nnz > RT_CHUNKS * WAVE) {
+                    Pairs sp = gram_row(C, rowptr, rownnz, r);
+                    sp.narrow = NARROW ? 1u : 0u;
+                    for (uint32_t j = max(ns, (uint32_t)(RT_CHUNKS * WAVE)) + lane; j < nnz; j += WAVE) {
+                        const uint32_t ix = ranktab_index<NARROW>(T, sp.raw(j).x, true);
+                        mark_bit(r, T.word[ix >> 5], ix);
+                    }
+                }
+            }
+        }
+    } else if (rank) {
 #pragma unroll
         for (int k = 0; k < GR_OWN; k++) {
             const uint32_t nnz = own_shape[k] & 0xFFFFu, ns = own_shape[k] >> 16, r = wave + 8 * k;
