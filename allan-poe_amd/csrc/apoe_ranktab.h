@@ -21,6 +21,20 @@ namespace apoe {
 
 #ifdef __HIPCC__
 
+// Inclusive prefix sum over the wave with DPP adds only (no LDS crossbar): four shifted adds inside each row of 16
+// lanes, then the last lane of a row is added to the row after it (row_bcast:15 for rows 1 and 3, row_bcast:31 for
+// rows 2 and 3).
+__device__ __forceinline__ uint32_t wave_scan_add_dpp(uint32_t v) {
+    int x = (int)v;
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, false); // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, false); // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, false); // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, false); // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false); // row_bcast:15 into rows 1 and 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false); // row_bcast:31 into rows 2 and 3
+    return (uint32_t)x;
+}
+
 constexpr int RT_T = 8;     // pivots per table: two float4 per term
 constexpr int RT_OVF = 32;  // overflow entries (wide corpora only)
 
@@ -122,12 +136,7 @@ __device__ __forceinline__ uint32_t ranktab_build_bits(const RankTab& T, EachFn 
             mine += __popc(two.x) + __popc(two.z);
         }
     }
-    uint32_t incl = mine;
-#pragma unroll
-    for (int o = 1; o < WAVE; o <<= 1) {
-        const uint32_t up = __shfl_up(incl, o, WAVE);
-        if (lane >= o) incl += up;
-    }
+    const uint32_t incl = wave_scan_add_dpp(mine);
     if (lane == WAVE - 1) scan[wave] = incl;
     __syncthreads();
     uint32_t before = incl - mine, total = 0;
