@@ -1,6 +1,6 @@
 // Hybrid Gram matrix of up to 64 documents, built once per workgroup in LDS:
-// dense part on the matrix cores (fp32 MFMA 32x32x2, one 32x32 tile per wave, rows read
-// straight from the packed records), sparse part by scattering a few pivot rows at a time
+// dense part on the matrix cores (fp32 MFMA 32x32x2, every wave the three upper 32x32 tiles over its
+// share of the dimensions, rows read straight from the packed records), sparse part by scattering a few pivot rows at a time
 // into LDS term tables that the later rows look their terms up in (the hashed tables below; the prune's
 // default is the rank table of apoe_ranktab.h with the rows held in registers, prune.hip).
 #pragma once
