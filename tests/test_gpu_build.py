@@ -229,6 +229,23 @@ def test_gpu_built_index_recall(gpu_world, join):
     gq.close()
 
 
+def test_prune_gives_the_same_rows_on_every_run(gpu_world):
+    """The gather-once prune adds its partial Gram tiles in a fixed order and selects with one wave: the same lists
+    give the same rows, detour counts and keyword candidates bit for bit, run after run."""
+    import apoe
+    w = gpu_world
+    outs = []
+    for _ in range(3):
+        knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
+        knn.upload(w["knn_ids"], w["knn_dist"])
+        knn.prune(32)
+        outs.append(knn.prune_download())
+        knn.close()
+    for o in outs[1:]:
+        for a, b in zip(outs[0], o):
+            assert np.array_equal(a, b)
+
+
 def test_prune_of_short_and_ragged_lists_matches_oracle(gpu_world):
     """Lists with fewer than K usable entries (distance at the empty mark, or the node itself): 0, 1, 2, 7, 8, 9,
     31, 33 and 63 neighbours. The gather-once prune deals rows out to its waves and takes pivots eight at a time,
