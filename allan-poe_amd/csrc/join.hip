@@ -166,6 +166,46 @@ __device__ __forceinline__ floatx16 join_dense_block(const CorpusView& C, const 
     return acc;
 }
 
+// The same block with the row operand staged in LDS (`A`: row r at float4 index r * JT_A_STRIDE, all 1024 dimensions):
+// the four waves that share the picker rows read them from memory once per tile instead of once each, and a wave's
+// registers hold twice as many column blocks in flight. `pb0` = the dense row of this lane's column.
+constexpr int JT_A_STRIDE = DIM / 4 + 1; // float4 per staged row: the odd stride spreads the 32 rows of a read over the LDS banks
+__device__ __forceinline__ floatx16 join_dense_block_lds(const float4* A, uint32_t nr, const float4* pb0, int lane, int b_begin, int b_end) {
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.f;
+    const uint32_t ia = min((uint32_t)(lane & 31), nr - 1);
+    const float4* pa = A + ia * JT_A_STRIDE + (lane >> 5);
+    const float4* pb = pb0 + (lane >> 5);
+    constexpr int NB = 8;
+    float4 bb[2][NB];
+#pragma unroll
+    for (int u = 0; u < NB; u++) bb[0][u] = pb[2 * (b_begin + u)];
+#pragma unroll 1
+    for (int b = b_begin; b < b_end; b += 2 * NB) {
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int cur = b + half * NB, nb = cur + NB; // first block of this batch and of the batch after it
+            if (cur >= b_end) break;
+            if (nb < b_end) {
+#pragma unroll
+                for (int u = 0; u < NB; u++) bb[half ^ 1][u] = pb[2 * (nb + u)];
+            }
+            float4 a[NB];
+#pragma unroll
+            for (int u = 0; u < NB; u++) a[u] = pa[2 * (cur + u)];
+#pragma unroll
+            for (int u = 0; u < NB; u++) {
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].x, bb[half][u].x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].y, bb[half][u].y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].z, bb[half][u].z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].w, bb[half][u].w, acc, 0, 0, 0);
+            }
+        }
+    }
+    return acc;
+}
+
 template <bool NARROW>
 __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void join_tile_kernel(JoinArgs a) {
     a.C.narrow = NARROW ? 1u : 0u;
@@ -243,10 +283,26 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
             const bool active = blk * 32 < M;
             const uint32_t per = (DIM / 8) / parts; // 8-float blocks of the dimensions per part: 16, 32 or 64
             floatx16 acc;
+            // the picker rows go through LDS when they fit the table region, which is free until the sparse part
+            const bool staged = R * (uint32_t)JT_A_STRIDE * 16u <= RankTabLds(a.index_bits, a.slot_cap, NARROW).total;
+            float4* A = reinterpret_cast<float4*>(smem + L.tab);
+            if (staged) {
+                for (uint32_t i = tid; i < R * (DIM / 4); i += JT_THREADS) {
+                    const uint32_t r = i / (DIM / 4), c = i % (DIM / 4);
+                    A[r * JT_A_STRIDE + c] = reinterpret_cast<const float4*>(rowptr[r] - DENSE_BYTES)[c];
+                }
+                __syncthreads();
+            }
             if (active) {
-                // the usual shape (more than 64 columns) with compile-time loop bounds
-                if (nblk == 4) acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, part ? DIM / 16 : 0, part ? DIM / 8 : DIM / 16);
-                else acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, (int)(part * per), (int)((part + 1) * per));
+                if (staged) {
+                    const uint32_t ib = min((uint32_t)(lane & 31), min(32u, M - blk * 32) - 1);
+                    acc = join_dense_block_lds(A, R, reinterpret_cast<const float4*>(rowptr[JT_ROWS + blk * 32 + ib] - DENSE_BYTES), lane, (int)(part * per),
+                                               (int)((part + 1) * per));
+                } else if (nblk == 4) { // the usual shape (more than 64 columns) with compile-time loop bounds
+                    acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, part ? DIM / 16 : 0, part ? DIM / 8 : DIM / 16);
+                } else {
+                    acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, (int)(part * per), (int)((part + 1) * per));
+                }
             }
             auto store = [&](bool add) {
 #pragma unroll
