@@ -53,7 +53,7 @@ PYBIND11_MODULE(hybrid_search, m) {
         "Build the hybrid index", py::arg("dense_data_path"), py::arg("sparse_data_path"), py::arg("bm25_data_path"),
         py::arg("output_graph_path"), py::arg("degree") = 32, py::arg("nnd_k") = 64, py::arg("nnd_iters") = 25,
         py::arg("dense_build_scale") = 7.0f, py::arg("seed") = 20251125ull, py::arg("device") = 0, py::arg("knn_save_path") = "",
-        py::arg("knn_load_path") = "", py::arg("half_rows") = false, py::arg("nnd_join") = 0);
+        py::arg("knn_load_path") = "", py::arg("half_rows") = false, py::arg("nnd_join") = -1);
 
     m.def(
         "search_index",

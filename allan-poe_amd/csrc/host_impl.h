@@ -31,7 +31,8 @@ struct BuildOptions {
     bool half_rows = false;
     // 0: the reference's expansion step (index.cu:156-376). 1: the same pairs as a local join around the picked
     // neighbour (rows gathered once per tile, dense part on the matrix cores). 2: the join, both endpoints updated.
-    int nnd_join = 0;
+    // -1 (default): the join (1) when the handle allows it -- K = 64 lists on fp32 rows -- else the expansion step.
+    int nnd_join = -1;
 };
 
 struct SearchOptions {
