@@ -33,6 +33,11 @@ constexpr int JT_STRIDE = JT_COLS + 1;
 constexpr int JT_SEEN = 512; // slots of the id set that removes repeated columns
 constexpr uint32_t JOIN_K = 64;
 constexpr int JOIN_PICKS = 4; // index.cu:157,171-181
+#ifndef APOE_JOIN_SLOTS
+#define APOE_JOIN_SLOTS 128
+#endif
+constexpr uint32_t JOIN_P = APOE_JOIN_SLOTS; // proposal slots per node (64 or 128): two proposals whose ids hash to one slot are one proposal, the closer one
+constexpr int JOIN_PL = JOIN_P / WAVE; // ... per lane of the wave that merges them
 constexpr int JT_BATCH = 2;   // column rows a wave probes together
 constexpr int JT_OWN = JT_COLS / (JT_THREADS / WAVE); // columns of a tile that one wave owns: their pairs stay in its registers
 
@@ -406,40 +411,77 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
     }
 }
 
-// One wave per node: its proposals (one slot per lane) merged into its list; a node whose list changed registers
+// One wave per node: its proposals (JOIN_PL slots per lane) merged into its list; a node whose list changed registers
 // with every entry of its list (as step 6 of the expansion kernel). Proposal slots are left empty.
 __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* ids, float* dist, unsigned long long* prop, unsigned long long* rev,
                                                          uint32_t* rev_cnt, unsigned long long* inserted) {
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const uint32_t u = blockIdx.x * 4 + wave;
     if (u >= n) return;
-    const size_t base = (size_t)u * JOIN_K;
-    const unsigned long long key = prop[base + lane];
-    if (__ballot(key != ~0ull) == 0) return;
-    prop[base + lane] = ~0ull;
+    const size_t base = (size_t)u * JOIN_K, pbase = (size_t)u * JOIN_P;
+    unsigned long long key[JOIN_PL];
+    bool some = false;
+#pragma unroll
+    for (int s = 0; s < JOIN_PL; s++) {
+        key[s] = prop[pbase + s * WAVE + lane];
+        some |= key[s] != ~0ull;
+    }
+    if (__ballot(some) == 0) return;
+#pragma unroll
+    for (int s = 0; s < JOIN_PL; s++) prop[pbase + s * WAVE + lane] = ~0ull;
     const uint32_t own_id = ids[base + lane];
     const float own_d = dist[base + lane];
-    const uint32_t c = (uint32_t)key;
-    bool valid = key != ~0ull && c != u && c < n;
-    for (uint32_t i = 0; i < JOIN_K; i++) valid = valid && (((uint32_t)__builtin_amdgcn_readlane((int)own_id, i) & ~FLAG) != c);
-    const uint64_t nb = __ballot(valid);
-    if (nb == 0) return;
-    const float d = join_key_dist(key);
-    // new: rank among the new ones by (distance, id), plus the old entries strictly closer (new first on ties)
-    uint32_t rank_new = 0, le_old = 0;
-    for (uint64_t rest = nb; rest; rest &= rest - 1) {
-        const uint32_t i = __builtin_ctzll(rest);
-        const unsigned long long ki = readlane64(key, i);
-        rank_new += ki < key;
-        le_old += join_key_dist(ki) <= own_d; // old entry: new ones at or below its distance go first
+    // a proposal counts if it names another node that is not in the list yet (one id always hashes to one slot: no repeats among them)
+    bool valid[JOIN_PL];
+    float d[JOIN_PL];
+#pragma unroll
+    for (int s = 0; s < JOIN_PL; s++) {
+        const uint32_t c = (uint32_t)key[s];
+        valid[s] = key[s] != ~0ull && c != u && c < n;
+        d[s] = join_key_dist(key[s]);
     }
-    for (uint32_t i = 0; i < JOIN_K; i++) rank_new += valid && readlane_f32(own_d, i) < d;
+    for (uint32_t i = 0; i < JOIN_K; i++) {
+        const uint32_t x = (uint32_t)__builtin_amdgcn_readlane((int)own_id, i) & ~FLAG;
+#pragma unroll
+        for (int s = 0; s < JOIN_PL; s++) valid[s] = valid[s] && x != (uint32_t)key[s];
+    }
+    uint64_t nb[JOIN_PL], any = 0;
+#pragma unroll
+    for (int s = 0; s < JOIN_PL; s++) { nb[s] = __ballot(valid[s]); any |= nb[s]; }
+    if (any == 0) return;
+    // new: rank among the new ones by (distance, id), plus the old entries strictly closer (new first on ties)
+    uint32_t rank_new[JOIN_PL], le_old = 0;
+#pragma unroll
+    for (int s = 0; s < JOIN_PL; s++) rank_new[s] = 0;
+#pragma unroll
+    for (int t = 0; t < JOIN_PL; t++) {
+        for (uint64_t rest = nb[t]; rest; rest &= rest - 1) {
+            const unsigned long long ki = readlane64(key[t], (uint32_t)__builtin_ctzll(rest));
+#pragma unroll
+            for (int s = 0; s < JOIN_PL; s++) rank_new[s] += ki < key[s];
+            le_old += join_key_dist(ki) <= own_d; // old entry: new ones at or below its distance go first
+        }
+    }
+    for (uint32_t i = 0; i < JOIN_K; i++) {
+        const float di = readlane_f32(own_d, i);
+#pragma unroll
+        for (int s = 0; s < JOIN_PL; s++) rank_new[s] += di < d[s];
+    }
     const uint32_t rank_old = (uint32_t)lane + le_old;
-    const bool new_in = valid && rank_new < JOIN_K, old_in = rank_old < JOIN_K;
-    const uint32_t n_ins = __popcll(__ballot(new_in));
+    const bool old_in = rank_old < JOIN_K;
+    bool new_in[JOIN_PL];
+    uint32_t n_ins = 0;
+#pragma unroll
+    for (int s = 0; s < JOIN_PL; s++) {
+        new_in[s] = valid[s] && rank_new[s] < JOIN_K;
+        n_ins += __popcll(__ballot(new_in[s]));
+    }
     if (n_ins == 0) return;
     if (old_in) { ids[base + rank_old] = own_id; dist[base + rank_old] = own_d; }
-    if (new_in) { ids[base + rank_new] = c; dist[base + rank_new] = d; }
+#pragma unroll
+    for (int s = 0; s < JOIN_PL; s++) {
+        if (new_in[s]) { ids[base + rank_new[s]] = (uint32_t)key[s]; dist[base + rank_new[s]] = d[s]; }
+    }
     if (lane == 0) atomicAdd(inserted, (unsigned long long)n_ins);
     // reverse registration (index.cu:362-372): (distance, u) in one word, slot count % K keeps the closer one beyond K
     auto reg = [&](uint32_t e, float dv) {
@@ -452,7 +494,10 @@ __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* i
         else atomicMin(at, k);
     };
     if (old_in) reg(own_id, own_d);
-    if (new_in) reg(c, d);
+#pragma unroll
+    for (int s = 0; s < JOIN_PL; s++) {
+        if (new_in[s]) reg((uint32_t)key[s], d[s]);
+    }
 }
 
 __global__ static void join_account_kernel(const unsigned long long* work, unsigned long long* counter) {
@@ -484,12 +529,12 @@ int join_alloc(apoe_knn* g) {
     APOE_TRY(g->tile_cnt.alloc(n + 1));
     APOE_TRY(g->tile_off.alloc(n + 1));
     APOE_TRY(g->tile_v.alloc(n + n * JOIN_PICKS / JT_ROWS + 1));
-    APOE_TRY(g->prop.alloc(n * JOIN_K));
+    APOE_TRY(g->prop.alloc(n * JOIN_P));
     APOE_TRY(g->join_work.alloc(4));
     size_t temp_bytes = 0;
     APOE_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, temp_bytes, g->pick_cnt.p, g->pick_off.p, (int)(n + 1), g->ctx->stream));
     APOE_TRY(g->scan_tmp.alloc(temp_bytes));
-    fill_u64_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->prop.p, (uint64_t)n * JOIN_K, ~0ull);
+    fill_u64_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->prop.p, (uint64_t)n * JOIN_P, ~0ull);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
 }
@@ -525,7 +570,7 @@ int launch_nnd_join_iterate(apoe_knn* g) {
     a.C = g->corpus->view();
     a.dense_mul = g->dense_scale * g->dense_scale;
     a.n = n;
-    a.P = JOIN_K;
+    a.P = JOIN_P;
     a.symmetric = g->join_symmetric ? 1u : 0u;
     a.ids = g->ids.p;
     a.dist = g->dist.p;

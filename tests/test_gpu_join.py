@@ -31,7 +31,7 @@ def test_first_join_step_equals_the_oracle_step(gpu_world, mode):
     ins = knn.iterate(last=True)
     ids, dist = knn.download()
     st = O.nnd_init(w["C"].n, 64, 77)
-    oins, _ = O.join_iterate(w["C"], 7.0, st, slots=64, symmetric=(mode == 2))
+    oins, _ = O.join_iterate(w["C"], 7.0, st, slots=128, symmetric=(mode == 2))
     oids = st.ids & 0x7FFFFFFF
     same = np.all(ids == oids, axis=1)
     print(f"mode {mode}: inserted {ins} (oracle {oins}); identical rows {same.mean():.4f}")
@@ -65,7 +65,7 @@ def test_join_lists_invariants_and_recall(gpu_world, exact_knn, mode):
     # list quality: against the oracle's join and against the oracle's expansion step (the reference's algorithm)
     st = O.nnd_init(n, 64, 5)
     for it in range(8):
-        O.join_iterate(C, 7.0, st, slots=64, symmetric=(mode == 2))
+        O.join_iterate(C, 7.0, st, slots=128, symmetric=(mode == 2))
         if it < 7:
             st.rev_cnt[:] = 0
     O.nnd_merge_reverse(st)
