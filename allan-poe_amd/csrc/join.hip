@@ -32,7 +32,10 @@ constexpr int JT_THREADS = 512;
 constexpr int JT_STRIDE = JT_COLS + 1;
 constexpr int JT_SEEN = 512; // slots of the id set that removes repeated columns
 constexpr uint32_t JOIN_K = 64;
-constexpr int JOIN_PICKS = 4; // index.cu:157,171-181
+#ifndef APOE_JOIN_PICKS
+#define APOE_JOIN_PICKS 4
+#endif
+constexpr int JOIN_PICKS = APOE_JOIN_PICKS; // index.cu:157,171-181
 #ifndef APOE_JOIN_SLOTS
 #define APOE_JOIN_SLOTS 128
 #endif
