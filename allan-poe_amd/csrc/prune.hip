@@ -252,7 +252,7 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
 constexpr int GRAM_THREADS = 512; // 8 waves share one node's tables: more lookups in flight per byte of LDS
 
 struct GramPruneLds {
-    uint32_t G, tabs, ovf_cnt, rowptr, rownnz, umap, R, F, idmap, nb_id, nb_dist, nrm, det, order, sel_gi, sel_live, sel_kw, o_fwd, o_det, o_kw, ctl, total;
+    uint32_t G, tabs, ovf_cnt, rowptr, rownnz, umap, R, F, idmap, nb_id, nb_dist, nrm, det, order, o_fwd, o_det, o_kw, ctl, total;
     // union_slots != 0: the table region holds one union table (apoe_gram.h) instead of tgroup pivot tables;
     // rank_slots != 0: it holds a rank table (apoe_ranktab.h) of rank_bits index bits instead
     __host__ __device__ __forceinline__ GramPruneLds(uint32_t term_slots, uint32_t tgroup, uint32_t umap_slots, uint32_t map_slots, uint32_t words,
@@ -275,9 +275,6 @@ struct GramPruneLds {
         nrm = o; o += GRAM_ROWS * 4;
         det = o; o += GRAM_ROWS * 4;
         order = o; o += GRAM_ROWS * 4;
-        sel_gi = o; o += GRAM_ROWS * 4;
-        sel_live = o; o += GRAM_ROWS * 4;
-        sel_kw = o; o += GRAM_ROWS * 4;
         o_fwd = o; o += GRAM_ROWS * 4;
         o_det = o; o += GRAM_ROWS * 4;
         o_kw = o; o += (1 + APOE_KW_CAND) * 4;
@@ -393,9 +390,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     float* nrm = reinterpret_cast<float*>(smem + L.nrm);
     uint32_t* det = reinterpret_cast<uint32_t*>(smem + L.det);
     uint32_t* order = reinterpret_cast<uint32_t*>(smem + L.order);
-    uint32_t* sel_gi = reinterpret_cast<uint32_t*>(smem + L.sel_gi);
-    uint32_t* sel_live = reinterpret_cast<uint32_t*>(smem + L.sel_live);
-    uint32_t* sel_kw = reinterpret_cast<uint32_t*>(smem + L.sel_kw);
     uint32_t* o_fwd = reinterpret_cast<uint32_t*>(smem + L.o_fwd);
     uint32_t* o_det = reinterpret_cast<uint32_t*>(smem + L.o_det);
     uint32_t* o_kw = reinterpret_cast<uint32_t*>(smem + L.o_kw);
