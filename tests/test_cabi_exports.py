@@ -45,3 +45,25 @@ def test_module_surface_matches_reference():
              "cands", "sparse_weight", "bm25_weight", "dense_weight", "kg_weight"]
     pos = [doc.index(k + ":") for k in order]
     assert pos == sorted(pos)
+
+
+def test_header_is_plain_c_and_a_c_program_links(tmp_path):
+    """include/apoe.h is the boundary a cgo / JNI / FFI binding compiles against: it must be valid C99 by itself, and a C
+    program that calls through it must link against the library and get a status code back."""
+    import subprocess
+    import apoe
+    src = tmp_path / "caller.c"
+    src.write_text('#include "apoe.h"\n'
+                   "#include <stdio.h>\n"
+                   "int main(void) {\n"
+                   "    apoe_ctx* ctx = 0;\n"
+                   "    int st = apoe_ctx_create(99, &ctx);\n"
+                   '    printf("%d %s\\n", st, apoe_last_error_string());\n'
+                   "    return st == APOE_OK;\n"
+                   "}\n")
+    exe = tmp_path / "caller"
+    libdir = os.path.dirname(apoe.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+                    "-L", libdir, "-lapoe", "-Wl,-rpath," + libdir], check=True, capture_output=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split(None, 1)
+    assert int(out[0]) < 0 and len(out[1].strip()) > 0
