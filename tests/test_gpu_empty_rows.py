@@ -96,3 +96,28 @@ def test_search_matches_oracle(holes_world):
         same = ids == oid
         assert_dist_close(dist[same], odist[same], "pool distances")
     g.close()
+
+
+def test_queries_without_pairs_match_oracle(holes_world):
+    """Queries that have no SPLADE pairs, no BM25 pairs or no sparse pairs at all (a dense-only query in a hybrid batch):
+    their LDS term tables are empty, every probe misses."""
+    import apoe
+    import apoe_synth as S
+    import oracle as O
+    w = holes_world
+    dense, s_off, s_idx, s_val, b_off, b_idx, b_val = S.to_numpy(S.queries(120, seed=73, device="cpu"))
+    q = np.arange(120)
+    s_off, s_idx, s_val = _drop_rows(s_off, s_idx, s_val, ~((q % 3 == 0) | (q % 12 == 0)))
+    b_off, b_idx, b_val = _drop_rows(b_off, b_idx, b_val, ~((q % 4 == 0) | (q % 12 == 0)))
+    queries = (dense, s_off, s_idx, s_val, b_off, b_idx, b_val)
+    Q = O.HybridSet(*queries)
+    gq = apoe.Queries(w["ctx"], *queries)
+    g = apoe.Graph(w["ctx"], w["rows"], w["entry"])
+    for w3 in ((1.0, 1.0, 1.0), (0.0, 1.0, 1.0), (1.0, 0.5, 2.0)):
+        ids, dist, _ = apoe.search(w["ctx"], w["gc"], gq, g, w3, 64)
+        oid, odist, _ = O.search(w["C"], Q, w["rows"], w["entry"], w3, 64)
+        assert assert_topk_match(ids, dist, oid, odist, 10, f"queries without pairs, weights {w3}") > 0.97
+        same = ids == oid
+        assert_dist_close(dist[same], odist[same], "pool distances")
+    g.close()
+    gq.close()
