@@ -287,7 +287,10 @@ void build_index_impl(const std::string& dense_data_path, const std::string& spa
             check(apoe_corpus_make_half_rows(h.ctx, h.corpus), "apoe_corpus_make_half_rows");
             check(apoe_knn_use_half_rows(h.knn, 1), "apoe_knn_use_half_rows");
         }
-        const int join = opt.nnd_join >= 0 ? opt.nnd_join : (opt.nnd_k == 64 && !opt.half_rows ? 1 : 0);
+        unsigned info[4] = {0, 0, 0, 0};
+        check(apoe_corpus_info(h.corpus, info), "apoe_corpus_info");
+        const bool rows_fit = info[2] + info[3] <= APOE_JOIN_MAX_ROW_TERMS; // longest SPLADE row + longest BM25 row
+        const int join = opt.nnd_join >= 0 ? opt.nnd_join : (opt.nnd_k == 64 && !opt.half_rows && rows_fit ? 1 : 0);
         if (join) check(apoe_knn_set_join(h.knn, join), "apoe_knn_set_join");
         check(apoe_nnd_init(h.knn, opt.seed), "apoe_nnd_init");
         for (unsigned it = 0; it < opt.nnd_iters; it++) check(apoe_nnd_iterate(h.knn, it + 1 == opt.nnd_iters, nullptr), "apoe_nnd_iterate");

@@ -519,7 +519,7 @@ static void join_table_shape(const apoe_corpus* c, uint32_t* index_bits, uint32_
     *span = next_pow2(std::max(c->max_term + 1, 1024u));
     *index_bits = c->narrow ? 2 * *span : 65536u;
     const uint32_t want = RT_T * (c->max_nnz_s + c->max_nnz_b);
-    *slot_cap = std::min<uint32_t>(std::max<uint32_t>((want + 63) & ~63u, 256u), 2304u);
+    *slot_cap = std::min<uint32_t>(std::max<uint32_t>((want + 63) & ~63u, 256u), (uint32_t)APOE_JOIN_MAX_ROW_TERMS);
 }
 
 int join_alloc(apoe_knn* g) {

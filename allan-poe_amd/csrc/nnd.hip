@@ -514,6 +514,9 @@ int apoe_knn_set_join(apoe_knn* g, int mode) {
     APOE_REQUIRE(g, "null argument");
     APOE_REQUIRE(mode >= 0 && mode <= 2, "join mode must be 0 (expansion step), 1 (local join) or 2 (local join, both endpoints), got %d", mode);
     APOE_REQUIRE(mode == 0 || g->K == 64, "the local-join step is built for K = 64 lists, this handle has K = %u", g->K);
+    APOE_REQUIRE(mode == 0 || g->corpus->max_nnz_s + g->corpus->max_nnz_b <= APOE_JOIN_MAX_ROW_TERMS,
+                 "the local-join step holds documents of up to %d sparse terms in its table, this corpus has rows of up to %u + %u: use the expansion step (mode 0)",
+                 APOE_JOIN_MAX_ROW_TERMS, g->corpus->max_nnz_s, g->corpus->max_nnz_b);
     g->join = mode;
     g->join_symmetric = mode == 2;
     return APOE_OK;
@@ -548,6 +551,13 @@ int apoe_nnd_iterate(apoe_knn* g, int last, uint64_t* inserted) {
         unsigned long long h = 0;
         APOE_HIP(hipMemcpy(&h, g->counter.p, sizeof(h), hipMemcpyDeviceToHost));
         *inserted = h;
+    }
+    if (g->join) { // a picker row whose terms did not fit the tile's table was evaluated without its sparse part
+        unsigned long long c3[3] = {0, 0, 0};
+        APOE_TRY(join_step_counters(g, c3));
+        if (c3[2]) g->ready = false;
+        APOE_REQUIRE_STATE(c3[2] == 0, "the local-join step could not hold the sparse terms of %llu rows in its table (too many terms share table "
+                           "slots): the lists of this handle are not valid, build again with the expansion step (apoe_knn_set_join(..., 0))", c3[2]);
     }
     return APOE_OK;
 }

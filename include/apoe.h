@@ -36,6 +36,7 @@ extern "C" {
 #define APOE_KW_SLOTS 8         /* index.cu:15 KEYEDGEFINAL: row width = degree + 8 */
 #define APOE_KW_CAND 32         /* index.cu:14 KEYEDGE */
 #define APOE_MAX_CANDS 2048     /* pool size limit (the reference stops at 512, query.cu:9) */
+#define APOE_JOIN_MAX_ROW_TERMS 2304 /* sparse terms of one document (both paths) that the local-join step's LDS table holds */
 
 typedef struct apoe_ctx apoe_ctx;
 typedef struct apoe_corpus apoe_corpus;
@@ -144,7 +145,8 @@ int apoe_knn_use_half_rows(apoe_knn* g, int on);
  *      second kernel; lists are read as the step found them (the reference reads them while they change);
  *   2  as 1, and every pair is offered to the column node as well (insertion into both endpoints' lists, as
  *      the classic NN-Descent join does; the reference's step updates the picking node only).
- * K must be 64 for 1 and 2. May be changed between steps. */
+ * K must be 64 for 1 and 2, and no document may have more than APOE_JOIN_MAX_ROW_TERMS sparse terms (longest SPLADE row +
+ * longest BM25 row): a tile keeps the terms of a picker row in an LDS table. May be changed between steps. */
 int apoe_knn_set_join(apoe_knn* g, int mode);
 /* initialize_graph + cal_power (index.cu:890-892). */
 int apoe_nnd_init(apoe_knn* g, uint64_t seed);

@@ -127,3 +127,37 @@ def test_search_matches_oracle(heavy_world, w3):
     ids2, dist2, _ = apoe.search(w["ctx"], w["gc"], w["gq"], g, w3, 64, variant=0x100)
     assert np.array_equal(ids, ids2) and np.array_equal(dist, dist2)
     g.close()
+
+
+def test_join_refuses_rows_longer_than_its_table(gpu_ctx):
+    """One document with more sparse terms than the join tile's LDS table holds (APOE_JOIN_MAX_ROW_TERMS = 2304): the
+    join is refused with a message when it is chosen, instead of evaluating that row without its sparse part."""
+    import apoe
+    import apoe_synth as S
+    n = 200
+    dense, s_off, s_idx, s_val, b_off, b_idx, b_val = S.to_numpy(S.corpus(n, seed=63, device="cpu"))
+    rng = np.random.default_rng(9)
+
+    def with_long_row(off, idx, val, row, terms):
+        cnt = np.diff(off.astype(np.int64))
+        keep = np.repeat(np.arange(n) != row, cnt)
+        new_i = np.sort(rng.choice(30000, terms, replace=False)).astype(np.uint32)
+        new_v = rng.uniform(0.5, 2.0, terms).astype(np.float32)
+        at = int(off[row] - 0)  # rows before `row` keep their place; its pairs are replaced
+        i2, v2 = idx[keep], val[keep]
+        i2 = np.concatenate([i2[:at], new_i, i2[at:]])
+        v2 = np.concatenate([v2[:at], new_v, v2[at:]])
+        cnt[row] = terms
+        o2 = np.zeros(n + 1, np.uint32)
+        o2[1:] = np.cumsum(cnt)
+        return o2, i2, v2
+
+    s_off, s_idx, s_val = with_long_row(s_off, s_idx, s_val, 17, 1500)
+    b_off, b_idx, b_val = with_long_row(b_off, b_idx, b_val, 17, 900)
+    gc = apoe.Corpus(gpu_ctx, dense, s_off, s_idx, s_val, b_off, b_idx, b_val)
+    assert gc.info()[2] + gc.info()[3] > 2304
+    knn = apoe.Knn(gpu_ctx, gc, 64, 7.0)
+    with pytest.raises(RuntimeError, match="expansion step"):
+        knn.set_join(1)
+    knn.close()
+    gc.close()
