@@ -937,16 +937,26 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     const SearchLds L(a.slots_s, a.slots_b, a.ovf_cap, a.cands, mode, a.kw_slots);
     APOE_REQUIRE(L.total <= 64 * 1024, "search needs %u bytes of LDS (query rows with up to %u sparse terms)", L.total, q->max_nnz);
 
-    // variant 0: two waves per query (the measured best); 1, 2, 3: one, four, eight waves
+    // variant 0: two waves per query (the measured best up to pools of 1024; four for larger ones, below); 1, 2, 3: one, four, eight waves
     int nw = 2;
     const uint32_t shape = p->variant & 0xFFu;
     if (shape == 1) nw = 1;
     else if (shape == 2) nw = 4;
     else if (shape == 3) nw = 8;
+    else APOE_REQUIRE(shape == 0 || shape == 4, "launch shape %u is not one of 0 (default), 1, 2, 3, 4 (one, four, eight, two waves per query)", shape);
     // persistent grid: as many workgroups as can be resident, never more than queries
     int per_cu = 1;
     APOE_TRY(launch_mode(ctx, mode, nw, a, 0, L.total, &per_cu));
     if (per_cu < 1) per_cu = 1;
+    if (shape == 0 && per_cu <= 8 && mode != MODE_KEYWORD) { // (the keyword search measures the same or worse with four: it stays at two)
+        // a pool so large that LDS, not registers, limits the resident queries (8 or fewer per CU: 16 waves): with four
+        // waves per query the same queries keep twice the loads in flight (1 M docs: 167 against 191 ms at cands 1500,
+        // 234 against 290 ms at 2048; the same at 1024, where 9 queries fit; knowledge-graph search: 66 against 77 ms at
+        // cands 512, 150 against 195 ms at 1024)
+        int per_cu4 = 0;
+        APOE_TRY(launch_mode(ctx, mode, 4, a, 0, L.total, &per_cu4));
+        if (per_cu4 * 4 > per_cu * 2) { nw = 4; per_cu = per_cu4; } // more waves on the CU than with two per query
+    }
     uint32_t grid = std::min<uint32_t>(q_count, (uint32_t)per_cu * (uint32_t)ctx->num_cus);
 
     a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;

@@ -187,8 +187,10 @@ typedef struct {
     uint32_t cands;                  /* pool size, 1..APOE_MAX_CANDS */
     uint32_t max_iter;               /* 0 -> 1000 (query.cu:7 MAX_ITER) */
     uint32_t q_begin, q_count;       /* query range; q_count 0 -> all from q_begin */
-    uint32_t variant;                /* low byte: launch shape, 0 = default (2 waves per query), 1/2/3 =
-                                        1/4/8 waves. 0x100: read the dense row of every candidate; by
+    uint32_t variant;                /* low byte: launch shape, 0 = default (2 waves per query; 4 when the pool is so
+                                        large that fewer than 9 queries fit a CU, plain and KG search), 1/2/3 =
+                                        1/4/8 waves, 4 = 2 waves whatever the pool; other values are refused.
+                                        0x100: read the dense row of every candidate; by
                                         default a candidate whose sparse part plus the Cauchy-Schwarz
                                         bound of its dense part cannot beat the worst entry of the full
                                         pool is dropped without reading its dense row (same results).

@@ -7,7 +7,7 @@ from parity import assert_dist_close, assert_topk_match, recall_at_k
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("cands", [32, 128])
 def test_search_matches_oracle(gpu_world, cands, variant):
     import apoe
@@ -107,3 +107,16 @@ def test_pool_sizes_at_the_edges(gpu_world, cands):
     if cands == 2048:
         with pytest.raises(apoe.ApoeError, match="cands"):
             apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], (1, 1, 1), cands + 1, q_count=nq)
+
+
+def test_large_pool_picks_its_shape_and_unknown_shapes_are_refused(gpu_world):
+    """With the default shape a pool of 2048 entries runs with four waves per query (fewer queries fit a CU): the rows
+    are those of the two-wave launch. A shape code that does not exist is an error, not a silent default."""
+    import apoe
+    w = gpu_world
+    a = apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], (1.0, 1.0, 1.0), 2048, max_iter=4096, variant=0)
+    b = apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], (1.0, 1.0, 1.0), 2048, max_iter=4096, variant=4)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    assert a[2].evaluations == b[2].evaluations
+    with pytest.raises(RuntimeError, match="launch shape"):
+        apoe.search(w["ctx"], w["gc"], w["gq"], w["gg"], (1.0, 1.0, 1.0), 32, variant=9)
