@@ -937,40 +937,56 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     const SearchLds L(a.slots_s, a.slots_b, a.ovf_cap, a.cands, mode, a.kw_slots);
     APOE_REQUIRE(L.total <= 64 * 1024, "search needs %u bytes of LDS (query rows with up to %u sparse terms)", L.total, q->max_nnz);
 
-    // variant 0: two waves per query (the measured best up to pools of 1024; four for larger ones, below); 1, 2, 3: one, four, eight waves
+    a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;
+    // workspace: [counters: 8 x u64][once-per-query arguments][visited bitmaps]
+    const size_t cold_at = 8 * sizeof(unsigned long long), bitmaps_at = (cold_at + sizeof(SearchCold) + 255) & ~(size_t)255;
+    const size_t bitmap_bytes = (size_t)a.bitmap_words * sizeof(uint32_t);
+    size_t fit = SIZE_MAX; // workgroups whose visited bitmaps fit the workspace
+    if (static_ws) {
+        fit = (APOE_NOALLOC_WS_BYTES - bitmaps_at) / bitmap_bytes;
+        APOE_REQUIRE(fit >= 1, "the static workspace of %u bytes holds no visited bitmap of %zu bytes", (unsigned)APOE_NOALLOC_WS_BYTES, bitmap_bytes);
+    }
+
+    // Launch shape (waves per query). 1, 2, 3, 4: one, four, eight, two waves, as the caller says. 0, the default:
+    //  * a batch that is resident all at once is bound by the time of ONE query, and that falls with the waves it has
+    //    (alone, cands 256: 4.2 / 2.9 / 2.2 ms with 2 / 4 / 8 waves): eight waves while all queries still fit the
+    //    machine that way (768 at 3 per CU), else four while they fit (1 536), e.g. 100 queries at cands 256 in 3.4
+    //    instead of 7.9 ms, 1 024 in 5.6 instead of 8.8 ms; four also for batches of up to two rounds of the two-wave
+    //    grid (6 144 queries), whose second round ends sooner that way (4-9 % at 4 096 to 6 144 queries, cands 64-512);
+    //  * a longer batch is bound by the memory system and runs best with two waves per query and as many queries as fit
+    //    (12 per CU) - unless the pool is so large that LDS leaves room for at most 8 queries on a CU: then four waves
+    //    per query keep twice the loads in flight (1 M docs: 167 against 191 ms at cands 1500, 234 against 290 ms at
+    //    2048, the same at 1024, where 9 queries fit; knowledge-graph search: 66 against 77 ms at cands 512, 150
+    //    against 195 ms at 1024; the keyword search measures the same or worse with four and stays at two).
     int nw = 2;
     const uint32_t shape = p->variant & 0xFFu;
     if (shape == 1) nw = 1;
     else if (shape == 2) nw = 4;
     else if (shape == 3) nw = 8;
     else APOE_REQUIRE(shape == 0 || shape == 4, "launch shape %u is not one of 0 (default), 1, 2, 3, 4 (one, four, eight, two waves per query)", shape);
-    // persistent grid: as many workgroups as can be resident, never more than queries
+    auto resident_per_cu = [&](int waves, int* out) -> int {
+        *out = 1;
+        APOE_TRY(launch_mode(ctx, mode, waves, a, 0, L.total, out));
+        if (*out < 1) *out = 1;
+        return APOE_OK;
+    };
     int per_cu = 1;
-    APOE_TRY(launch_mode(ctx, mode, nw, a, 0, L.total, &per_cu));
-    if (per_cu < 1) per_cu = 1;
-    if (shape == 0 && per_cu <= 8 && mode != MODE_KEYWORD) { // (the keyword search measures the same or worse with four: it stays at two)
-        // a pool so large that LDS, not registers, limits the resident queries (8 or fewer per CU: 16 waves): with four
-        // waves per query the same queries keep twice the loads in flight (1 M docs: 167 against 191 ms at cands 1500,
-        // 234 against 290 ms at 2048; the same at 1024, where 9 queries fit; knowledge-graph search: 66 against 77 ms at
-        // cands 512, 150 against 195 ms at 1024)
-        int per_cu4 = 0;
-        APOE_TRY(launch_mode(ctx, mode, 4, a, 0, L.total, &per_cu4));
-        if (per_cu4 * 4 > per_cu * 2) { nw = 4; per_cu = per_cu4; } // more waves on the CU than with two per query
-    }
-    uint32_t grid = std::min<uint32_t>(q_count, (uint32_t)per_cu * (uint32_t)ctx->num_cus);
-
-    a.bitmap_words = ((c->n + 31) / 32 + 3) & ~3u;
-    // workspace: [counters: 8 x u64][once-per-query arguments][visited bitmaps]
-    const size_t cold_at = 8 * sizeof(unsigned long long), bitmaps_at = (cold_at + sizeof(SearchCold) + 255) & ~(size_t)255;
-    const size_t bitmap_bytes = (size_t)a.bitmap_words * sizeof(uint32_t);
-    char* ws = static_ws;
-    if (static_ws) {
-        const size_t fit = (APOE_NOALLOC_WS_BYTES - bitmaps_at) / bitmap_bytes;
-        APOE_REQUIRE(fit >= 1, "the static workspace of %u bytes holds no visited bitmap of %zu bytes", (unsigned)APOE_NOALLOC_WS_BYTES, bitmap_bytes);
-        grid = (uint32_t)std::min<size_t>(grid, fit);
+    if (shape == 0) {
+        const size_t at_once = std::min<size_t>(q_count, fit); // queries in flight if every one of them had a workgroup
+        int pc8 = 1, pc4 = 1;
+        APOE_TRY(resident_per_cu(8, &pc8));
+        APOE_TRY(resident_per_cu(4, &pc4));
+        APOE_TRY(resident_per_cu(2, &per_cu));
+        if (at_once <= (size_t)pc8 * ctx->num_cus) { nw = 8; per_cu = pc8; }
+        else if (at_once <= (size_t)pc4 * ctx->num_cus || at_once <= 2 * (size_t)per_cu * ctx->num_cus) { nw = 4; per_cu = pc4; }
+        else if (per_cu <= 8 && mode != MODE_KEYWORD && pc4 * 4 > per_cu * 2) { nw = 4; per_cu = pc4; }
     } else {
-        APOE_TRY(ctx->search_workspace(bitmaps_at + (size_t)grid * bitmap_bytes, &ws));
+        APOE_TRY(resident_per_cu(nw, &per_cu));
     }
+    // persistent grid: as many workgroups as can be resident, never more than queries or bitmaps
+    const uint32_t grid = (uint32_t)std::min<size_t>(std::min<size_t>(q_count, fit), (size_t)per_cu * (size_t)ctx->num_cus);
+    char* ws = static_ws;
+    if (!static_ws) APOE_TRY(ctx->search_workspace(bitmaps_at + (size_t)grid * bitmap_bytes, &ws));
     unsigned long long* work = reinterpret_cast<unsigned long long*>(ws);
     search_setup_kernel<<<1, WAVE, 0, ctx->stream>>>(work, reinterpret_cast<SearchCold*>(ws + cold_at), cold);
     APOE_HIP(hipGetLastError());
