@@ -248,6 +248,18 @@ def main():
         log(f"[bench] KG search cands 128: {sk.kernel_ms:.2f} ms, entity document in the top 10 for {hits / nq_truth:.3f} of the queries")
         gkg.close()
 
+    # ---- short batches: the launch shape follows the batch (more waves per query while the whole batch is resident at once) ----
+    short_batches = None
+    if not args.no_sweeps:
+        short_batches = []
+        for nq_short in (1, 100, 1000):
+            if nq_short > args.queries:
+                continue
+            apoe.search(ctx, gc, gq, graph, w3, cands, q_count=nq_short)
+            ms_short = min(apoe.search(ctx, gc, gq, graph, w3, cands, q_count=nq_short)[2].kernel_ms for _ in range(3))
+            short_batches.append(dict(queries=nq_short, cands=cands, kernel_ms=ms_short, qps=nq_short / (ms_short / 1e3)))
+            log(f"[bench] {nq_short} queries at cands {cands}: {ms_short:.2f} ms")
+
     # ---- where the recall target IS reached: the same generators, build and search on smaller corpora ----
     smaller = None
     if not args.no_sweeps:
@@ -429,6 +441,7 @@ def main():
             "kernel_ms": avg_kernel_ms,
             **({"weight_sweep_without_rebuild": weight_sweep} if weight_sweep else {}),
             **({"knowledge_graph_search": kg_search} if kg_search else {}),
+            **({"short_batches": short_batches} if short_batches else {}),
             **({"same_generators_smaller_corpora": smaller} if smaller else {}),
             **({"extras": extras} if extras else {}),
         },
