@@ -41,6 +41,7 @@ constexpr int JOIN_PICKS = APOE_JOIN_PICKS; // index.cu:157,171-181
 #endif
 constexpr uint32_t JOIN_P = APOE_JOIN_SLOTS; // proposal slots per node (64 or 128): two proposals whose ids hash to one slot are one proposal, the closer one
 constexpr int JOIN_PL = JOIN_P / WAVE; // ... per lane of the wave that merges them
+constexpr int JOIN_COUNT_PARTS = 256, JOIN_COUNT_AT = 8; // partial insertion counters in the step's work array, one per 64-byte line, from word 8
 constexpr int JT_BATCH = 2;   // column rows a wave probes together
 constexpr int JT_OWN = JT_COLS / (JT_THREADS / WAVE); // columns of a tile that one wave owns: their pairs stay in its registers
 
@@ -236,6 +237,7 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
     constexpr int NW = JT_THREADS / WAVE;
     const uint32_t n_tiles = a.tile_off[a.n];
 
+    if (tid == 0) { ctl[2] = 0; ctl[3] = 0; } // pairs and rows of this workgroup's tiles
     while (true) {
         __syncthreads();
         if (tid == 0) { ctl[0] = (uint32_t)atomicAdd(a.work, 1ull); ctl[1] = 0; }
@@ -407,10 +409,15 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
             }
             if (d < col_worst[c]) atomicMin(&a.prop[(size_t)cid * a.P + prop_slot(uid, a.P)], dist_id_key(d, uid));
         }
-        if (tid == 0) {
-            atomicAdd(a.work + 1, (unsigned long long)R * M);
-            atomicAdd(a.work + 2, (unsigned long long)(R + M));
+        if (tid == 0) { // summed here, sent once when the workgroup leaves: a million atomics on one address per step would queue up
+            ctl[2] += R * M;
+            ctl[3] += R + M;
+            if (ctl[2] >= 0x40000000u) { atomicAdd(a.work + 1, (unsigned long long)ctl[2]); ctl[2] = 0; }
         }
+    }
+    if (tid == 0) {
+        atomicAdd(a.work + 1, (unsigned long long)ctl[2]);
+        atomicAdd(a.work + 2, (unsigned long long)ctl[3]);
     }
 }
 
@@ -485,7 +492,7 @@ __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* i
     for (int s = 0; s < JOIN_PL; s++) {
         if (new_in[s]) { ids[base + rank_new[s]] = (uint32_t)key[s]; dist[base + rank_new[s]] = d[s]; }
     }
-    if (lane == 0) atomicAdd(inserted, (unsigned long long)n_ins);
+    if (lane == 0) atomicAdd(inserted + (blockIdx.x % JOIN_COUNT_PARTS) * 8, (unsigned long long)n_ins); // one address for every node would serialise a million atomics
     // reverse registration (index.cu:362-372): (distance, u) in one word, slot count % K keeps the closer one beyond K
     auto reg = [&](uint32_t e, float dv) {
         const uint32_t v = e & ~FLAG;
@@ -503,9 +510,12 @@ __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* i
     }
 }
 
-__global__ static void join_account_kernel(const unsigned long long* work, unsigned long long* counter) {
+__global__ static void join_account_kernel(unsigned long long* work, unsigned long long* counter) {
     counter[2] += work[1]; // pairs evaluated
     counter[3] += work[2]; // rows gathered (each read in full, dense part included)
+    unsigned long long inserted = 0; // the partial counts of join_apply_kernel
+    for (int p = 0; p < JOIN_COUNT_PARTS; p++) inserted += work[JOIN_COUNT_AT + p * 8];
+    counter[0] = inserted;
 }
 
 __global__ __launch_bounds__(256) static void fill_u64_kernel(unsigned long long* p, uint64_t count, unsigned long long v) {
@@ -533,7 +543,7 @@ int join_alloc(apoe_knn* g) {
     APOE_TRY(g->tile_off.alloc(n + 1));
     APOE_TRY(g->tile_v.alloc(n + n * JOIN_PICKS / JT_ROWS + 1));
     APOE_TRY(g->prop.alloc(n * JOIN_P));
-    APOE_TRY(g->join_work.alloc(4));
+    APOE_TRY(g->join_work.alloc(JOIN_COUNT_AT + JOIN_COUNT_PARTS * 8));
     size_t temp_bytes = 0;
     APOE_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, temp_bytes, g->pick_cnt.p, g->pick_off.p, (int)(n + 1), g->ctx->stream));
     APOE_TRY(g->scan_tmp.alloc(temp_bytes));
@@ -556,7 +566,7 @@ int launch_nnd_join_iterate(apoe_knn* g) {
     APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), st)); // [0] inserted; [2], [3] accumulate over the build
     fill_u32_kernel2<<<1024, 256, 0, st>>>(g->pick_cnt.p, (uint64_t)n + 1, 0u);
     fill_u32_kernel2<<<1024, 256, 0, st>>>(g->pick_fill.p, (uint64_t)n + 1, 0u);
-    fill_u64_kernel<<<1, 64, 0, st>>>(g->join_work.p, 4, 0ull);
+    fill_u64_kernel<<<8, 256, 0, st>>>(g->join_work.p, JOIN_COUNT_AT + JOIN_COUNT_PARTS * 8, 0ull);
     join_pick_kernel<<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->picks.p, g->pick_cnt.p);
     APOE_HIP(hipGetLastError());
     join_tile_count_kernel<<<(n + 256) / 256, 256, 0, st>>>(n, g->pick_cnt.p, g->tile_cnt.p);
@@ -594,7 +604,7 @@ int launch_nnd_join_iterate(apoe_knn* g) {
     if (per_cu < 1) per_cu = 1;
     kernel<<<(uint32_t)per_cu * (uint32_t)ctx->num_cus, JT_THREADS, L.total, st>>>(a);
     APOE_HIP(hipGetLastError());
-    join_apply_kernel<<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->dist.p, g->prop.p, g->rev.p, g->rev_cnt.p, g->counter.p);
+    join_apply_kernel<<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->dist.p, g->prop.p, g->rev.p, g->rev_cnt.p, g->join_work.p + JOIN_COUNT_AT);
     APOE_HIP(hipGetLastError());
     join_account_kernel<<<1, 1, 0, st>>>(g->join_work.p, g->counter.p);
     APOE_HIP(hipGetLastError());
