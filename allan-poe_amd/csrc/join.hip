@@ -421,8 +421,9 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
     }
 }
 
-// One wave per node: its proposals (JOIN_PL slots per lane) merged into its list; a node whose list changed registers
-// with every entry of its list (as step 6 of the expansion kernel). Proposal slots are left empty.
+// One wave per node: its proposals (JOIN_PL slots per lane) merged into its list; the entries that are new in the list register
+// with their nodes' reverse lists (index.cu:362-372 registers every entry of a changed list and starts the reverse lists again with
+// every step; the join keeps them over the steps, so an entry registers once, when it enters). Proposal slots are left empty.
 __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* ids, float* dist, unsigned long long* prop, unsigned long long* rev,
                                                          uint32_t* rev_cnt, unsigned long long* inserted) {
     const int wave = threadIdx.x / WAVE, lane = lane_id();
@@ -493,7 +494,7 @@ __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* i
         if (new_in[s]) { ids[base + rank_new[s]] = (uint32_t)key[s]; dist[base + rank_new[s]] = d[s]; }
     }
     if (lane == 0) atomicAdd(inserted + (blockIdx.x % JOIN_COUNT_PARTS) * 8, (unsigned long long)n_ins); // one address for every node would serialise a million atomics
-    // reverse registration (index.cu:362-372): (distance, u) in one word, slot count % K keeps the closer one beyond K
+    // reverse registration of the new entries: (distance, u) in one word, slot count % K keeps the closer one beyond K
     auto reg = [&](uint32_t e, float dv) {
         const uint32_t v = e & ~FLAG;
         if (v >= n) return;
@@ -503,7 +504,6 @@ __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* i
         if (slot < JOIN_K) *at = k;
         else atomicMin(at, k);
     };
-    if (old_in) reg(own_id, own_d);
 #pragma unroll
     for (int s = 0; s < JOIN_PL; s++) {
         if (new_in[s]) reg((uint32_t)key[s], d[s]);

@@ -540,7 +540,7 @@ int apoe_nnd_iterate(apoe_knn* g, int last, uint64_t* inserted) {
     float ms = 0.f;
     APOE_TRY(timed(g->ctx, &ms, [&]() -> int {
         APOE_TRY(launch_nnd_iterate(g, nullptr));
-        if (!last) { // reset_reverse_num, index.cu:896
+        if (!last && !g->join) { // reset_reverse_num, index.cu:896; the join's reverse lists grow over the steps (join_apply_kernel)
             fill_u32_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->rev_cnt.p, g->n, 0u);
             APOE_HIP(hipGetLastError());
         }

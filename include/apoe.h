@@ -142,7 +142,9 @@ int apoe_knn_use_half_rows(apoe_knn* g, int on);
  *   1  the same pairs as a local join around the picked neighbour: all pickers of a node v are the rows of a
  *      tile, N(v) and R(v) its columns, every row gathered once, the dense part of the tile on the matrix
  *      cores, survivors sent to the row nodes' lists by 64-bit atomicMin on proposal slots and merged by a
- *      second kernel; lists are read as the step found them (the reference reads them while they change);
+ *      second kernel; lists are read as the step found them (the reference reads them while they change); an
+ *      entry registers with its node's reverse list once, when it enters, and the reverse lists are kept over
+ *      the steps (the reference registers every entry of a changed list and starts them again with every step);
  *   2  as 1, and every pair is offered to the column node as well (insertion into both endpoints' lists, as
  *      the classic NN-Descent join does; the reference's step updates the picking node only).
  * K must be 64 for 1 and 2, and no document may have more than APOE_JOIN_MAX_ROW_TERMS sparse terms (longest SPLADE row +

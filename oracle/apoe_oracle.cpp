@@ -794,7 +794,8 @@ uint64_t orc_join_iterate(const orc_set* corpus, float dense_scale, uint32_t K, 
         }
     }
     if (evals) *evals += n_eval;
-    /* 3. apply; a node whose list changed registers with every entry of its list (index.cu:362-372) */
+    /* 3. apply; the entries that are new in a list register with their nodes' reverse lists, which are kept over the
+     * steps (index.cu:362-372 registers every entry of a changed list and index.cu:896 starts the lists again) */
     uint64_t inserted = 0;
 #pragma omp parallel num_threads(nthreads(threads)) reduction(+ : inserted)
     {
@@ -823,7 +824,7 @@ uint64_t orc_join_iterate(const orc_set* corpus, float dense_scale, uint32_t K, 
             if (!ins) continue;
             for (uint32_t j = 0; j < K; j++) {
                 const uint32_t v = list[j].id & ~ORC_FLAG;
-                if (v >= n) continue;
+                if (v >= n || !list[j].ent) continue;
                 const float dv = list[j].dist;
                 const uint32_t slot = __atomic_fetch_add(&rev_cnt[v], 1u, __ATOMIC_RELAXED);
                 uint32_t* at = &rev[(size_t)v * K + slot % K];

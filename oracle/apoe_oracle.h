@@ -120,7 +120,11 @@ void orc_nnd_merge_reverse(uint32_t n, uint32_t K, uint32_t* ids, float* dist, c
  * merges): the classic join's insertion into both endpoints, which the reference's step does
  * not do.
  * Then every node merges its proposals (new before old on equal distance, index.cu:333-351);
- * a node whose list changed registers with every entry of its list (index.cu:362-372).
+ * the entries that are NEW in a list register with the reverse lists of their nodes (slot
+ * count mod K, the closer one stays beyond K). The reference registers every entry of a changed
+ * list and starts the reverse lists again with every step (index.cu:362-372, :896); the join
+ * keeps the reverse lists over the steps -- the caller does not reset rev_cnt between join
+ * steps -- so an entry registers once, when it enters.
  */
 typedef struct {
     uint32_t slots;      /* proposal slots per node, a power of two */

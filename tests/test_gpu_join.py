@@ -65,9 +65,7 @@ def test_join_lists_invariants_and_recall(gpu_world, exact_knn, mode):
     # list quality: against the oracle's join and against the oracle's expansion step (the reference's algorithm)
     st = O.nnd_init(n, 64, 5)
     for it in range(8):
-        O.join_iterate(C, 7.0, st, slots=128, symmetric=(mode == 2))
-        if it < 7:
-            st.rev_cnt[:] = 0
+        O.join_iterate(C, 7.0, st, slots=128, symmetric=(mode == 2))  # the join keeps its reverse lists over the steps
     O.nnd_merge_reverse(st)
     se = O.nnd_init(n, 64, 5)
     for it in range(8):

@@ -26,11 +26,13 @@ def _world(ctx, n, nq=20):
 def _oracle_lists(C, join):
     import oracle as O
     st = O.nnd_init(C.n, 64, 3)
-    for _ in range(STEPS):
+    for it in range(STEPS):
         if join:
             O.join_iterate(C, 7.0, st, slots=128, symmetric=(join == 2))
         else:
             O.nnd_iterate(C, 7.0, st)
+            if it < STEPS - 1:
+                st.rev_cnt[:] = 0  # index.cu:896
     O.nnd_merge_reverse(st)
     return st.ids & 0x7FFFFFFF, st.dist
 
