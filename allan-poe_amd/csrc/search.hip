@@ -63,7 +63,7 @@ struct SearchArgs {
 
 // LDS carve-up shared by host (size) and device (pointers).
 struct SearchLds {
-    uint32_t qd, part, tab, ovf, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ring_id,
+    uint32_t qd, stat, part, tab, ovf, pool_id, pool_dist, pool_ent, pool_hop, new_lb, new_id, new_dist, new_ent, new_hop, seed_id, seed_ent, seed_dist, link, ring_id,
         ring_dist, kwset, ctl, total;
     __host__ __device__ SearchLds(uint32_t slots_s, uint32_t slots_b, uint32_t ovf_cap, uint32_t cands, int mode, uint32_t kw_slots) {
         const bool kg = mode == MODE_KG, kwd = mode == MODE_KEYWORD;
@@ -71,6 +71,7 @@ struct SearchLds {
         uint32_t o = 0;
         qd = o; o += DENSE_BYTES;       // the query's dense row, weight applied
         ctl = o; o += 16 * 4;
+        stat = o; o += 8 * 8;           // the workgroup's counters (work[1..7]), sent once when it leaves
         part = o; o += MAX_NEW * 16;    // sparse sum of a fresh candidate as four partial sums (one per 16 lanes)
         new_lb = o; o += MAX_NEW * 4;
         new_id = o; o += MAX_NEW * 4;
@@ -287,6 +288,8 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(MODE =
     uint32_t* bitmap = a.bitmaps + (size_t)blockIdx.x * a.bitmap_words;
     const uint64_t lane_lt = (1ull << lane) - 1;
 
+    unsigned long long* stat = reinterpret_cast<unsigned long long*>(smem + L.stat);
+    if (tid < 8) stat[tid] = 0;
     while (true) {
         __syncthreads();
         if (tid == 0) ctl[CTL_QUERY] = (uint32_t)atomicAdd(a.work, 1ull);
@@ -789,16 +792,18 @@ __global__ __launch_bounds__(NW* WAVE) __attribute__((amdgpu_waves_per_eu(MODE =
             st_ns += __shfl_xor(st_ns, o, WAVE);
             st_nb += __shfl_xor(st_nb, o, WAVE);
         }
-        if (lane == 0) {
-            if (st_exp) atomicAdd(a.work + 1, st_exp);
-            if (st_eval) atomicAdd(a.work + 2, st_eval);
-            if (st_ns) atomicAdd(a.work + 3, (unsigned long long)st_ns);
-            if (st_nb) atomicAdd(a.work + 4, (unsigned long long)st_nb);
-            if (st_dense) atomicAdd(a.work + 5, st_dense);
-            if (st_again) atomicAdd(a.work + 6, st_again);
-            if (st_again_pairs) atomicAdd(a.work + 7, st_again_pairs);
+        if (lane == 0) { // summed in LDS over the workgroup's queries: seven atomics per query on one memory line would queue up
+            if (st_exp) atomicAdd(stat + 1, (unsigned long long)st_exp);
+            if (st_eval) atomicAdd(stat + 2, (unsigned long long)st_eval);
+            if (st_ns) atomicAdd(stat + 3, (unsigned long long)st_ns);
+            if (st_nb) atomicAdd(stat + 4, (unsigned long long)st_nb);
+            if (st_dense) atomicAdd(stat + 5, (unsigned long long)st_dense);
+            if (st_again) atomicAdd(stat + 6, (unsigned long long)st_again);
+            if (st_again_pairs) atomicAdd(stat + 7, (unsigned long long)st_again_pairs);
         }
     }
+    __syncthreads();
+    if (tid >= 1 && tid < 8 && stat[tid]) atomicAdd(a.work + tid, stat[tid]);
 }
 
 // Counters and once-per-query arguments of a launch, written on the stream (no host copy from a stack frame,
