@@ -864,6 +864,7 @@ static int launch_shape(apoe_ctx* ctx, int nw, const SearchArgs& a, uint32_t gri
         case 1: return launch_variant<1, MODE>(ctx, a, grid, lds, per_cu);
         case 4: return launch_variant<4, MODE>(ctx, a, grid, lds, per_cu);
         case 8: return launch_variant<8, MODE>(ctx, a, grid, lds, per_cu);
+        case 16: return launch_variant<16, MODE>(ctx, a, grid, lds, per_cu);
         default: return launch_variant<2, MODE>(ctx, a, grid, lds, per_cu);
     }
 }
@@ -952,11 +953,11 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
         APOE_REQUIRE(fit >= 1, "the static workspace of %u bytes holds no visited bitmap of %zu bytes", (unsigned)APOE_NOALLOC_WS_BYTES, bitmap_bytes);
     }
 
-    // Launch shape (waves per query). 1, 2, 3, 4: one, four, eight, two waves, as the caller says. 0, the default:
+    // Launch shape (waves per query). 1, 2, 3, 4, 5: one, four, eight, two, sixteen waves, as the caller says. 0, the default:
     //  * a batch that is resident all at once is bound by the time of ONE query, and that falls with the waves it has
-    //    (alone, cands 256: 4.2 / 2.9 / 2.2 ms with 2 / 4 / 8 waves): eight waves while all queries still fit the
-    //    machine that way (768 at 3 per CU), else four while they fit (1 536), e.g. 100 queries at cands 256 in 3.4
-    //    instead of 7.9 ms, 1 024 in 5.6 instead of 8.8 ms; four also for batches of up to two rounds of the two-wave
+    //    (alone, cands 256: 4.2 / 2.9 / 2.0 / 1.7 ms with 2 / 4 / 8 / 16 waves): sixteen waves while every query has a
+    //    CU of its own (256), eight while all queries still fit the machine that way (768 at 3 per CU), else four while
+    //    they fit (1 536), e.g. 100 queries at cands 256 in 2.4 instead of 7.9 ms, 1 024 in 5.6 instead of 8.8 ms; four also for batches of up to two rounds of the two-wave
     //    grid (6 144 queries), whose second round ends sooner that way (4-9 % at 4 096 to 6 144 queries, cands 64-512);
     //  * a longer batch is bound by the memory system and runs best with two waves per query and as many queries as fit
     //    (12 per CU) - unless the pool is so large that LDS leaves room for at most 8 queries on a CU: then four waves
@@ -968,7 +969,8 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     if (shape == 1) nw = 1;
     else if (shape == 2) nw = 4;
     else if (shape == 3) nw = 8;
-    else APOE_REQUIRE(shape == 0 || shape == 4, "launch shape %u is not one of 0 (default), 1, 2, 3, 4 (one, four, eight, two waves per query)", shape);
+    else if (shape == 5) nw = 16;
+    else APOE_REQUIRE(shape == 0 || shape == 4, "launch shape %u is not one of 0 (default), 1, 2, 3, 4, 5 (one, four, eight, two, sixteen waves per query)", shape);
     auto resident_per_cu = [&](int waves, int* out) -> int {
         *out = 1;
         APOE_TRY(launch_mode(ctx, mode, waves, a, 0, L.total, out));
@@ -978,11 +980,13 @@ int launch_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, co
     int per_cu = 1;
     if (shape == 0) {
         const size_t at_once = std::min<size_t>(q_count, fit); // queries in flight if every one of them had a workgroup
-        int pc8 = 1, pc4 = 1;
+        int pc16 = 1, pc8 = 1, pc4 = 1;
+        APOE_TRY(resident_per_cu(16, &pc16));
         APOE_TRY(resident_per_cu(8, &pc8));
         APOE_TRY(resident_per_cu(4, &pc4));
         APOE_TRY(resident_per_cu(2, &per_cu));
-        if (at_once <= (size_t)pc8 * ctx->num_cus) { nw = 8; per_cu = pc8; }
+        if (at_once <= (size_t)pc16 * ctx->num_cus) { nw = 16; per_cu = pc16; }
+        else if (at_once <= (size_t)pc8 * ctx->num_cus) { nw = 8; per_cu = pc8; }
         else if (at_once <= (size_t)pc4 * ctx->num_cus || at_once <= 2 * (size_t)per_cu * ctx->num_cus) { nw = 4; per_cu = pc4; }
         else if (per_cu <= 8 && mode != MODE_KEYWORD && pc4 * 4 > per_cu * 2) { nw = 4; per_cu = pc4; }
     } else {

@@ -189,11 +189,12 @@ typedef struct {
     uint32_t cands;                  /* pool size, 1..APOE_MAX_CANDS */
     uint32_t max_iter;               /* 0 -> 1000 (query.cu:7 MAX_ITER) */
     uint32_t q_begin, q_count;       /* query range; q_count 0 -> all from q_begin */
-    uint32_t variant;                /* low byte: launch shape = waves per query. 0 = default: 8 while the whole
-                                        batch is resident at once that way, else 4 up to two rounds of the 2-wave
-                                        grid (about 6 000 queries), else 2 - or 4 when the pool is so large that
-                                        fewer than 9 queries fit a CU (plain and KG search). 1/2/3/4 = 1/4/8/2
-                                        waves whatever the batch; other values are refused. Rows do not depend on it.
+    uint32_t variant;                /* low byte: launch shape = waves per query. 0 = default: 16 while every query
+                                        has a CU of its own, 8 while the whole batch is resident at once that way,
+                                        else 4 up to two rounds of the 2-wave grid (about 6 000 queries), else 2 -
+                                        or 4 when the pool is so large that fewer than 9 queries fit a CU (plain
+                                        and KG search). 1/2/3/4/5 = 1/4/8/2/16 waves whatever the batch; other
+                                        values are refused. Rows do not depend on it.
                                         0x100: read the dense row of every candidate; by
                                         default a candidate whose sparse part plus the Cauchy-Schwarz
                                         bound of its dense part cannot beat the worst entry of the full

@@ -44,7 +44,7 @@ def rows_match(ids, dist, oid, odist, what):
     return same.mean()
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("cands,rule", [(64, "rare"), (16, "common"), (128, "common"), (32, "rare")])
 def test_keyword_search_matches_oracle(gpu_world, cands, rule, variant):
     import apoe

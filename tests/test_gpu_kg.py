@@ -21,7 +21,7 @@ def kg_world(gpu_world):
     return out
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("cands,kg_weight", [(64, 40.0), (128, 5.0), (32, 400.0)])
 def test_kg_search_matches_oracle(kg_world, cands, kg_weight, variant):
     import apoe

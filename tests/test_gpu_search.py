@@ -7,7 +7,7 @@ from parity import assert_dist_close, assert_topk_match, recall_at_k
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("cands", [32, 128])
 def test_search_matches_oracle(gpu_world, cands, variant):
     import apoe
