@@ -13,9 +13,13 @@
 //                in symmetric mode the pair is offered to the column node as well (both endpoints, as the classic
 //                NN-Descent join does; the reference's step updates u only)
 // and a second kernel merges every node's proposals into its sorted list (wave-level rank merge, new before old
-// on equal distance, index.cu:333-351) and registers reverse edges as the expansion step does (index.cu:362-372).
-// Lists are read as the step found them, proposals are minima under a total order: the step does not depend on
-// the order in which tiles run.
+// on equal distance, index.cu:333-351) and registers the entries that are new in a list with their nodes' reverse
+// lists (slot = registrations so far, modulo K; every registration a 64-bit atomicMin, so beyond K the closer entry
+// of a slot stays, index.cu:362-372). Lists are read as the step found them and proposals are minima under a total
+// order, so the lists a step leaves do not depend on the order in which tiles run. The reverse lists are append-only
+// over the steps: a node that later drops v stays in R(v) (a stale column costs one evaluation and can never enter a
+// list wrongly: its distance is computed again), and while a list has fewer than K registrations its content does
+// not depend on the order either; beyond K, which entries share a slot follows the arrival order of the counter.
 #include <hipcub/hipcub.hpp>
 
 #include <algorithm>
@@ -500,9 +504,9 @@ __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* i
         if (v >= n) return;
         const uint32_t slot = atomicAdd(&rev_cnt[v], 1u);
         const unsigned long long k = dist_id_key(dv, u);
-        unsigned long long* at = rev + (size_t)v * JOIN_K + (slot % JOIN_K);
-        if (slot < JOIN_K) *at = k;
-        else atomicMin(at, k);
+        // every registration is a minimum (the lists start at ~0 and the join never starts them again): a store into a slot
+        // that a later registration of the same step has already reached through its wrap-around could undo that one
+        atomicMin(rev + (size_t)v * JOIN_K + (slot % JOIN_K), k);
     };
 #pragma unroll
     for (int s = 0; s < JOIN_PL; s++) {

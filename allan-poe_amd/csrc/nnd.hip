@@ -642,6 +642,74 @@ int apoe_knn_upload(apoe_knn* g, const uint32_t* ids, const float* dist) {
     return APOE_OK;
 }
 
+// Reverse lists as (id, distance) arrays: a slot is one 64-bit word (distance key << 32 | id) on the device.
+__global__ __launch_bounds__(256) static void rev_unpack_kernel(uint64_t total, const unsigned long long* rev, uint32_t* ids, float* dist) {
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (uint64_t)gridDim.x * blockDim.x) {
+        const unsigned long long k = rev[t];
+        const uint32_t id = (uint32_t)k;
+        ids[t] = id;
+        dist[t] = id != EMPTY ? key_dist(k) : INF_DIS;
+    }
+}
+
+__global__ __launch_bounds__(256) static void rev_pack_kernel(uint32_t n, uint64_t total, const uint32_t* ids, const float* dist, unsigned long long* rev,
+                                                              unsigned long long* bad) {
+    unsigned long long mine = 0;
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t id = ids[t];
+        mine += id >= n && id != EMPTY;
+        rev[t] = id < n ? dist_id_key(dist[t], id) : ~0ull;
+    }
+    if (mine) atomicAdd(bad, mine);
+}
+
+int apoe_knn_download_reverse(apoe_knn* g, uint32_t* rev_ids, float* rev_dist, uint32_t* rev_cnt) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_REQUIRE_STATE(g->ready, "the lists are empty: call apoe_nnd_init or apoe_knn_upload first");
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    const size_t total = (size_t)g->n * g->K;
+    if (rev_ids || rev_dist) {
+        DevBuf<uint32_t> ti;
+        DevBuf<float> td;
+        APOE_TRY(ti.alloc(total));
+        APOE_TRY(td.alloc(total));
+        const uint32_t grid = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 16);
+        rev_unpack_kernel<<<grid, 256, 0, g->ctx->stream>>>(total, g->rev.p, ti.p, td.p);
+        APOE_HIP(hipGetLastError());
+        if (rev_ids) APOE_TRY(copy_out(g->ctx, rev_ids, ti.p, total * sizeof(uint32_t)));
+        if (rev_dist) APOE_TRY(copy_out(g->ctx, rev_dist, td.p, total * sizeof(float)));
+    }
+    if (rev_cnt) APOE_TRY(copy_out(g->ctx, rev_cnt, g->rev_cnt.p, (size_t)g->n * sizeof(uint32_t)));
+    return APOE_OK;
+}
+
+int apoe_knn_upload_reverse(apoe_knn* g, const uint32_t* rev_ids, const float* rev_dist, const uint32_t* rev_cnt) {
+    APOE_REQUIRE(g && rev_ids && rev_dist && rev_cnt, "null argument");
+    APOE_REQUIRE_STATE(g->ready, "the lists are empty: call apoe_nnd_init or apoe_knn_upload first");
+    APOE_HIP(hipSetDevice(g->ctx->device));
+    hipStream_t st = g->ctx->stream;
+    const size_t total = (size_t)g->n * g->K;
+    DevBuf<uint32_t> ti;
+    DevBuf<float> td;
+    DevBuf<unsigned long long> packed;
+    APOE_TRY(ti.alloc(total));
+    APOE_TRY(td.alloc(total));
+    APOE_TRY(packed.alloc(total));
+    APOE_TRY(copy_in(g->ctx, ti.p, rev_ids, total * sizeof(uint32_t)));
+    APOE_TRY(copy_in(g->ctx, td.p, rev_dist, total * sizeof(float)));
+    APOE_HIP(hipMemsetAsync(g->counter.p + 1, 0, sizeof(unsigned long long), st));
+    const uint32_t grid = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 16);
+    rev_pack_kernel<<<grid, 256, 0, st>>>(g->n, total, ti.p, td.p, packed.p, g->counter.p + 1);
+    APOE_HIP(hipGetLastError());
+    unsigned long long bad = 0;
+    APOE_TRY(copy_out(g->ctx, &bad, g->counter.p + 1, sizeof(bad)));
+    APOE_REQUIRE(bad == 0, "%llu uploaded reverse ids are neither below the %u documents of the corpus nor the empty slot 0xFFFFFFFF", bad, g->n);
+    APOE_HIP(hipMemcpyAsync(g->rev.p, packed.p, total * sizeof(unsigned long long), hipMemcpyDeviceToDevice, st));
+    APOE_TRY(copy_in(g->ctx, g->rev_cnt.p, rev_cnt, (size_t)g->n * sizeof(uint32_t)));
+    APOE_HIP(hipStreamSynchronize(st));
+    return APOE_OK;
+}
+
 float apoe_knn_elapsed_ms(const apoe_knn* g) { return g ? g->elapsed_ms : 0.f; }
 
 int apoe_knn_counters(apoe_knn* g, uint64_t* out2) {

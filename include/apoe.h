@@ -160,6 +160,13 @@ int apoe_nnd_merge_reverse(apoe_knn* g);
 /* Copy the kNN graph out / in (ids without flag bits, distances), [n][K] each. */
 int apoe_knn_download(apoe_knn* g, uint32_t* ids, float* dist);
 int apoe_knn_upload(apoe_knn* g, const uint32_t* ids, const float* dist);
+/* The reverse lists as they stand (reverse_graph_dev / reverse_distance / reverse_num, index.cu:90,93,845-846):
+ * rev_ids/rev_dist [n][K] (a slot never written holds id 0xFFFFFFFF, distance INF_DIS), rev_cnt [n] = registrations
+ * counted so far (may exceed K: later ones replaced slot count % K when closer, index.cu:362-372). Any pointer may
+ * be NULL. With the upload they make apoe_nnd_merge_reverse checkable on a state of the caller's making; uploaded
+ * ids must name a document or be 0xFFFFFFFF. */
+int apoe_knn_download_reverse(apoe_knn* g, uint32_t* rev_ids, float* rev_dist, uint32_t* rev_cnt);
+int apoe_knn_upload_reverse(apoe_knn* g, const uint32_t* rev_ids, const float* rev_dist, const uint32_t* rev_cnt);
 /* allan_poe (index.cu:539-714): RNG-IP prune to `degree` + keyword-edge candidates. */
 int apoe_prune(apoe_knn* g, uint32_t degree);
 /* Intermediate result of apoe_prune: fwd/det [n][degree], cnt [n], kw [n][1+APOE_KW_CAND]. */
