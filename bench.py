@@ -248,6 +248,21 @@ def main():
         log(f"[bench] KG search cands 128: {sk.kernel_ms:.2f} ms, entity document in the top 10 for {hits / nq_truth:.3f} of the queries")
         gkg.close()
 
+    # ---- the reference's own semantics: user weights 1/1/1 go through the query-time calibration (query.cu:1847-1881),
+    # ground truth is brute force under the calibrated weights ----
+    calibrated = None
+    if not args.no_sweeps and not args.calibrate:
+        wc = apoe.calibrate_weights(ctx, gc, gq, (1.0, 1.0, 1.0))
+        tc, _ = B.hybrid_topk(corpus, queries, wc, 10, nq=nq_truth)
+        calibrated = dict(user_weights=(1.0, 1.0, 1.0), effective_weights_dense_sparse_bm25=tuple(float(x) for x in wc), sweep=[])
+        for ec in (64, 128, 256):
+            apoe.search(ctx, gc, gq, graph, wc, ec)
+            ids_c, _, sc = apoe.search(ctx, gc, gq, graph, wc, ec)
+            calibrated["sweep"].append(dict(cands=ec, kernel_ms=sc.kernel_ms, qps=args.queries / (sc.kernel_ms / 1e3),
+                                            recall_at_10=recall_at_k(ids_c[:nq_truth], tc, 10), algo_gbs=sc.algo_bytes / (sc.kernel_ms / 1e3) / 1e9,
+                                            dense_rows_per_evaluation=sc.dense_rows / max(sc.evaluations, 1)))
+            log(f"[bench] calibrated weights {tuple(round(float(x), 2) for x in wc)} cands {ec}: {sc.kernel_ms:.2f} ms, recall {calibrated['sweep'][-1]['recall_at_10']:.4f}")
+
     # ---- short batches: the launch shape follows the batch (more waves per query while the whole batch is resident at once) ----
     short_batches = None
     if not args.no_sweeps:
@@ -386,14 +401,15 @@ def main():
         q_np = S.to_numpy(queries)
         Q_ = O.HybridSet(*q_np).head(ncpu)
         rows, entry = graph.download()
-        threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+        threads = O.max_threads()  # omp_get_max_threads(): every host core this process is given
         t0 = time.perf_counter()
         oid, odist, _ = O.search(C_, Q_, rows, entry, w3, cands, max_iter=iter_cap(cands) or 1000, threads=threads)
         cpu_s = time.perf_counter() - t0
         agree = float(np.mean(oid[:, :10] == out_ids[:ncpu, :10].cpu().numpy().view(np.uint32)))
         cpu = dict(value=ncpu / cpu_s, unit="queries/s", cores=threads, kind="port",
                    sample=f"first {ncpu} of the {args.queries} queries, same corpus, graph, weights and cands={cands}; "
-                          f"{cpu_s:.1f}s; top-10 ids equal to the GPU's at {agree:.4f} of positions")
+                          f"{cpu_s:.1f}s on omp_get_max_threads() = {threads} threads (the host shows {os.cpu_count()} logical CPUs); "
+                          f"top-10 ids equal to the GPU's at {agree:.4f} of positions")
         log(f"[bench] cpu oracle: {cpu['value']:.0f} QPS on {threads} threads; top-10 agreement {agree:.4f}")
 
     if ok:
@@ -441,6 +457,7 @@ def main():
             "kernel_ms": avg_kernel_ms,
             **({"weight_sweep_without_rebuild": weight_sweep} if weight_sweep else {}),
             **({"knowledge_graph_search": kg_search} if kg_search else {}),
+            **({"reference_semantics_calibrated_weights": calibrated} if calibrated else {}),
             **({"short_batches": short_batches} if short_batches else {}),
             **({"same_generators_smaller_corpora": smaller} if smaller else {}),
             **({"extras": extras} if extras else {}),

@@ -603,6 +603,8 @@ void orc_search_kg(const orc_set* corpus, const orc_set* queries, const orc_kg* 
 
 /* ------------------------------------------------------------------ NN-Descent */
 
+int orc_max_threads(void) { return omp_get_max_threads(); }
+
 uint32_t orc_rand_id(uint64_t seed, uint64_t counter, uint32_t n) {
     return (uint32_t)(mix64(seed ^ mix64(counter)) % n);
 }

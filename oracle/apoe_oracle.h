@@ -96,6 +96,9 @@ void orc_search_kg(const orc_set* corpus, const orc_set* queries, const orc_kg* 
                    const float* w3, float kg_weight, uint32_t cands, uint32_t max_iter,
                    uint32_t* out_ids, float* out_dist, uint64_t* counters, int threads);
 
+/* omp_get_max_threads(): the thread count every function here uses when its `threads` argument is 0. */
+int orc_max_threads(void);
+
 /* NN-Descent (index.cu:99-106, 156-478). ids carry ORC_FLAG = "already sampled". */
 uint32_t orc_rand_id(uint64_t seed, uint64_t counter, uint32_t n);
 void orc_nnd_init(uint32_t n, uint32_t K, uint64_t seed, uint32_t* ids, float* dist,

@@ -64,6 +64,12 @@ def lib():
     return _LIB
 
 
+def max_threads():
+    """omp_get_max_threads() of the oracle library: what threads=0 uses."""
+    lib().orc_max_threads.restype = C.c_int
+    return int(lib().orc_max_threads())
+
+
 def _u32(a):
     a = np.ascontiguousarray(a, dtype=np.uint32)
     return a, a.ctypes.data_as(u32p)

@@ -203,25 +203,31 @@ def _mean_recall(graphs, ctx, gc, gq, truth, cands):
 def test_gpu_built_index_recall(gpu_world, join):
     """Whole GPU build (expansion step and local join): recall@10 of the search on it within 0.5 points of the
     oracle-built index. Both builds start from random lists (and the GPU's expansion step races, as the reference's
-    does), so each side is the mean over three seeds, measured on 2 000 queries against exact brute force."""
+    does), so each side is the mean over three seeds, measured on 2 000 queries against exact brute force. On the
+    wide pair format one GPU build is compared with the oracle-built index of the shared world (one seed on each
+    side: 1.5 points)."""
     import apoe
     import apoe_synth as S
     import oracle as O
     w = gpu_world
-    if w["gc"].pair_bytes() == 8:
-        pytest.skip("one pair format is enough here: the build kernels are compared per format in the tests above")
+    wide = w["gc"].pair_bytes() == 8
     q_arrays = S.to_numpy(S.queries(2000, seed=412))
+    if wide:
+        q_arrays = q_arrays[:5] + (q_arrays[5] + np.uint32(70000),) + q_arrays[6:]
     Q = O.HybridSet(*q_arrays)
     gq = apoe.Queries(w["ctx"], *q_arrays)
     truth, _ = O.bruteforce_topk(w["C"], Q, (1.0, 1.0, 1.0), 10)
-    seeds = (5, 6, 7)
+    seeds = (5,) if wide else (5, 6, 7)
     g_gpu = [apoe.build_graph(w["ctx"], w["gc"], K=64, iters=8, degree=32, dense_scale=7.0, seed=s, join=join)[0] for s in seeds]
-    g_orc = [apoe.Graph(w["ctx"], *O.build_index(w["C"], dense_scale=7.0, K=64, iters=8, d=32, seed=s)) for s in seeds]
+    if wide:
+        g_orc = [apoe.Graph(w["ctx"], w["rows"], w["entry"])]
+    else:
+        g_orc = [apoe.Graph(w["ctx"], *O.build_index(w["C"], dense_scale=7.0, K=64, iters=8, d=32, seed=s)) for s in seeds]
     for cands in (64, 128):
         r_g, all_g = _mean_recall(g_gpu, w["ctx"], w["gc"], gq, truth, cands)
         r_c, all_c = _mean_recall(g_orc, w["ctx"], w["gc"], gq, truth, cands)
         print(f"join={join} cands={cands}: recall@10 gpu-built {r_g:.4f} {np.round(all_g, 4)}, oracle-built {r_c:.4f} {np.round(all_c, 4)}")
-        assert r_g >= r_c - 0.005
+        assert r_g >= r_c - (0.015 if wide else 0.005)
     rows, entry = g_gpu[0].download()
     assert rows.shape == (w["C"].n, 40) and len(entry) == 32
     for g in g_gpu + g_orc:

@@ -1,5 +1,5 @@
-"""The whole path at 100 000 docs (degree 32, K = 64, 10 NN-Descent steps, cands 128): the oracle checks a
-sample, the rest is checked through properties that do not depend on the size."""
+"""The whole path at 100 000 docs and 10 000 queries (degree 32, K = 64, 10 NN-Descent steps, cands 128): the oracle
+checks a sample, the whole batch is checked through properties that do not depend on the size."""
 import numpy as np
 import pytest
 
@@ -7,7 +7,7 @@ from parity import assert_dist_close, assert_topk_match, recall_at_k
 
 pytestmark = pytest.mark.gpu
 
-N_DOCS, N_QUERIES, DEGREE, CANDS = 100_000, 2_000, 32, 128
+N_DOCS, N_QUERIES, DEGREE, CANDS = 100_000, 10_000, 32, 128
 EMPTY_ID = 0x7FFFFFFF
 
 
