@@ -125,8 +125,6 @@ struct JoinLds {
     uint32_t G, tab, row_list, rowptr, rownnz, row_id, col_id, row_worst, col_worst, seen, scan, ctl, total;
     __host__ __device__ JoinLds(uint32_t index_bits, uint32_t slot_cap, bool narrow) {
         uint32_t o = 0;
-        tab = o; o += RankTabLds(index_bits, slot_cap, narrow).total;
-        o = (o + 15) & ~15u;
         G = o; o += JT_ROWS * JT_STRIDE * 4;
         row_list = o; o += JT_ROWS * JOIN_K * 4;
         o = (o + 7) & ~7u;
@@ -139,84 +137,72 @@ struct JoinLds {
         seen = o; o += JT_SEEN * 4;
         scan = o; o += 20 * 4;
         ctl = o; o += 8 * 4;
+        o = (o + 15) & ~15u;
+        // the rank table of the sparse part; before it is built, the same bytes hold the dense parts of the picker rows
+        const uint32_t table = RankTabLds(index_bits, slot_cap, narrow).total, rows = (uint32_t)(JT_ROWS * DENSE_BYTES);
+        tab = o; o += table > rows ? table : rows;
         total = o;
     }
 };
 
-// acc = <rows, cols> over the 8-float blocks [b_begin, b_end) of the dimensions for the 32 x 32 block of row ids `ra` (nr of them) and column ids
-// `cb` (nc of them); operand layout as gram_dense_upper (apoe_gram.h). Rows / columns beyond the counts repeat the last one.
-__device__ __forceinline__ floatx16 join_dense_block(const CorpusView& C, const uint32_t* ra, uint32_t nr, const uint32_t* cb, uint32_t nc, int lane,
-                                                     int b_begin, int b_end) {
-    floatx16 acc;
+// Dense part of a tile on v_mfma_f32_16x16x4_f32. A wave owns 16 columns and a range of 16-float blocks of the
+// dimensions; the picker rows come from LDS (`A`: row r, float4 c at A[r * 256 + (c ^ (r & 7))] -- the swizzle spreads
+// the sixteen rows of a read over the banks without padding), the column rows straight from memory. Lane (j, g), j =
+// lane % 16, g = lane / 16, supplies float4 number 4 b + g of block b for row j (A operand) and for column j (B
+// operand): the four multiplies of a block take one component each, so k-slot g of multiply c stands for dimension
+// 16 b + 4 g + c on both sides. RING column blocks are in flight ahead of the one being multiplied (a ring of
+// registers, refilled as it is consumed). Rows 16..31 of the tile take a second accumulator fed from the same column
+// registers, and only when the tile has them: a tile of at most 16 rows costs half the matrix time.
+// Result: lane (j, g) holds row 4 g + e (+ 16), column j in acc0[e] (acc1[e]).
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+template <int RING>
+__device__ __forceinline__ void join_dense16(const float4* A, uint32_t nr, const float4* pb, int lane, int b_begin, int b_end, floatx4& acc0,
+                                             floatx4& acc1) {
+    const int j = lane & 15, g = lane >> 4;
+    const uint32_t i0 = min((uint32_t)j, nr - 1), i1 = min(16u + (uint32_t)j, nr - 1);
+    const float4* a0 = A + i0 * (DIM / 4);
+    const float4* a1 = A + i1 * (DIM / 4);
+    const uint32_t s0 = i0 & 7, s1 = i1 & 7;
+    const bool two = nr > 16; // wave-uniform
+    float4 ring[RING];
 #pragma unroll
-    for (int v = 0; v < 16; v++) acc[v] = 0.f;
-    const uint32_t ia = min((uint32_t)(lane & 31), nr - 1), ib = min((uint32_t)(lane & 31), nc - 1);
-    const float4* pa = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[ra[ia]]) * 16) + (lane >> 5);
-    const float4* pb = reinterpret_cast<const float4*>(C.recs + desc_off(C.desc[cb[ib]]) * 16) + (lane >> 5);
-    // operands of the next four 8-float blocks are requested before the current four are multiplied
-    constexpr int NB = 4;
-    float4 a[2][NB], bb[2][NB];
-#pragma unroll
-    for (int u = 0; u < NB; u++) { a[0][u] = pa[2 * (b_begin + u)]; bb[0][u] = pb[2 * (b_begin + u)]; }
+    for (int u = 0; u < RING; u++) ring[u] = pb[4 * (b_begin + u)];
 #pragma unroll 1
-    for (int b = b_begin; b < b_end; b += 2 * NB) {
+    for (int b = b_begin; b < b_end; b += RING) {
+        const bool more = b + RING < b_end;
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int nb = b + (half + 1) * NB; // first block of the batch after this one
-            if (nb < b_end) {
-#pragma unroll
-                for (int u = 0; u < NB; u++) { a[half ^ 1][u] = pa[2 * (nb + u)]; bb[half ^ 1][u] = pb[2 * (nb + u)]; }
-            }
-#pragma unroll
-            for (int u = 0; u < NB; u++) {
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[half][u].x, bb[half][u].x, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[half][u].y, bb[half][u].y, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[half][u].z, bb[half][u].z, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[half][u].w, bb[half][u].w, acc, 0, 0, 0);
+        for (int u = 0; u < RING; u++) {
+            const float4 bv = ring[u];
+            if (more) ring[u] = pb[4 * (b + u + RING)];
+            const uint32_t c = 4u * (uint32_t)(b + u) + (uint32_t)g;
+            const float4 av = a0[c ^ s0];
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, bv.x, acc0, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, bv.y, acc0, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, bv.z, acc0, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, bv.w, acc0, 0, 0, 0);
+            if (two) {
+                const float4 aw = a1[c ^ s1];
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(aw.x, bv.x, acc1, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(aw.y, bv.y, acc1, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(aw.z, bv.z, acc1, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(aw.w, bv.w, acc1, 0, 0, 0);
             }
         }
     }
-    return acc;
 }
 
-// The same block with the row operand staged in LDS (`A`: row r at float4 index r * JT_A_STRIDE, all 1024 dimensions):
-// the four waves that share the picker rows read them from memory once per tile instead of once each, and a wave's
-// registers hold twice as many column blocks in flight. `pb0` = the dense row of this lane's column.
-constexpr int JT_A_STRIDE = DIM / 4 + 1; // float4 per staged row: the odd stride spreads the 32 rows of a read over the LDS banks
-__device__ __forceinline__ floatx16 join_dense_block_lds(const float4* A, uint32_t nr, const float4* pb0, int lane, int b_begin, int b_end) {
-    floatx16 acc;
+// 64 values, one per lane, in ascending order over the lanes (bitonic network, 21 exchanges).
+__device__ __forceinline__ uint32_t wave_sort_u32(uint32_t v, int lane) {
 #pragma unroll
-    for (int v = 0; v < 16; v++) acc[v] = 0.f;
-    const uint32_t ia = min((uint32_t)(lane & 31), nr - 1);
-    const float4* pa = A + ia * JT_A_STRIDE + (lane >> 5);
-    const float4* pb = pb0 + (lane >> 5);
-    constexpr int NB = 8;
-    float4 bb[2][NB];
+    for (int k = 2; k <= WAVE; k <<= 1) {
 #pragma unroll
-    for (int u = 0; u < NB; u++) bb[0][u] = pb[2 * (b_begin + u)];
-#pragma unroll 1
-    for (int b = b_begin; b < b_end; b += 2 * NB) {
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int cur = b + half * NB, nb = cur + NB; // first block of this batch and of the batch after it
-            if (cur >= b_end) break;
-            if (nb < b_end) {
-#pragma unroll
-                for (int u = 0; u < NB; u++) bb[half ^ 1][u] = pb[2 * (nb + u)];
-            }
-            float4 a[NB];
-#pragma unroll
-            for (int u = 0; u < NB; u++) a[u] = pa[2 * (cur + u)];
-#pragma unroll
-            for (int u = 0; u < NB; u++) {
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].x, bb[half][u].x, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].y, bb[half][u].y, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].z, bb[half][u].z, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].w, bb[half][u].w, acc, 0, 0, 0);
-            }
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            const uint32_t o = __shfl_xor(v, j, WAVE);
+            const bool take_min = ((lane & j) == 0) == ((lane & k) == 0 || k == WAVE);
+            v = take_min ? min(v, o) : max(v, o);
         }
     }
-    return acc;
+    return v;
 }
 
 template <bool NARROW>
@@ -270,60 +256,55 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
         const uint32_t M = uniform(ctl[1]);
         if (M == 0) continue;
         // the rows' own lists (who is already a neighbour), the columns' thresholds, where every row's pairs are
-        for (uint32_t t = tid; t < R * JOIN_K; t += JT_THREADS) row_list[t] = a.ids[(size_t)row_id[t / JOIN_K] * JOIN_K + (t % JOIN_K)] & ~FLAG;
+        {   // each row's list in ascending id order (the proposals look an id up by binary search): wave w reads and sorts rows w, w + 8, ...
+            uint32_t mine[JT_ROWS / NW];
+#pragma unroll
+            for (int k = 0; k < JT_ROWS / NW; k++) {
+                const uint32_t r = wave + k * NW;
+                mine[k] = r < R ? a.ids[(size_t)row_id[r] * JOIN_K + lane] & ~FLAG : 0u;
+            }
+#pragma unroll
+            for (int k = 0; k < JT_ROWS / NW; k++) {
+                const uint32_t r = wave + k * NW;
+                if (r < R) row_list[r * JOIN_K + lane] = wave_sort_u32(mine[k], lane);
+            }
+        }
         if ((uint32_t)tid < M) col_worst[tid] = a.symmetric ? a.dist[(size_t)col_id[tid] * JOIN_K + JOIN_K - 1] : -INF_DIS;
         gram_rows_gather(a.C, row_id, R, rowptr, rownnz, tid, JT_THREADS);
         gram_rows_gather(a.C, col_id, M, rowptr + JT_ROWS, rownnz + JT_ROWS, tid, JT_THREADS);
         __syncthreads();
-        // each row's list in ascending id order, in place: a wave reads a whole list before it writes any of it
-        for (uint32_t r = wave; r < R; r += NW) {
-            uint32_t* lst = row_list + r * JOIN_K;
-            const uint32_t mine = lst[lane];
-            uint32_t rank = 0;
-            for (uint32_t i = 0; i < JOIN_K; i++) {
-                const uint32_t x = lst[i];
-                rank += x < mine || (x == mine && i < (uint32_t)lane);
-            }
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            lst[rank] = mine;
-        }
-        // dense part: the eight waves share the 32-column blocks that exist (1, 2 or 4 by the number of columns) and, for
-        // each block, equal parts of the dimensions (8, 4 or 2): no wave idles when a tile has few columns. The partial
-        // tiles are added into G in a fixed order, a barrier between them.
+        // dense part: the eight waves share the 16-column blocks that exist (8, 4, 2 or 1 by the number of columns) and, for
+        // each block, equal parts of the dimensions (1, 2, 4 or 8): no wave idles when a tile has few columns. The picker
+        // rows are staged in the table region, which is free until the sparse part. Partial tiles are added into G in a
+        // fixed order, a barrier between them.
         {
-            const uint32_t nblk = M <= 32 ? 1u : M <= 64 ? 2u : 4u, parts = (uint32_t)NW / nblk;
+            const uint32_t nblk = M <= 16 ? 1u : M <= 32 ? 2u : M <= 64 ? 4u : 8u, parts = (uint32_t)NW / nblk;
             const uint32_t blk = (uint32_t)wave % nblk, part = (uint32_t)wave / nblk;
-            const bool active = blk * 32 < M;
-            const uint32_t per = (DIM / 8) / parts; // 8-float blocks of the dimensions per part: 16, 32 or 64
-            floatx16 acc;
-            // the picker rows go through LDS when they fit the table region, which is free until the sparse part
-            const bool staged = R * (uint32_t)JT_A_STRIDE * 16u <= RankTabLds(a.index_bits, a.slot_cap, NARROW).total;
+            const bool active = blk * 16 < M;
+            const uint32_t per = (DIM / 16) / parts; // 16-float blocks of the dimensions per part: 64, 32, 16 or 8
             float4* A = reinterpret_cast<float4*>(smem + L.tab);
-            if (staged) {
-                for (uint32_t i = tid; i < R * (DIM / 4); i += JT_THREADS) {
-                    const uint32_t r = i / (DIM / 4), c = i % (DIM / 4);
-                    A[r * JT_A_STRIDE + c] = reinterpret_cast<const float4*>(rowptr[r] - DENSE_BYTES)[c];
-                }
-                __syncthreads();
+            const uint32_t jcol = min(blk * 16 + (uint32_t)(lane & 15), M - 1);
+            const float4* pb = reinterpret_cast<const float4*>(rowptr[JT_ROWS + jcol] - DENSE_BYTES) + (lane >> 4);
+#pragma unroll 4
+            for (uint32_t i = tid; i < R * (DIM / 4); i += JT_THREADS) {
+                const uint32_t r = i / (DIM / 4), c = i % (DIM / 4);
+                A[r * (DIM / 4) + (c ^ (r & 7))] = reinterpret_cast<const float4*>(rowptr[r] - DENSE_BYTES)[c];
             }
+            __syncthreads();
+            floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
             if (active) {
-                if (staged) {
-                    const uint32_t ib = min((uint32_t)(lane & 31), min(32u, M - blk * 32) - 1);
-                    acc = join_dense_block_lds(A, R, reinterpret_cast<const float4*>(rowptr[JT_ROWS + blk * 32 + ib] - DENSE_BYTES), lane, (int)(part * per),
-                                               (int)((part + 1) * per));
-                } else if (nblk == 4) { // the usual shape (more than 64 columns) with compile-time loop bounds
-                    acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, part ? DIM / 16 : 0, part ? DIM / 8 : DIM / 16);
-                } else {
-                    acc = join_dense_block(a.C, row_id, R, col_id + blk * 32, min(32u, M - blk * 32), lane, (int)(part * per), (int)((part + 1) * per));
-                }
+                if (per >= 16) join_dense16<16>(A, R, pb, lane, (int)(part * per), (int)((part + 1) * per), acc0, acc1);
+                else join_dense16<8>(A, R, pb, lane, (int)(part * per), (int)((part + 1) * per), acc0, acc1);
             }
             auto store = [&](bool add) {
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    const int i = 8 * (e / 4) + 4 * (lane >> 5) + (e % 4), j = lane & 31;
-                    float* at = &G[i * JT_STRIDE + blk * 32 + j];
-                    *at = add ? *at + a.dense_mul * acc[e] : a.dense_mul * acc[e];
+                for (int e = 0; e < 4; e++) {
+                    float* at = &G[(4 * (lane >> 4) + e) * JT_STRIDE + blk * 16 + (lane & 15)];
+                    *at = add ? *at + a.dense_mul * acc0[e] : a.dense_mul * acc0[e];
+                    if (R > 16) {
+                        float* at1 = at + 16 * JT_STRIDE;
+                        *at1 = add ? *at1 + a.dense_mul * acc1[e] : a.dense_mul * acc1[e];
+                    }
                 }
             };
             for (uint32_t ph = 0; ph < parts; ph++) {
@@ -565,7 +546,7 @@ int launch_nnd_join_iterate(apoe_knn* g) {
     uint32_t index_bits, slot_cap, span;
     join_table_shape(g->corpus, &index_bits, &slot_cap, &span);
     const JoinLds L(index_bits, slot_cap, g->corpus->narrow);
-    APOE_REQUIRE(L.total <= 150 * 1024, "the local-join tile needs %u bytes of LDS", L.total);
+    APOE_REQUIRE(L.total <= ctx->lds_per_block, "the local-join tile needs %u bytes of LDS, a workgroup may have %zu", L.total, ctx->lds_per_block);
 
     APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), st)); // [0] inserted; [2], [3] accumulate over the build
     fill_u32_kernel2<<<1024, 256, 0, st>>>(g->pick_cnt.p, (uint64_t)n + 1, 0u);
