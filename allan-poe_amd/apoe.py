@@ -40,7 +40,7 @@ EXPORTS = [
     "apoe_corpus_destroy", "apoe_corpus_info", "apoe_corpus_bytes", "apoe_corpus_pair_bytes", "apoe_corpus_make_half_rows", "apoe_queries_create", "apoe_queries_destroy",
     "apoe_kg_create", "apoe_kg_destroy", "apoe_calibrate_weights", "apoe_hybrid_distance_batch", "apoe_hybrid_distance_pairs", "apoe_norms",
     "apoe_knn_create", "apoe_knn_destroy", "apoe_knn_use_half_rows", "apoe_knn_set_join", "apoe_nnd_init", "apoe_nnd_iterate", "apoe_nnd_merge_reverse",
-    "apoe_knn_download", "apoe_knn_upload", "apoe_knn_download_reverse", "apoe_knn_upload_reverse", "apoe_prune", "apoe_prune_download", "apoe_finalize_graph",
+    "apoe_knn_download", "apoe_knn_upload", "apoe_knn_download_reverse", "apoe_knn_upload_reverse", "apoe_knn_set_prune_form", "apoe_prune", "apoe_prune_download", "apoe_finalize_graph",
     "apoe_knn_elapsed_ms", "apoe_knn_counters", "apoe_graph_create", "apoe_graph_destroy", "apoe_graph_info", "apoe_graph_download",
     "apoe_search", "apoe_search_noalloc",
 ]
@@ -279,6 +279,10 @@ class Knn:
     def upload_reverse(self, rev_ids, rev_dist, rev_cnt):
         ri, rd, rc = _ptr(rev_ids, np.uint32), _ptr(rev_dist, np.float32), _ptr(rev_cnt, np.uint32)
         _check(lib().apoe_knn_upload_reverse(self.h, ri[1], rd[1], rc[1]))
+
+    def set_prune_form(self, form):
+        """0: the gather-once forms of the prune where they apply (default); 1: the table-probing kernel."""
+        _check(lib().apoe_knn_set_prune_form(self.h, C.c_int(form)))
 
     def prune(self, degree):
         _check(lib().apoe_prune(self.h, C.c_uint32(degree)))

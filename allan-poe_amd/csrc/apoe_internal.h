@@ -185,6 +185,8 @@ int launch_nnd_init(apoe_knn* g, uint64_t seed);
 int launch_nnd_iterate(apoe_knn* g, uint64_t* inserted);
 int launch_nnd_join_iterate(apoe_knn* g);
 int join_step_counters(apoe_knn* g, unsigned long long* out3);
+int launch_gram_tiles(apoe_knn* g, uint32_t node0, uint32_t n_nodes, float* gram, unsigned long long* unfit);
+bool gram_tiles_fit(const apoe_knn* g);
 int launch_nnd_merge_reverse(apoe_knn* g);
 int launch_prune(apoe_knn* g, uint32_t degree);
 int launch_final_graph(apoe_knn* g, uint32_t* rows_dev);

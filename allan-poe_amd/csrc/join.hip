@@ -205,6 +205,121 @@ __device__ __forceinline__ uint32_t wave_sort_u32(uint32_t v, int lane) {
     return v;
 }
 
+// The hybrid inner products of a tile, G[r * JT_STRIDE + c] = dense_mul * <row r, column c>_dense + <row r, column c>_sparse for
+// the R rows and M columns whose record addresses and shapes `rowptr` / `rownnz` hold (rows at [0, JT_ROWS), columns at
+// [JT_ROWS, JT_ROWS + JT_COLS): gram_rows_gather). All JT_THREADS threads call it after a barrier behind those arrays; it
+// ends with a barrier. `tabreg` = the table region of JoinLds, `unfit` = counter of rows whose terms did not fit the table.
+template <bool NARROW>
+__device__ __forceinline__ void tile_hybrid_ips(const CorpusView& C, float dense_mul, char* tabreg, const RankTab& T, uint32_t index_bits, uint32_t slot_cap,
+                                                float* G, const unsigned long long* rowptr, const uint32_t* rownnz, uint32_t* scan, uint32_t R,
+                                                uint32_t M, unsigned long long* unfit, int tid, int wave, int lane) {
+    constexpr int NW = JT_THREADS / WAVE;
+    // dense part: the eight waves share the 16-column blocks that exist (8, 4, 2 or 1 by the number of columns) and, for
+    // each block, equal parts of the dimensions (1, 2, 4 or 8): no wave idles when a tile has few columns. The picker
+    // rows are staged in the table region, which is free until the sparse part. Partial tiles are added into G in a
+    // fixed order, a barrier between them.
+    {
+        const uint32_t nblk = M <= 16 ? 1u : M <= 32 ? 2u : M <= 64 ? 4u : 8u, parts = (uint32_t)NW / nblk;
+        const uint32_t blk = (uint32_t)wave % nblk, part = (uint32_t)wave / nblk;
+        const bool active = blk * 16 < M;
+        const uint32_t per = (DIM / 16) / parts; // 16-float blocks of the dimensions per part: 64, 32, 16 or 8
+        float4* A = reinterpret_cast<float4*>(tabreg);
+        const uint32_t jcol = min(blk * 16 + (uint32_t)(lane & 15), M - 1);
+        const float4* pb = reinterpret_cast<const float4*>(rowptr[JT_ROWS + jcol] - DENSE_BYTES) + (lane >> 4);
+#pragma unroll 4
+        for (uint32_t i = tid; i < R * (DIM / 4); i += JT_THREADS) {
+            const uint32_t r = i / (DIM / 4), c = i % (DIM / 4);
+            A[r * (DIM / 4) + (c ^ (r & 7))] = reinterpret_cast<const float4*>(rowptr[r] - DENSE_BYTES)[c];
+        }
+        __syncthreads();
+        floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+        if (active) {
+            if (per >= 16) join_dense16<16>(A, R, pb, lane, (int)(part * per), (int)((part + 1) * per), acc0, acc1);
+            else join_dense16<8>(A, R, pb, lane, (int)(part * per), (int)((part + 1) * per), acc0, acc1);
+        }
+        auto store = [&](bool add) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float* at = &G[(4 * (lane >> 4) + e) * JT_STRIDE + blk * 16 + (lane & 15)];
+                *at = add ? *at + dense_mul * acc0[e] : dense_mul * acc0[e];
+                if (R > 16) {
+                    float* at1 = at + 16 * JT_STRIDE;
+                    *at1 = add ? *at1 + dense_mul * acc1[e] : dense_mul * acc1[e];
+                }
+            }
+        };
+        for (uint32_t ph = 0; ph < parts; ph++) {
+            if (active && part == ph) store(ph != 0);
+            if (ph + 1 < parts) __syncthreads();
+        }
+    }
+    __syncthreads();
+    // sparse part: groups of eight rows in the rank table, every column probes it once per group. The pairs of a
+    // group's rows are requested while the group before it is probed; the pairs of a wave's columns stay in its
+    // registers for the whole tile: a build and the probes find their operands there.
+    auto row_pairs = [&](uint32_t i) { Pairs p = gram_row(C, rowptr, rownnz, i); p.narrow = NARROW ? 1u : 0u; return p; };
+    auto col_pairs = [&](uint32_t b) { Pairs p = gram_row(C, rowptr + JT_ROWS, rownnz + JT_ROWS, b); p.narrow = NARROW ? 1u : 0u; return p; };
+    uint32_t a0 = 0;
+    PivotRegs pv;
+    ranktab_pivots_load(pv, [&](uint32_t t) { return row_pairs(a0 + t); }, min((uint32_t)RT_T, R - a0), tid, JT_THREADS);
+    // the wave's columns wave, wave + NW, ...: read once per tile, probed once per group; their shapes
+    // (nnz | ns << 16) are wave-uniform and stay in scalar registers
+    RtRow<NARROW> own[JT_OWN];
+    uint32_t own_shape[JT_OWN];
+#pragma unroll
+    for (int k = 0; k < JT_OWN; k++) {
+        const uint32_t b = wave + k * NW;
+        own_shape[k] = 0;
+        if (b < M) {
+            own_shape[k] = uniform(rownnz[JT_ROWS + b]);
+            rt_row_load(own[k], col_pairs(b), lane);
+        }
+    }
+    while (a0 < R) {
+        uint32_t nt = min((uint32_t)RT_T, R - a0);
+        uint32_t built;
+        while (true) {
+            built = ranktab_build<NARROW>(T, [&](uint32_t t) { return row_pairs(a0 + t); }, pv, nt, scan, tid, JT_THREADS);
+            if (built != EMPTY || nt == 1) break;
+            nt = (nt + 1) / 2; // the registers hold the first pivots of the group whatever nt is
+        }
+        const uint32_t a1 = a0 + nt;
+        if (a1 < R) ranktab_pivots_load(pv, [&](uint32_t t) { return row_pairs(a1 + t); }, min((uint32_t)RT_T, R - a1), tid, JT_THREADS);
+        if (built == EMPTY) { // one row alone does not fit: its sparse part is missing, the host is told
+            if (tid == 0) atomicAdd(unfit, 1ull);
+            a0 = a1;
+            continue;
+        }
+        const uint32_t n_ovf = NARROW ? 0u : uniform(min(scan[16], (uint32_t)RT_OVF));
+#pragma unroll
+        for (int q = 0; q < JT_OWN / JT_BATCH; q++) {
+            const uint32_t b0 = wave + q * JT_BATCH * NW;
+            if (b0 < M) { // wave-uniform
+                float acc[JT_BATCH][RT_T];
+                RtRow<NARROW> rows[JT_BATCH];
+                uint32_t shape[JT_BATCH];
+#pragma unroll
+                for (int k = 0; k < JT_BATCH; k++) {
+                    rows[k] = own[q * JT_BATCH + k];
+                    rows[k].touch();
+                    shape[k] = own_shape[q * JT_BATCH + k];
+                    asm volatile("" : "+s"(shape[k])); // as touch(): the lane masks of a row are made where they are used
+#pragma unroll
+                    for (int t = 0; t < RT_T; t++) acc[k][t] = 0.f;
+                }
+                ranktab_probe_rows<NARROW, JT_BATCH>(T, rows, shape, [&](int k) { return col_pairs(b0 + k * NW); }, n_ovf, acc, lane);
+                uint32_t t, r;
+                const float z = wave_sum_2x8(acc, lane, &t, &r);
+                const uint32_t b = b0 + r * NW;
+                if ((lane & 15) < 4 && t < nt && b < M) G[(a0 + t) * JT_STRIDE + b] += z;
+            }
+            __builtin_amdgcn_sched_barrier(0); // one batch at a time: the scheduler must not pile up the reads of all of them
+        }
+        a0 = a1;
+        __syncthreads();
+    }
+}
+
 template <bool NARROW>
 __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void join_tile_kernel(JoinArgs a) {
     a.C.narrow = NARROW ? 1u : 0u;
@@ -273,110 +388,7 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
         gram_rows_gather(a.C, row_id, R, rowptr, rownnz, tid, JT_THREADS);
         gram_rows_gather(a.C, col_id, M, rowptr + JT_ROWS, rownnz + JT_ROWS, tid, JT_THREADS);
         __syncthreads();
-        // dense part: the eight waves share the 16-column blocks that exist (8, 4, 2 or 1 by the number of columns) and, for
-        // each block, equal parts of the dimensions (1, 2, 4 or 8): no wave idles when a tile has few columns. The picker
-        // rows are staged in the table region, which is free until the sparse part. Partial tiles are added into G in a
-        // fixed order, a barrier between them.
-        {
-            const uint32_t nblk = M <= 16 ? 1u : M <= 32 ? 2u : M <= 64 ? 4u : 8u, parts = (uint32_t)NW / nblk;
-            const uint32_t blk = (uint32_t)wave % nblk, part = (uint32_t)wave / nblk;
-            const bool active = blk * 16 < M;
-            const uint32_t per = (DIM / 16) / parts; // 16-float blocks of the dimensions per part: 64, 32, 16 or 8
-            float4* A = reinterpret_cast<float4*>(smem + L.tab);
-            const uint32_t jcol = min(blk * 16 + (uint32_t)(lane & 15), M - 1);
-            const float4* pb = reinterpret_cast<const float4*>(rowptr[JT_ROWS + jcol] - DENSE_BYTES) + (lane >> 4);
-#pragma unroll 4
-            for (uint32_t i = tid; i < R * (DIM / 4); i += JT_THREADS) {
-                const uint32_t r = i / (DIM / 4), c = i % (DIM / 4);
-                A[r * (DIM / 4) + (c ^ (r & 7))] = reinterpret_cast<const float4*>(rowptr[r] - DENSE_BYTES)[c];
-            }
-            __syncthreads();
-            floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-            if (active) {
-                if (per >= 16) join_dense16<16>(A, R, pb, lane, (int)(part * per), (int)((part + 1) * per), acc0, acc1);
-                else join_dense16<8>(A, R, pb, lane, (int)(part * per), (int)((part + 1) * per), acc0, acc1);
-            }
-            auto store = [&](bool add) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float* at = &G[(4 * (lane >> 4) + e) * JT_STRIDE + blk * 16 + (lane & 15)];
-                    *at = add ? *at + a.dense_mul * acc0[e] : a.dense_mul * acc0[e];
-                    if (R > 16) {
-                        float* at1 = at + 16 * JT_STRIDE;
-                        *at1 = add ? *at1 + a.dense_mul * acc1[e] : a.dense_mul * acc1[e];
-                    }
-                }
-            };
-            for (uint32_t ph = 0; ph < parts; ph++) {
-                if (active && part == ph) store(ph != 0);
-                if (ph + 1 < parts) __syncthreads();
-            }
-        }
-        __syncthreads();
-        // sparse part: groups of eight rows in the rank table, every column probes it once per group. The pairs of a
-        // group's rows are requested while the group before it is probed; the pairs of a wave's columns stay in its
-        // registers for the whole tile: a build and the probes find their operands there.
-        auto row_pairs = [&](uint32_t i) { Pairs p = gram_row(a.C, rowptr, rownnz, i); p.narrow = NARROW ? 1u : 0u; return p; };
-        auto col_pairs = [&](uint32_t b) { Pairs p = gram_row(a.C, rowptr + JT_ROWS, rownnz + JT_ROWS, b); p.narrow = NARROW ? 1u : 0u; return p; };
-        uint32_t a0 = 0;
-        PivotRegs pv;
-        ranktab_pivots_load(pv, [&](uint32_t t) { return row_pairs(a0 + t); }, min((uint32_t)RT_T, R - a0), tid, JT_THREADS);
-        // the wave's columns wave, wave + NW, ...: read once per tile, probed once per group; their shapes
-        // (nnz | ns << 16) are wave-uniform and stay in scalar registers
-        RtRow<NARROW> own[JT_OWN];
-        uint32_t own_shape[JT_OWN];
-#pragma unroll
-        for (int k = 0; k < JT_OWN; k++) {
-            const uint32_t b = wave + k * NW;
-            own_shape[k] = 0;
-            if (b < M) {
-                own_shape[k] = uniform(rownnz[JT_ROWS + b]);
-                rt_row_load(own[k], col_pairs(b), lane);
-            }
-        }
-        while (a0 < R) {
-            uint32_t nt = min((uint32_t)RT_T, R - a0);
-            uint32_t built;
-            while (true) {
-                built = ranktab_build<NARROW>(T, [&](uint32_t t) { return row_pairs(a0 + t); }, pv, nt, scan, tid, JT_THREADS);
-                if (built != EMPTY || nt == 1) break;
-                nt = (nt + 1) / 2; // the registers hold the first pivots of the group whatever nt is
-            }
-            const uint32_t a1 = a0 + nt;
-            if (a1 < R) ranktab_pivots_load(pv, [&](uint32_t t) { return row_pairs(a1 + t); }, min((uint32_t)RT_T, R - a1), tid, JT_THREADS);
-            if (built == EMPTY) { // one row alone does not fit: its sparse part is missing, the host is told
-                if (tid == 0) atomicAdd(a.work + 3, 1ull);
-                a0 = a1;
-                continue;
-            }
-            const uint32_t n_ovf = NARROW ? 0u : uniform(min(scan[16], (uint32_t)RT_OVF));
-#pragma unroll
-            for (int q = 0; q < JT_OWN / JT_BATCH; q++) {
-                const uint32_t b0 = wave + q * JT_BATCH * NW;
-                if (b0 < M) { // wave-uniform
-                    float acc[JT_BATCH][RT_T];
-                    RtRow<NARROW> rows[JT_BATCH];
-                    uint32_t shape[JT_BATCH];
-#pragma unroll
-                    for (int k = 0; k < JT_BATCH; k++) {
-                        rows[k] = own[q * JT_BATCH + k];
-                        rows[k].touch();
-                        shape[k] = own_shape[q * JT_BATCH + k];
-                        asm volatile("" : "+s"(shape[k])); // as touch(): the lane masks of a row are made where they are used
-#pragma unroll
-                        for (int t = 0; t < RT_T; t++) acc[k][t] = 0.f;
-                    }
-                    ranktab_probe_rows<NARROW, JT_BATCH>(T, rows, shape, [&](int k) { return col_pairs(b0 + k * NW); }, n_ovf, acc, lane);
-                    uint32_t t, r;
-                    const float z = wave_sum_2x8(acc, lane, &t, &r);
-                    const uint32_t b = b0 + r * NW;
-                    if ((lane & 15) < 4 && t < nt && b < M) G[(a0 + t) * JT_STRIDE + b] += z;
-                }
-                __builtin_amdgcn_sched_barrier(0); // one batch at a time: the scheduler must not pile up the reads of all of them
-            }
-            a0 = a1;
-            __syncthreads();
-        }
+        tile_hybrid_ips<NARROW>(a.C, a.dense_mul, smem + L.tab, T, a.index_bits, a.slot_cap, G, rowptr, rownnz, scan, R, M, a.work + 3, tid, wave, lane);
         // proposals
         for (uint32_t p = tid; p < R * M; p += JT_THREADS) {
             const uint32_t r = p / M, c = p % M;
@@ -510,6 +522,84 @@ __global__ __launch_bounds__(256) static void fill_u32_kernel2(uint32_t* p, uint
     for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < count; t += (uint64_t)gridDim.x * blockDim.x) p[t] = v;
 }
 
+// ---- hybrid Gram matrices of whole neighbour lists, tile by tile (the prune of lists longer than 64 entries) ----
+//
+// For node u = node0 + q / GT_PER_NODE the valid entries of its list (distance below INF_DIS, a document, not u itself),
+// in list order, are the rows and columns of a Gram matrix of at most 128 x 128. Tile t = q % GT_PER_NODE computes rows
+// [32 t, 32 t + 32) against the columns [32 t, m): the upper triangle, diagonal blocks whole. The products go to
+// gram[(q / GT_PER_NODE) * 128 * 128 + i * 128 + j] for i <= j (entries below the diagonal of a diagonal block are
+// written too). Same tile body as the local join: every row of a tile is gathered once, dense part on the matrix cores,
+// sparse part through the rank table.
+constexpr uint32_t GT_MAX = 128;                 // longest list
+constexpr uint32_t GT_PER_NODE = GT_MAX / JT_ROWS; // tiles per node
+struct GramTileArgs {
+    CorpusView C;
+    float dense_mul;
+    uint32_t K, node0, n_nodes;
+    const uint32_t* ids;
+    const float* dist;
+    float* gram;
+    unsigned long long* work; // [0] next tile, [3] a row did not fit the table
+    uint32_t index_bits, slot_cap, span;
+};
+
+template <bool NARROW>
+__global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void gram_tile_kernel(GramTileArgs a) {
+    a.C.narrow = NARROW ? 1u : 0u;
+    extern __shared__ __align__(16) char smem[];
+    const JoinLds L(a.index_bits, a.slot_cap, NARROW);
+    const RankTab T = ranktab_at(smem + L.tab, a.index_bits, a.slot_cap, a.span, NARROW);
+    float* G = reinterpret_cast<float*>(smem + L.G);
+    unsigned long long* rowptr = reinterpret_cast<unsigned long long*>(smem + L.rowptr);
+    uint32_t* rownnz = reinterpret_cast<uint32_t*>(smem + L.rownnz);
+    uint32_t* row_id = reinterpret_cast<uint32_t*>(smem + L.row_id);
+    uint32_t* col_id = reinterpret_cast<uint32_t*>(smem + L.col_id);
+    uint32_t* valid = reinterpret_cast<uint32_t*>(smem + L.seen); // the node's valid list entries, in list order
+    uint32_t* scan = reinterpret_cast<uint32_t*>(smem + L.scan);
+    volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl); // [0] tile, [1] valid entries
+    static_assert(JT_SEEN >= (int)GT_MAX, "the id set's words hold a whole list");
+    const int tid = threadIdx.x, wave = (int)uniform(tid / WAVE), lane = lane_id();
+    const uint32_t n_tiles = a.n_nodes * GT_PER_NODE;
+    const uint64_t lane_lt = (1ull << lane) - 1;
+    while (true) {
+        __syncthreads();
+        if (tid == 0) ctl[0] = (uint32_t)atomicAdd(a.work, 1ull);
+        __syncthreads();
+        const uint32_t q = uniform(ctl[0]);
+        if (q >= n_tiles) break;
+        const uint32_t slot = q / GT_PER_NODE, t = q % GT_PER_NODE, u = a.node0 + slot;
+        if (wave == 0) {
+            const size_t base = (size_t)u * a.K;
+            uint32_t m = 0;
+            for (uint32_t b0 = 0; b0 < a.K; b0 += WAVE) {
+                const uint32_t v = (a.ids[base + b0 + lane] & ~FLAG);
+                const float dv = a.dist[base + b0 + lane];
+                const bool ok = dv < INF_DIS && v < a.C.n && v != u;
+                const uint64_t b = __ballot(ok);
+                if (ok) valid[m + __popcll(b & lane_lt)] = v;
+                m += __popcll(b);
+            }
+            if (lane == 0) ctl[1] = m;
+        }
+        __syncthreads();
+        const uint32_t m = uniform(ctl[1]), r0 = t * JT_ROWS;
+        if (r0 >= m) continue;
+        const uint32_t R = min((uint32_t)JT_ROWS, m - r0), M = m - r0;
+        if ((uint32_t)tid < R) row_id[tid] = valid[r0 + tid];
+        if ((uint32_t)tid < M) col_id[tid] = valid[r0 + tid];
+        __syncthreads();
+        gram_rows_gather(a.C, row_id, R, rowptr, rownnz, tid, JT_THREADS);
+        gram_rows_gather(a.C, col_id, M, rowptr + JT_ROWS, rownnz + JT_ROWS, tid, JT_THREADS);
+        __syncthreads();
+        tile_hybrid_ips<NARROW>(a.C, a.dense_mul, smem + L.tab, T, a.index_bits, a.slot_cap, G, rowptr, rownnz, scan, R, M, a.work + 3, tid, wave, lane);
+        float* out = a.gram + (size_t)slot * GT_MAX * GT_MAX;
+        for (uint32_t p = tid; p < R * M; p += JT_THREADS) {
+            const uint32_t r = p / M, c = p % M;
+            out[(size_t)(r0 + r) * GT_MAX + r0 + c] = G[r * JT_STRIDE + c];
+        }
+    }
+}
+
 static void join_table_shape(const apoe_corpus* c, uint32_t* index_bits, uint32_t* slot_cap, uint32_t* span) {
     *span = next_pow2(std::max(c->max_term + 1, 1024u));
     *index_bits = c->narrow ? 2 * *span : 65536u;
@@ -594,6 +684,56 @@ int launch_nnd_join_iterate(apoe_knn* g) {
     join_account_kernel<<<1, 1, 0, st>>>(g->join_work.p, g->counter.p);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
+}
+
+// Gram matrices (upper triangles) of the lists of nodes [node0, node0 + n_nodes) into gram[n_nodes][128][128]. *unfit = rows
+// whose sparse terms did not fit the tile's table (their products lack the sparse part: the caller must not use the result).
+int launch_gram_tiles(apoe_knn* g, uint32_t node0, uint32_t n_nodes, float* gram, unsigned long long* unfit) {
+    apoe_ctx* ctx = g->ctx;
+    hipStream_t st = ctx->stream;
+    APOE_REQUIRE(g->K <= GT_MAX, "Gram tiles are built for lists of at most %u entries", GT_MAX);
+    if (!g->join_work.p) APOE_TRY(g->join_work.alloc(JOIN_COUNT_AT + JOIN_COUNT_PARTS * 8));
+    uint32_t index_bits, slot_cap, span;
+    join_table_shape(g->corpus, &index_bits, &slot_cap, &span);
+    const JoinLds L(index_bits, slot_cap, g->corpus->narrow);
+    APOE_REQUIRE(L.total <= ctx->lds_per_block, "a Gram tile needs %u bytes of LDS, a workgroup may have %zu", L.total, ctx->lds_per_block);
+    fill_u64_kernel<<<1, 64, 0, st>>>(g->join_work.p, 8, 0ull);
+    APOE_HIP(hipGetLastError());
+    GramTileArgs a{};
+    a.C = g->corpus->view();
+    a.dense_mul = g->dense_scale * g->dense_scale;
+    a.K = g->K;
+    a.node0 = node0;
+    a.n_nodes = n_nodes;
+    a.ids = g->ids.p;
+    a.dist = g->dist.p;
+    a.gram = gram;
+    a.work = g->join_work.p;
+    a.index_bits = index_bits;
+    a.slot_cap = slot_cap;
+    a.span = span;
+    auto kernel = g->corpus->narrow ? &gram_tile_kernel<true> : &gram_tile_kernel<false>;
+    APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
+    int per_cu = 1;
+    APOE_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), JT_THREADS, L.total));
+    if (per_cu < 1) per_cu = 1;
+    kernel<<<(uint32_t)per_cu * (uint32_t)ctx->num_cus, JT_THREADS, L.total, st>>>(a);
+    APOE_HIP(hipGetLastError());
+    if (unfit) {
+        unsigned long long h[4] = {0, 0, 0, 0};
+        APOE_HIP(hipMemcpyAsync(h, g->join_work.p, sizeof(h), hipMemcpyDeviceToHost, st));
+        APOE_HIP(hipStreamSynchronize(st));
+        *unfit = h[3];
+    }
+    return APOE_OK;
+}
+
+// Whether launch_gram_tiles can serve this handle: lists of at most 128 entries, rows that fit a tile's table, LDS for a tile.
+bool gram_tiles_fit(const apoe_knn* g) {
+    if (g->K > GT_MAX || g->corpus->max_nnz_s + g->corpus->max_nnz_b > (uint32_t)APOE_JOIN_MAX_ROW_TERMS) return false;
+    uint32_t index_bits, slot_cap, span;
+    join_table_shape(g->corpus, &index_bits, &slot_cap, &span);
+    return JoinLds(index_bits, slot_cap, g->corpus->narrow).total <= g->ctx->lds_per_block;
 }
 
 // Pairs evaluated and rows gathered by the tiles of the last step, and whether a row did not fit the table.

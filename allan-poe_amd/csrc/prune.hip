@@ -239,6 +239,244 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
     if (tid == 0) cnt_out[u] = ctl[PC_CNT];
 }
 
+// ---- the prune on a Gram matrix that the tile kernel of join.hip has left in memory (lists of up to 128 entries) ----
+
+constexpr uint32_t PS_MAX = 128;            // longest list
+constexpr uint32_t PS_STRIDE = PS_MAX + 1;  // odd stride: a column read does not collide on the LDS banks
+constexpr int PS_THREADS = 256;
+
+struct SelectLds {
+    uint32_t G, idmap, umap, R, nb_id, nb_dist, nrm, det, order, o_fwd, o_det, o_kw, ctl, total;
+    __host__ __device__ SelectLds(uint32_t umap_slots, uint32_t map_slots, uint32_t words) {
+        uint32_t o = 0;
+        G = o; o += PS_MAX * PS_STRIDE * 4;
+        o = (o + 7) & ~7u;
+        idmap = o; o += map_slots * 8;
+        umap = o; o += umap_slots * 8;
+        R = o; o += PS_MAX * words * 4;
+        nb_id = o; o += PS_MAX * 4;
+        nb_dist = o; o += PS_MAX * 4;
+        nrm = o; o += PS_MAX * 4;
+        det = o; o += PS_MAX * 4;
+        order = o; o += PS_MAX * 4;
+        o_fwd = o; o += PS_MAX * 4;
+        o_det = o; o += PS_MAX * 4;
+        o_kw = o; o += (1 + APOE_KW_CAND) * 4;
+        ctl = o; o += 16 * 4;
+        total = o;
+    }
+};
+
+// allan_poe (index.cu:539-714) for node u = node0 + blockIdx.x, as prune_kernel, with every inner product <c, s> read from the
+// node's Gram matrix gram[blockIdx.x][i][j] (i <= j: positions in the list of valid entries) instead of being evaluated:
+// detour counts and the (detour, rank) order as there; the keyword flag of a pair from bit masks R[i] = the BM25 terms of u
+// that row i holds (flag(c, s) = R[s] has a bit that R[c] lacks); the sequential selection by wave 0 alone on the LDS copy of
+// the matrix, two selected members per lane (slots `lane` and `lane + 64` of the selection order).
+__global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, const float* __restrict__ norms, uint32_t K, const uint32_t* __restrict__ ids,
+                                                                  const float* __restrict__ dist, uint32_t d, uint32_t node0, const float* __restrict__ gram,
+                                                                  uint32_t* fwd, uint32_t* det_out, uint32_t* cnt_out, uint32_t* kw_out, uint32_t umap_slots,
+                                                                  uint32_t map_slots, uint32_t words) {
+    extern __shared__ __align__(16) char smem[];
+    const SelectLds L(umap_slots, map_slots, words);
+    float* G = reinterpret_cast<float*>(smem + L.G);
+    uint2* idmap = reinterpret_cast<uint2*>(smem + L.idmap);
+    uint2* umap = reinterpret_cast<uint2*>(smem + L.umap);
+    uint32_t* R = reinterpret_cast<uint32_t*>(smem + L.R);
+    uint32_t* nb_id = reinterpret_cast<uint32_t*>(smem + L.nb_id);
+    float* nb_dist = reinterpret_cast<float*>(smem + L.nb_dist);
+    float* nrm = reinterpret_cast<float*>(smem + L.nrm);
+    uint32_t* det = reinterpret_cast<uint32_t*>(smem + L.det);
+    uint32_t* order = reinterpret_cast<uint32_t*>(smem + L.order);
+    uint32_t* o_fwd = reinterpret_cast<uint32_t*>(smem + L.o_fwd);
+    uint32_t* o_det = reinterpret_cast<uint32_t*>(smem + L.o_det);
+    uint32_t* o_kw = reinterpret_cast<uint32_t*>(smem + L.o_kw);
+    volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
+
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const uint32_t u = node0 + blockIdx.x, umask = umap_slots - 1, mmask = map_slots - 1;
+    const size_t base = (size_t)u * K;
+    const uint64_t lane_lt = (1ull << lane) - 1;
+    const float* gu = gram + (size_t)blockIdx.x * PS_MAX * PS_MAX;
+
+    for (uint32_t i = tid; i < map_slots; i += PS_THREADS) idmap[i] = make_uint2(EMPTY, 0u);
+    for (uint32_t i = tid; i < umap_slots; i += PS_THREADS) umap[i] = make_uint2(EMPTY, 0u);
+    for (uint32_t i = tid; i < PS_MAX * words; i += PS_THREADS) R[i] = 0;
+    for (uint32_t i = tid; i < PS_MAX; i += PS_THREADS) det[i] = 0;
+    if (tid < 16) ctl[tid] = 0;
+    __syncthreads();
+    // valid list entries, in list order (the rows and columns of the Gram matrix)
+    if (wave == 0) {
+        uint32_t m = 0;
+        for (uint32_t b0 = 0; b0 < K; b0 += WAVE) {
+            const uint32_t v = ids[base + b0 + lane] & ~FLAG;
+            const float dv = dist[base + b0 + lane];
+            const bool ok = dv < INF_DIS && v < C.n && v != u;
+            const uint64_t b = __ballot(ok);
+            if (ok) {
+                const uint32_t pos = m + __popcll(b & lane_lt);
+                nb_id[pos] = v;
+                nb_dist[pos] = dv;
+                nrm[pos] = norms[v];
+            }
+            m += __popcll(b);
+        }
+        if (lane == 0) ctl[PC_M] = m;
+    }
+    {   // u's BM25 terms -> their index in u's row
+        const uint64_t du = C.desc[u];
+        const Pairs sp = record_pairs(C, du);
+        const uint32_t ns = desc_nnz_s(du), nb = desc_nnz_b(du);
+        for (uint32_t j = tid; j < nb; j += PS_THREADS) {
+            const uint32_t key = sp.key(ns + j);
+            uint32_t h = term_hash(key, umask);
+            while (true) {
+                const uint32_t old = atomicCAS(&umap[h].x, EMPTY, key);
+                if (old == EMPTY) { umap[h].y = j; break; }
+                if (old == key) break;
+                h = (h + 1) & umask;
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t m = ctl[PC_M];
+    // the Gram matrix: rows of the upper triangle, as the tiles wrote them
+    for (uint32_t t = tid; t < m * PS_MAX; t += PS_THREADS) {
+        const uint32_t i = t / PS_MAX, j = t % PS_MAX;
+        if (j >= i && j < m) G[i * PS_STRIDE + j] = gu[(size_t)i * PS_MAX + j];
+    }
+    // (a) detour counts
+    for (uint32_t i = tid; i < m; i += PS_THREADS) {
+        const uint32_t key = nb_id[i];
+        uint32_t h = term_hash(key, mmask);
+        while (true) {
+            const uint32_t old = atomicCAS(&idmap[h].x, EMPTY, key);
+            if (old == EMPTY) { idmap[h].y = i; break; }
+            if (old == key) break;
+            h = (h + 1) & mmask;
+        }
+    }
+    // R[r] = bits of u's BM25 terms that row r holds too: one wave per row, lanes over its BM25 pairs
+    for (uint32_t r = wave; r < m; r += PS_THREADS / WAVE) {
+        const uint64_t dr = C.desc[nb_id[r]];
+        const Pairs sp = record_pairs(C, dr);
+        const uint32_t ns = desc_nnz_s(dr), nb = desc_nnz_b(dr);
+        for (uint32_t j = lane; j < nb; j += WAVE) {
+            const uint32_t key = sp.key(ns + j);
+            uint32_t h = term_hash(key, umask);
+            while (true) {
+                const uint2 e = umap[h];
+                if (e.x == key) { atomicOr(&R[r * words + (e.y >> 5)], 1u << (e.y & 31)); break; }
+                if (e.x == EMPTY) break;
+                h = (h + 1) & umask;
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t t = tid; t < m * K; t += PS_THREADS) {
+        const uint32_t r = t / K, j = t % K;
+        const size_t at = (size_t)nb_id[r] * K + j;
+        const uint32_t x = ids[at] & ~FLAG;
+        const float dx = dist[at];
+        uint32_t h = term_hash(x, mmask);
+        while (true) {
+            const uint2 e = idmap[h];
+            if (e.x == x) {
+                if (e.y > r && dx < nb_dist[e.y]) atomicAdd(&det[e.y], 1u);
+                break;
+            }
+            if (e.x == EMPTY) break;
+            h = (h + 1) & mmask;
+        }
+    }
+    __syncthreads();
+    // (b) stable order by detour count
+    for (uint32_t i = tid; i < m; i += PS_THREADS) {
+        const uint32_t key = (det[i] << 16) | i;
+        uint32_t r = 0;
+        for (uint32_t j = 0; j < m; j++) r += ((det[j] << 16) | j) < key;
+        order[r] = i;
+    }
+    __syncthreads();
+    // (c)+(d) sequential selection, wave 0: member k of the selection order lives in slot k / 64 of lane k % 64
+    if (wave == 0) {
+        uint32_t gi[2] = {0, 0}, kw[2] = {0, 0}; // Gram index (position in the list) and keyword flag of the member
+        bool live[2] = {false, false};
+        float mn[2] = {0.f, 0.f};
+        uint32_t n_sel = 0;
+        if (m > 0) {
+            const uint32_t c0 = order[0];
+            if (lane == 0) { gi[0] = c0; live[0] = true; mn[0] = nrm[c0]; }
+            n_sel = 1;
+        }
+        for (uint32_t t = 1; t < m; t++) {
+            const uint32_t c = order[t];
+            const float norm_c = nrm[c];
+            bool rej = false, noflag = false;
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                const bool act = (uint32_t)lane + 64u * s < n_sel && live[s];
+                if (act) {
+                    const uint32_t lo = min(c, gi[s]), hi = max(c, gi[s]);
+                    const float p = G[lo * PS_STRIDE + hi];
+                    bool flag = false;
+                    for (uint32_t w = 0; w < words; w++) flag |= (R[gi[s] * words + w] & ~R[c * words + w]) != 0;
+                    rej |= norm_c < p;
+                    if (mn[s] < p) live[s] = false;
+                    noflag |= !flag;
+                }
+            }
+            const bool reject = __ballot(rej) != 0;
+            const bool allflag = __ballot(noflag) == 0;
+            if (!reject) {
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+                    if ((uint32_t)lane + 64u * s == n_sel) { gi[s] = c; live[s] = true; mn[s] = norm_c; kw[s] = allflag ? 1u : 0u; }
+                }
+                n_sel++;
+            }
+        }
+        // (e) emit: live members in selection order fill the row, flagged ones beyond d become keyword candidates
+        uint32_t seen_live = 0, seen_kw = 0;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const bool lv = (uint32_t)lane + 64u * s < n_sel && live[s];
+            const uint64_t lb = __ballot(lv);
+            const uint32_t pos = seen_live + __popcll(lb & lane_lt);
+            if (lv && pos < d) { o_fwd[pos] = nb_id[gi[s]]; o_det[pos] = det[gi[s]]; }
+            const bool kwc = lv && pos >= d && kw[s];
+            const uint64_t kb = __ballot(kwc);
+            const uint32_t kpos = seen_kw + __popcll(kb & lane_lt);
+            if (kwc && kpos < APOE_KW_CAND) o_kw[1 + kpos] = nb_id[gi[s]];
+            seen_live += __popcll(lb);
+            seen_kw += __popcll(kb);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (lane == 0) {
+            uint32_t cnt = min(seen_live, d);
+            const uint32_t nkw = min(seen_kw, (uint32_t)APOE_KW_CAND);
+            // fewer survivors than the row has slots: the remaining neighbours in order, each id once, then the node itself
+            for (uint32_t t = 0; t < m && cnt < d; t++) {
+                const uint32_t cidx = order[t], cid = nb_id[cidx];
+                bool present = false;
+                for (uint32_t j = 0; j < cnt; j++) present |= o_fwd[j] == cid;
+                if (!present) { o_fwd[cnt] = cid; o_det[cnt] = det[cidx]; cnt++; }
+            }
+            ctl[PC_CNT] = cnt;
+            for (; cnt < d; cnt++) { o_fwd[cnt] = u; o_det[cnt] = EMPTY; }
+            o_kw[0] = nkw;
+            for (uint32_t j = nkw; j < APOE_KW_CAND; j++) o_kw[1 + j] = 0;
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < d; i += PS_THREADS) {
+        fwd[(size_t)u * d + i] = o_fwd[i];
+        det_out[(size_t)u * d + i] = o_det[i];
+    }
+    for (uint32_t i = tid; i < 1 + APOE_KW_CAND; i += PS_THREADS) kw_out[(size_t)u * (1 + APOE_KW_CAND) + i] = o_kw[i];
+    if (tid == 0) cnt_out[u] = ctl[PC_CNT];
+}
+
 // ---- gather-once form of the prune (K = 64) ----
 
 #ifdef APOE_PRUNE_TIMING
@@ -896,6 +1134,28 @@ int launch_prune(apoe_knn* g, uint32_t degree) {
         if (!failed) return APOE_OK;
         // a row's terms clustered on the same table slots: redo with the table-probing kernel below
     }
+    // lists longer than 64 entries: Gram matrices by the tile kernel of the local join, a batch of nodes at a time, and the
+    // selection on them; a row too long for a tile's table sends the whole prune to the table-probing kernel below
+    if (g->K > GRAM_ROWS && g->K <= PS_MAX && !g->force_sequential_prune && gram_tiles_fit(g)) {
+        const SelectLds SL(uset_slots, map_slots, words);
+        if (SL.total <= ctx->lds_per_block) {
+            const uint32_t batch = std::min<uint32_t>(g->n, 32768u);
+            DevBuf<float> gram;
+            APOE_TRY(gram.alloc((size_t)batch * PS_MAX * PS_MAX));
+            APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&prune_select_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)SL.total));
+            unsigned long long unfit = 0;
+            for (uint32_t node0 = 0; node0 < g->n && !unfit; node0 += batch) {
+                const uint32_t cnt = std::min(batch, g->n - node0);
+                APOE_TRY(launch_gram_tiles(g, node0, cnt, gram.p, &unfit));
+                if (unfit) break;
+                prune_select_kernel<<<cnt, PS_THREADS, SL.total, ctx->stream>>>(g->corpus->view(), g->norms.p, g->K, g->ids.p, g->dist.p, degree, node0, gram.p,
+                                                                              g->fwd.p, g->det.p, g->cnt.p, g->kw.p, uset_slots, map_slots, words);
+                APOE_HIP(hipGetLastError());
+            }
+            APOE_HIP(hipStreamSynchronize(ctx->stream)); // the batch buffer is freed on return
+            if (!unfit) return APOE_OK;
+        }
+    }
     const PruneLds L(term_slots, uset_slots, map_slots, g->K);
     APOE_REQUIRE(L.total <= 64 * 1024, "prune needs %u bytes of LDS (rows with up to %u sparse terms)", L.total,
                  g->corpus->max_nnz_s + g->corpus->max_nnz_b);
@@ -947,6 +1207,13 @@ int apoe_debug_prune_ticks(unsigned long long* out16) {
     return 0;
 }
 #endif
+
+int apoe_knn_set_prune_form(apoe_knn* g, int form) {
+    APOE_REQUIRE(g, "null argument");
+    APOE_REQUIRE(form == 0 || form == 1, "prune form must be 0 (gather-once forms where they apply) or 1 (the table-probing kernel), got %d", form);
+    g->force_sequential_prune = form == 1;
+    return APOE_OK;
+}
 
 int apoe_prune(apoe_knn* g, uint32_t degree) {
     APOE_REQUIRE(g, "null argument");

@@ -167,6 +167,14 @@ int apoe_knn_upload(apoe_knn* g, const uint32_t* ids, const float* dist);
  * ids must name a document or be 0xFFFFFFFF. */
 int apoe_knn_download_reverse(apoe_knn* g, uint32_t* rev_ids, float* rev_dist, uint32_t* rev_cnt);
 int apoe_knn_upload_reverse(apoe_knn* g, const uint32_t* rev_ids, const float* rev_dist, const uint32_t* rev_cnt);
+/* Which form of the prune apoe_prune runs (all replace allan_poe, index.cu:539-714, and give the same rows):
+ *   0  (default) the forms that gather every neighbour row once: for K = 64 one workgroup builds the node's hybrid Gram
+ *      matrix in LDS and selects on it; for K = 128 the Gram matrices of a batch of nodes are computed by the tile kernel
+ *      of the local join (32 rows x up to 128 columns of a list at a time) into device memory and a second kernel selects
+ *      on them. A corpus whose rows do not fit the tables of these forms falls back to form 1 by itself;
+ *   1  the table-probing kernel: the candidate is the pivot, one wave per live selected member evaluates its product,
+ *      rows are read again at every selection step (what the reference does). */
+int apoe_knn_set_prune_form(apoe_knn* g, int form);
 /* allan_poe (index.cu:539-714): RNG-IP prune to `degree` + keyword-edge candidates. */
 int apoe_prune(apoe_knn* g, uint32_t degree);
 /* Intermediate result of apoe_prune: fwd/det [n][degree], cnt [n], kw [n][1+APOE_KW_CAND]. */

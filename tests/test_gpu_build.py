@@ -288,8 +288,10 @@ def test_prune_of_short_and_ragged_lists_matches_oracle(gpu_world):
     assert np.all(g_fwd == c_fwd, axis=1).mean() >= 0.995
 
 
-def test_prune_k128_sequential_kernel_matches_oracle(gpu_world):
-    """K = 128 lists go through the table-probing prune kernel (the gather-once form is K = 64 only)."""
+@pytest.mark.parametrize("form", [0, 1])
+def test_prune_k128_matches_oracle(gpu_world, form):
+    """K = 128 lists: form 0 = Gram matrices by the tile kernel of the local join + selection on them, form 1 = the
+    table-probing prune kernel. Both against the oracle on the oracle's own lists, and the final rows from them."""
     import apoe
     import oracle as O
     w = gpu_world
@@ -300,14 +302,23 @@ def test_prune_k128_sequential_kernel_matches_oracle(gpu_world):
         if it < 3:
             st.rev_cnt[:] = 0
     ids, dist = st.ids & 0x7FFFFFFF, st.dist.copy()
+    # a few short and ragged lists too: 0, 1, 31, 32, 33, 65 and 127 usable entries
+    rng = np.random.default_rng(5)
+    counts = (0, 1, 31, 32, 33, 65, 127)
+    nodes = rng.choice(C.n, size=10 * len(counts), replace=False)
+    for i, u in enumerate(nodes):
+        dist[u, counts[i % len(counts)]:] = apoe.INF_DIS
     knn = apoe.Knn(w["ctx"], w["gc"], 128, 7.0)
+    knn.set_prune_form(form)
     knn.upload(ids, dist)
     knn.prune(64)
     g_fwd, g_det, g_cnt, g_kw = knn.prune_download()
     c_fwd, c_det, c_cnt, c_kw = O.prune(C, 7.0, O.norms(C, 7.0), ids, dist, 64)
     same = np.all(g_fwd == c_fwd, axis=1)
     assert same.mean() >= 0.995
+    assert np.all(g_fwd[nodes] == c_fwd[nodes], axis=1).mean() >= 0.97
     assert np.array_equal(g_det[same], c_det[same]) and np.array_equal(g_cnt[same], c_cnt[same])
+    assert np.all(g_kw == c_kw, axis=1)[same].mean() >= 0.995
     graph = knn.finalize()
     rows, entry = graph.download()
     assert np.array_equal(rows, O.final_graph(g_fwd, g_det, g_cnt, g_kw))

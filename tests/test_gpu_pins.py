@@ -10,15 +10,16 @@ import pin_worlds as P
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("K", [64, 128])  # 64: gather-once prune on the Gram matrix; 128: sequential prune kernel
+@pytest.mark.parametrize("K,form", [(64, 0), (64, 1), (128, 0), (128, 1)])  # form 0: the gather-once prunes (Gram matrix in LDS / by tiles), 1: table-probing kernel
 @pytest.mark.parametrize("term_shift", [0, 70000])  # narrow and wide pair format of the device records
-def test_keyword_flag_world(gpu_ctx, K, term_shift):
+def test_keyword_flag_world(gpu_ctx, K, form, term_shift):
     import apoe
     import oracle as O
     arrays, ids, dist, expect = P.keyword_flag_world(K=K, term_shift=term_shift)
     gc = apoe.Corpus(gpu_ctx, *arrays)
     assert gc.pair_bytes() == (8 if term_shift else 6)
     knn = apoe.Knn(gpu_ctx, gc, K, 7.0)
+    knn.set_prune_form(form)
     knn.upload(ids, dist)
     knn.prune(expect["d"])
     fwd, det, cnt, kw = knn.prune_download()
