@@ -289,11 +289,25 @@ void build_index_impl(const std::string& dense_data_path, const std::string& spa
         }
         unsigned info[4] = {0, 0, 0, 0};
         check(apoe_corpus_info(h.corpus, info), "apoe_corpus_info");
-        const bool rows_fit = info[2] + info[3] <= APOE_JOIN_MAX_ROW_TERMS; // longest SPLADE row + longest BM25 row
-        const int join = opt.nnd_join >= 0 ? opt.nnd_join : (opt.nnd_k == 64 && !opt.half_rows && rows_fit ? 1 : 0);
-        if (join) check(apoe_knn_set_join(h.knn, join), "apoe_knn_set_join");
-        check(apoe_nnd_init(h.knn, opt.seed), "apoe_nnd_init");
-        for (unsigned it = 0; it < opt.nnd_iters; it++) check(apoe_nnd_iterate(h.knn, it + 1 == opt.nnd_iters, nullptr), "apoe_nnd_iterate");
+        // nnd_join < 0: the local join where its tile holds every row. A corpus in the wide pair format hashes a row's terms
+        // into the tile's table, which takes rows of about a thousand terms safely; beyond that, and if a step still meets a
+        // row that it cannot hold, the build runs (again) with the expansion step.
+        const unsigned longest = info[2] + info[3]; // longest SPLADE row + longest BM25 row
+        const bool wide = apoe_corpus_pair_bytes(h.corpus) == 8;
+        const bool rows_fit = longest <= (wide ? 1024u : (unsigned)APOE_JOIN_MAX_ROW_TERMS);
+        int join = opt.nnd_join >= 0 ? opt.nnd_join : (!opt.half_rows && rows_fit ? 1 : 0);
+        while (true) {
+            check(apoe_knn_set_join(h.knn, join), "apoe_knn_set_join");
+            check(apoe_nnd_init(h.knn, opt.seed), "apoe_nnd_init");
+            int status = APOE_OK;
+            for (unsigned it = 0; it < opt.nnd_iters && status == APOE_OK; it++) status = apoe_nnd_iterate(h.knn, it + 1 == opt.nnd_iters, nullptr);
+            if (status == APOE_ERR_STATE && join != 0 && opt.nnd_join < 0) { // a row did not fit the join's table
+                join = 0;
+                continue;
+            }
+            check(status, "apoe_nnd_iterate");
+            break;
+        }
         check(apoe_nnd_merge_reverse(h.knn), "apoe_nnd_merge_reverse");
     }
     if (!opt.knn_save_path.empty()) {

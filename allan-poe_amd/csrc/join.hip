@@ -35,16 +35,11 @@ constexpr int JT_COLS = 128;
 constexpr int JT_THREADS = 512;
 constexpr int JT_STRIDE = JT_COLS + 1;
 constexpr int JT_SEEN = 512; // slots of the id set that removes repeated columns
-constexpr uint32_t JOIN_K = 64;
-#ifndef APOE_JOIN_PICKS
-#define APOE_JOIN_PICKS 4
-#endif
-constexpr int JOIN_PICKS = APOE_JOIN_PICKS; // index.cu:157,171-181
-#ifndef APOE_JOIN_SLOTS
-#define APOE_JOIN_SLOTS 128
-#endif
-constexpr uint32_t JOIN_P = APOE_JOIN_SLOTS; // proposal slots per node (64 or 128): two proposals whose ids hash to one slot are one proposal, the closer one
-constexpr int JOIN_PL = JOIN_P / WAVE; // ... per lane of the wave that merges them
+// The kernels below are built for lists of KK = 64 and KK = 128 entries (index.cu:6 has K 64; a degree above 32 needs
+// 2 * degree <= K there, index.cu:702). A node has 2 * KK proposal slots: two proposals of one step whose ids hash to one
+// slot are one proposal, the closer one. With KK = 128 the columns of a picked node (its list and its reverse list, up to
+// 256) are two tiles: the list, then what the reverse list adds to it.
+constexpr int JOIN_PICKS = 4; // index.cu:157,171-181
 constexpr int JOIN_COUNT_PARTS = 256, JOIN_COUNT_AT = 8; // partial insertion counters in the step's work array, one per 64-byte line, from word 8
 constexpr int JT_BATCH = 2;   // column rows a wave probes together
 constexpr int JT_OWN = JT_COLS / (JT_THREADS / WAVE); // columns of a tile that one wave owns: their pairs stay in its registers
@@ -59,28 +54,43 @@ __device__ __forceinline__ float join_key_dist(unsigned long long key) {
 
 // One wave per node: the picking rule of the expansion step (group g takes the first unsampled slot >= g; none
 // left: slot 0 again), the picked neighbours counted per target.
+template <uint32_t KK>
 __global__ __launch_bounds__(256) void join_pick_kernel(uint32_t n, uint32_t* ids, uint32_t* picks, uint32_t* pick_cnt) {
+    constexpr int KL = KK / WAVE; // list entries per lane: entry e sits in register e / 64 of lane e % 64
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const uint32_t u = blockIdx.x * 4 + wave;
     if (u >= n) return;
-    const size_t base = (size_t)u * JOIN_K;
-    const uint32_t own = ids[base + lane];
-    uint64_t m0 = __ballot(!(own & FLAG));
+    const size_t base = (size_t)u * KK;
+    uint32_t own[KL];
+    uint64_t m0[KL];
+#pragma unroll
+    for (int k = 0; k < KL; k++) {
+        own[k] = ids[base + k * WAVE + lane];
+        m0[k] = __ballot(!(own[k] & FLAG));
+    }
     uint32_t slot[JOIN_PICKS], mine = EMPTY; // everything here is wave-uniform except `mine`: lane g keeps the g-th pick
 #pragma unroll
     for (int g = 0; g < JOIN_PICKS; g++) {
-        const uint64_t a = m0 & ~((1ull << g) - 1);
         uint32_t s = 0;
-        if (a) {
-            s = __ffsll((unsigned long long)a) - 1;
-            m0 &= ~(1ull << s);
-            if ((uint32_t)lane == s) ids[base + s] = own | FLAG;
+        bool found = false;
+#pragma unroll
+        for (int k = 0; k < KL; k++) {
+            const uint64_t a = k == 0 ? m0[0] & ~((1ull << g) - 1) : m0[k];
+            if (!found && a) {
+                s = k * WAVE + __ffsll((unsigned long long)a) - 1;
+                m0[k] &= ~(1ull << (s % WAVE));
+                if ((uint32_t)lane == s % WAVE) ids[base + s] = own[k] | FLAG;
+                found = true;
+            }
         }
         slot[g] = s;
         bool dup = false;
 #pragma unroll
         for (int t = 0; t < g; t++) dup |= slot[t] == s;
-        uint32_t v = (uint32_t)__builtin_amdgcn_readlane((int)own, s) & ~FLAG;
+        uint32_t v = 0;
+#pragma unroll
+        for (int k = 0; k < KL; k++)
+            if (s / WAVE == (uint32_t)k) v = (uint32_t)__builtin_amdgcn_readlane((int)own[k], s % WAVE) & ~FLAG;
         if (dup || v >= n) v = EMPTY;
         if (lane == g) mine = v;
     }
@@ -90,14 +100,14 @@ __global__ __launch_bounds__(256) void join_pick_kernel(uint32_t n, uint32_t* id
     }
 }
 
-__global__ __launch_bounds__(256) void join_tile_count_kernel(uint32_t n, const uint32_t* pick_cnt, uint32_t* tile_cnt) {
+__global__ __launch_bounds__(256) void join_tile_count_kernel(uint32_t n, uint32_t halves, const uint32_t* pick_cnt, uint32_t* tile_cnt) {
     const uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
-    if (v < n) tile_cnt[v] = (pick_cnt[v] + JT_ROWS - 1) / JT_ROWS;
+    if (v < n) tile_cnt[v] = (pick_cnt[v] + JT_ROWS - 1) / JT_ROWS * halves;
     if (v == n) tile_cnt[v] = 0;
 }
 
 // The pickers of every v side by side, and the node of every tile.
-__global__ __launch_bounds__(256) void join_fill_kernel(uint32_t n, const uint32_t* picks, const uint32_t* pick_off, const uint32_t* tile_off,
+__global__ __launch_bounds__(256) void join_fill_kernel(uint32_t n, uint32_t halves, const uint32_t* picks, const uint32_t* pick_off, const uint32_t* tile_off,
                                                         uint32_t* pick_fill, uint32_t* pick_src, uint32_t* tile_v) {
     const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (uint64_t)n * JOIN_PICKS) return;
@@ -105,7 +115,8 @@ __global__ __launch_bounds__(256) void join_fill_kernel(uint32_t n, const uint32
     if (v == EMPTY) return;
     const uint32_t k = atomicAdd(&pick_fill[v], 1u);
     pick_src[pick_off[v] + k] = (uint32_t)(t / JOIN_PICKS);
-    if (k % JT_ROWS == 0) tile_v[tile_off[v] + k / JT_ROWS] = v;
+    if (k % JT_ROWS == 0)
+        for (uint32_t h = 0; h < halves; h++) tile_v[tile_off[v] + k / JT_ROWS * halves + h] = v;
 }
 
 struct JoinArgs {
@@ -123,10 +134,12 @@ struct JoinArgs {
 
 struct JoinLds {
     uint32_t G, tab, row_list, rowptr, rownnz, row_id, col_id, row_worst, col_worst, seen, scan, ctl, total;
-    __host__ __device__ JoinLds(uint32_t index_bits, uint32_t slot_cap, bool narrow) {
+    // KK = 64: the picker rows' own lists have an array of their own; KK = 128: they are loaded when the products are done and
+    // sit behind the rank table, inside the region that staged the dense rows before
+    __host__ __device__ JoinLds(uint32_t index_bits, uint32_t slot_cap, bool narrow, uint32_t KK = 64) {
         uint32_t o = 0;
         G = o; o += JT_ROWS * JT_STRIDE * 4;
-        row_list = o; o += JT_ROWS * JOIN_K * 4;
+        row_list = o; o += KK == 64 ? JT_ROWS * 64 * 4 : 0;
         o = (o + 7) & ~7u;
         rowptr = o; o += (JT_ROWS + JT_COLS) * 8;
         rownnz = o; o += (JT_ROWS + JT_COLS) * 4;
@@ -139,7 +152,9 @@ struct JoinLds {
         ctl = o; o += 8 * 4;
         o = (o + 15) & ~15u;
         // the rank table of the sparse part; before it is built, the same bytes hold the dense parts of the picker rows
-        const uint32_t table = RankTabLds(index_bits, slot_cap, narrow).total, rows = (uint32_t)(JT_ROWS * DENSE_BYTES);
+        uint32_t table = (RankTabLds(index_bits, slot_cap, narrow).total + 15) & ~15u;
+        const uint32_t rows = (uint32_t)(JT_ROWS * DENSE_BYTES);
+        if (KK != 64) { row_list = o + table; table += JT_ROWS * KK * 4; }
         tab = o; o += table > rows ? table : rows;
         total = o;
     }
@@ -320,11 +335,34 @@ __device__ __forceinline__ void tile_hybrid_ips(const CorpusView& C, float dense
     }
 }
 
-template <bool NARROW>
+// 128 values, two per lane (element e = a of lane e for e < 64, b of lane e - 64 beyond), in ascending order of e.
+__device__ __forceinline__ void wave_sort_u32x2(uint32_t& a, uint32_t& b, int lane) {
+#pragma unroll
+    for (int k = 2; k <= 2 * WAVE; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            if (j == WAVE) { // partners sit in the same lane; k = 128: ascending everywhere
+                const uint32_t lo = min(a, b), hi = max(a, b);
+                a = lo;
+                b = hi;
+            } else {
+                const uint32_t oa = __shfl_xor(a, j, WAVE), ob = __shfl_xor(b, j, WAVE);
+                const bool lower = (lane & j) == 0;
+                const bool up_a = k >= WAVE ? true : (lane & k) == 0;              // element e = lane: bit 6 clear
+                const bool up_b = k == 2 * WAVE ? true : k == WAVE ? false : (lane & k) == 0; // element e = 64 + lane: bit 6 set
+                a = (lower == up_a) ? min(a, oa) : max(a, oa);
+                b = (lower == up_b) ? min(b, ob) : max(b, ob);
+            }
+        }
+    }
+}
+
+template <bool NARROW, uint32_t KK>
 __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void join_tile_kernel(JoinArgs a) {
+    constexpr uint32_t HALVES = KK / 64; // tiles per block of picker rows
     a.C.narrow = NARROW ? 1u : 0u;
     extern __shared__ __align__(16) char smem[];
-    const JoinLds L(a.index_bits, a.slot_cap, NARROW);
+    const JoinLds L(a.index_bits, a.slot_cap, NARROW, KK);
     const RankTab T = ranktab_at(smem + L.tab, a.index_bits, a.slot_cap, a.span, NARROW);
     float* G = reinterpret_cast<float*>(smem + L.G);
     uint32_t* row_list = reinterpret_cast<uint32_t*>(smem + L.row_list);
@@ -352,43 +390,79 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
         if (tile >= n_tiles) break;
         const uint32_t v = uniform(a.tile_v[tile]);
         const uint32_t p0 = uniform(a.pick_off[v]), cnt = uniform(a.pick_off[v + 1]) - p0;
-        const uint32_t r0 = (tile - uniform(a.tile_off[v])) * JT_ROWS;
+        const uint32_t local = tile - uniform(a.tile_off[v]);
+        const uint32_t r0 = local / HALVES * JT_ROWS, half = local % HALVES;
         const uint32_t R = min((uint32_t)JT_ROWS, cnt - r0);
 
         // rows: pickers of v; columns: N(v) and R(v) without repeats
         if (tid < JT_ROWS) {
             const uint32_t u = (uint32_t)tid < R ? a.pick_src[p0 + r0 + tid] : EMPTY;
             row_id[tid] = u;
-            row_worst[tid] = u != EMPTY ? a.dist[(size_t)u * JOIN_K + JOIN_K - 1] : -INF_DIS;
+            row_worst[tid] = u != EMPTY ? a.dist[(size_t)u * KK + KK - 1] : -INF_DIS;
         }
-        if (tid < 2 * (int)JOIN_K) {
-            uint32_t c;
-            if (tid < (int)JOIN_K) c = a.ids[(size_t)v * JOIN_K + tid] & ~FLAG;
-            else c = (uint32_t)a.rev[(size_t)v * JOIN_K + (tid - JOIN_K)];
-            if (c < a.n && id_set_insert(seen, JT_SEEN - 1, c)) col_id[atomicAdd(const_cast<uint32_t*>(&ctl[1]), 1u)] = c;
+        if (HALVES == 1) {
+            if (tid < 2 * (int)KK) {
+                uint32_t c;
+                if (tid < (int)KK) c = a.ids[(size_t)v * KK + tid] & ~FLAG;
+                else c = (uint32_t)a.rev[(size_t)v * KK + (tid - KK)];
+                if (c < a.n && id_set_insert(seen, JT_SEEN - 1, c)) col_id[atomicAdd(const_cast<uint32_t*>(&ctl[1]), 1u)] = c;
+            }
+        } else {
+            // first tile: the list of v without repeats; second tile: what the reverse list adds to it
+            uint32_t c = EMPTY, rc = EMPTY;
+            if (tid < (int)KK) {
+                c = a.ids[(size_t)v * KK + tid] & ~FLAG;
+                if (half == 1) rc = (uint32_t)a.rev[(size_t)v * KK + tid];
+                const bool fresh = c < a.n && id_set_insert(seen, JT_SEEN - 1, c);
+                if (fresh && half == 0) col_id[atomicAdd(const_cast<uint32_t*>(&ctl[1]), 1u)] = c;
+            }
+            if (half == 1) {
+                __syncthreads();
+                if (rc < a.n && id_set_insert(seen, JT_SEEN - 1, rc)) col_id[atomicAdd(const_cast<uint32_t*>(&ctl[1]), 1u)] = rc;
+            }
         }
         __syncthreads();
         const uint32_t M = uniform(ctl[1]);
         if (M == 0) continue;
         // the rows' own lists (who is already a neighbour), the columns' thresholds, where every row's pairs are
-        {   // each row's list in ascending id order (the proposals look an id up by binary search): wave w reads and sorts rows w, w + 8, ...
+        // each row's list in ascending id order (the proposals look an id up by binary search): wave w reads and sorts rows w, w + 8, ...
+        if (KK == 64) {
             uint32_t mine[JT_ROWS / NW];
 #pragma unroll
             for (int k = 0; k < JT_ROWS / NW; k++) {
                 const uint32_t r = wave + k * NW;
-                mine[k] = r < R ? a.ids[(size_t)row_id[r] * JOIN_K + lane] & ~FLAG : 0u;
+                mine[k] = r < R ? a.ids[(size_t)row_id[r] * KK + lane] & ~FLAG : 0u;
             }
 #pragma unroll
             for (int k = 0; k < JT_ROWS / NW; k++) {
                 const uint32_t r = wave + k * NW;
-                if (r < R) row_list[r * JOIN_K + lane] = wave_sort_u32(mine[k], lane);
+                if (r < R) row_list[r * KK + lane] = wave_sort_u32(mine[k], lane);
             }
         }
-        if ((uint32_t)tid < M) col_worst[tid] = a.symmetric ? a.dist[(size_t)col_id[tid] * JOIN_K + JOIN_K - 1] : -INF_DIS;
+        if ((uint32_t)tid < M) col_worst[tid] = a.symmetric ? a.dist[(size_t)col_id[tid] * KK + KK - 1] : -INF_DIS;
         gram_rows_gather(a.C, row_id, R, rowptr, rownnz, tid, JT_THREADS);
         gram_rows_gather(a.C, col_id, M, rowptr + JT_ROWS, rownnz + JT_ROWS, tid, JT_THREADS);
         __syncthreads();
         tile_hybrid_ips<NARROW>(a.C, a.dense_mul, smem + L.tab, T, a.index_bits, a.slot_cap, G, rowptr, rownnz, scan, R, M, a.work + 3, tid, wave, lane);
+        if (KK == 128) { // the rows' own lists, behind the table (the bytes staged dense rows until now: all waves are past that)
+            uint32_t lo[JT_ROWS / NW], hi[JT_ROWS / NW];
+#pragma unroll
+            for (int k = 0; k < JT_ROWS / NW; k++) {
+                const uint32_t r = wave + k * NW;
+                lo[k] = r < R ? a.ids[(size_t)row_id[r] * KK + lane] & ~FLAG : 0u;
+                hi[k] = r < R ? a.ids[(size_t)row_id[r] * KK + WAVE + lane] & ~FLAG : 0u;
+            }
+#pragma unroll
+            for (int k = 0; k < JT_ROWS / NW; k++) {
+                const uint32_t r = wave + k * NW;
+                if (r < R) {
+                    wave_sort_u32x2(lo[k], hi[k], lane);
+                    row_list[r * KK + lane] = lo[k];
+                    row_list[r * KK + WAVE + lane] = hi[k];
+                }
+            }
+            __syncthreads();
+        }
         // proposals
         for (uint32_t p = tid; p < R * M; p += JT_THREADS) {
             const uint32_t r = p / M, c = p % M;
@@ -396,13 +470,13 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
             if (uid == cid) continue;
             const float d = 1.0f - G[r * JT_STRIDE + c];
             if (d < row_worst[r]) {
-                const uint32_t* lst = row_list + r * JOIN_K;
-                uint32_t lo = 0, len = JOIN_K;
+                const uint32_t* lst = row_list + r * KK;
+                uint32_t lo = 0, len = KK;
                 while (len > 0) {
                     const uint32_t half = len >> 1;
                     if (lst[lo + half] < cid) { lo += half + 1; len -= half + 1; } else len = half;
                 }
-                if (lo >= JOIN_K || lst[lo] != cid) atomicMin(&a.prop[(size_t)uid * a.P + prop_slot(cid, a.P)], dist_id_key(d, cid));
+                if (lo >= KK || lst[lo] != cid) atomicMin(&a.prop[(size_t)uid * a.P + prop_slot(cid, a.P)], dist_id_key(d, cid));
             }
             if (d < col_worst[c]) atomicMin(&a.prop[(size_t)cid * a.P + prop_slot(uid, a.P)], dist_id_key(d, uid));
         }
@@ -418,76 +492,96 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
     }
 }
 
-// One wave per node: its proposals (JOIN_PL slots per lane) merged into its list; the entries that are new in the list register
-// with their nodes' reverse lists (index.cu:362-372 registers every entry of a changed list and starts the reverse lists again with
-// every step; the join keeps them over the steps, so an entry registers once, when it enters). Proposal slots are left empty.
+// One wave per node: its proposals (2 * KK slots, PL per lane) merged into its list (KL entries per lane: entry e in register
+// e / 64 of lane e % 64); the entries that are new in the list register with their nodes' reverse lists (index.cu:362-372
+// registers every entry of a changed list and starts the reverse lists again with every step; the join keeps them over the
+// steps, so an entry registers once, when it enters). Proposal slots are left empty.
+template <uint32_t KK>
 __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* ids, float* dist, unsigned long long* prop, unsigned long long* rev,
                                                          uint32_t* rev_cnt, unsigned long long* inserted) {
+    constexpr int KL = KK / WAVE, PL = 2 * KL;
+    constexpr uint32_t P = 2 * KK;
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const uint32_t u = blockIdx.x * 4 + wave;
     if (u >= n) return;
-    const size_t base = (size_t)u * JOIN_K, pbase = (size_t)u * JOIN_P;
-    unsigned long long key[JOIN_PL];
+    const size_t base = (size_t)u * KK, pbase = (size_t)u * P;
+    unsigned long long key[PL];
     bool some = false;
 #pragma unroll
-    for (int s = 0; s < JOIN_PL; s++) {
+    for (int s = 0; s < PL; s++) {
         key[s] = prop[pbase + s * WAVE + lane];
         some |= key[s] != ~0ull;
     }
     if (__ballot(some) == 0) return;
 #pragma unroll
-    for (int s = 0; s < JOIN_PL; s++) prop[pbase + s * WAVE + lane] = ~0ull;
-    const uint32_t own_id = ids[base + lane];
-    const float own_d = dist[base + lane];
-    // a proposal counts if it names another node that is not in the list yet (one id always hashes to one slot: no repeats among them)
-    bool valid[JOIN_PL];
-    float d[JOIN_PL];
+    for (int s = 0; s < PL; s++) prop[pbase + s * WAVE + lane] = ~0ull;
+    uint32_t own_id[KL];
+    float own_d[KL];
 #pragma unroll
-    for (int s = 0; s < JOIN_PL; s++) {
+    for (int k = 0; k < KL; k++) {
+        own_id[k] = ids[base + k * WAVE + lane];
+        own_d[k] = dist[base + k * WAVE + lane];
+    }
+    // a proposal counts if it names another node that is not in the list yet (one id always hashes to one slot: no repeats among them)
+    bool valid[PL];
+    float d[PL];
+#pragma unroll
+    for (int s = 0; s < PL; s++) {
         const uint32_t c = (uint32_t)key[s];
         valid[s] = key[s] != ~0ull && c != u && c < n;
         d[s] = join_key_dist(key[s]);
     }
-    for (uint32_t i = 0; i < JOIN_K; i++) {
-        const uint32_t x = (uint32_t)__builtin_amdgcn_readlane((int)own_id, i) & ~FLAG;
 #pragma unroll
-        for (int s = 0; s < JOIN_PL; s++) valid[s] = valid[s] && x != (uint32_t)key[s];
+    for (int k = 0; k < KL; k++) {
+        for (uint32_t i = 0; i < WAVE; i++) {
+            const uint32_t x = (uint32_t)__builtin_amdgcn_readlane((int)own_id[k], i) & ~FLAG;
+#pragma unroll
+            for (int s = 0; s < PL; s++) valid[s] = valid[s] && x != (uint32_t)key[s];
+        }
     }
-    uint64_t nb[JOIN_PL], any = 0;
+    uint64_t nb[PL], any = 0;
 #pragma unroll
-    for (int s = 0; s < JOIN_PL; s++) { nb[s] = __ballot(valid[s]); any |= nb[s]; }
+    for (int s = 0; s < PL; s++) { nb[s] = __ballot(valid[s]); any |= nb[s]; }
     if (any == 0) return;
     // new: rank among the new ones by (distance, id), plus the old entries strictly closer (new first on ties)
-    uint32_t rank_new[JOIN_PL], le_old = 0;
+    uint32_t rank_new[PL], le_old[KL];
 #pragma unroll
-    for (int s = 0; s < JOIN_PL; s++) rank_new[s] = 0;
+    for (int s = 0; s < PL; s++) rank_new[s] = 0;
 #pragma unroll
-    for (int t = 0; t < JOIN_PL; t++) {
+    for (int k = 0; k < KL; k++) le_old[k] = 0;
+#pragma unroll
+    for (int t = 0; t < PL; t++) {
         for (uint64_t rest = nb[t]; rest; rest &= rest - 1) {
             const unsigned long long ki = readlane64(key[t], (uint32_t)__builtin_ctzll(rest));
 #pragma unroll
-            for (int s = 0; s < JOIN_PL; s++) rank_new[s] += ki < key[s];
-            le_old += join_key_dist(ki) <= own_d; // old entry: new ones at or below its distance go first
+            for (int s = 0; s < PL; s++) rank_new[s] += ki < key[s];
+#pragma unroll
+            for (int k = 0; k < KL; k++) le_old[k] += join_key_dist(ki) <= own_d[k]; // old entry: new ones at or below its distance go first
         }
     }
-    for (uint32_t i = 0; i < JOIN_K; i++) {
-        const float di = readlane_f32(own_d, i);
 #pragma unroll
-        for (int s = 0; s < JOIN_PL; s++) rank_new[s] += di < d[s];
+    for (int k = 0; k < KL; k++) {
+        for (uint32_t i = 0; i < WAVE; i++) {
+            const float di = readlane_f32(own_d[k], i);
+#pragma unroll
+            for (int s = 0; s < PL; s++) rank_new[s] += di < d[s];
+        }
     }
-    const uint32_t rank_old = (uint32_t)lane + le_old;
-    const bool old_in = rank_old < JOIN_K;
-    bool new_in[JOIN_PL];
+    bool new_in[PL];
     uint32_t n_ins = 0;
 #pragma unroll
-    for (int s = 0; s < JOIN_PL; s++) {
-        new_in[s] = valid[s] && rank_new[s] < JOIN_K;
+    for (int s = 0; s < PL; s++) {
+        new_in[s] = valid[s] && rank_new[s] < KK;
         n_ins += __popcll(__ballot(new_in[s]));
     }
     if (n_ins == 0) return;
-    if (old_in) { ids[base + rank_old] = own_id; dist[base + rank_old] = own_d; }
 #pragma unroll
-    for (int s = 0; s < JOIN_PL; s++) {
+    for (int k = 0; k < KL; k++) {
+        const uint32_t rank_old = (uint32_t)(k * WAVE + lane) + le_old[k];
+        if (rank_old < KK) { ids[base + rank_old] = own_id[k]; dist[base + rank_old] = own_d[k]; }
+    }
+#pragma unroll
+    for (int s = 0; s < PL; s++) {
         if (new_in[s]) { ids[base + rank_new[s]] = (uint32_t)key[s]; dist[base + rank_new[s]] = d[s]; }
     }
     if (lane == 0) atomicAdd(inserted + (blockIdx.x % JOIN_COUNT_PARTS) * 8, (unsigned long long)n_ins); // one address for every node would serialise a million atomics
@@ -499,10 +593,10 @@ __global__ __launch_bounds__(256) void join_apply_kernel(uint32_t n, uint32_t* i
         const unsigned long long k = dist_id_key(dv, u);
         // every registration is a minimum (the lists start at ~0 and the join never starts them again): a store into a slot
         // that a later registration of the same step has already reached through its wrap-around could undo that one
-        atomicMin(rev + (size_t)v * JOIN_K + (slot % JOIN_K), k);
+        atomicMin(rev + (size_t)v * KK + (slot % KK), k);
     };
 #pragma unroll
-    for (int s = 0; s < JOIN_PL; s++) {
+    for (int s = 0; s < PL; s++) {
         if (new_in[s]) reg((uint32_t)key[s], d[s]);
     }
 }
@@ -616,13 +710,14 @@ int join_alloc(apoe_knn* g) {
     APOE_TRY(g->pick_src.alloc(n * JOIN_PICKS));
     APOE_TRY(g->tile_cnt.alloc(n + 1));
     APOE_TRY(g->tile_off.alloc(n + 1));
-    APOE_TRY(g->tile_v.alloc(n + n * JOIN_PICKS / JT_ROWS + 1));
-    APOE_TRY(g->prop.alloc(n * JOIN_P));
+    const size_t halves = g->K / 64, P = 2 * (size_t)g->K;
+    APOE_TRY(g->tile_v.alloc((n + n * JOIN_PICKS / JT_ROWS + 1) * halves));
+    APOE_TRY(g->prop.alloc(n * P));
     APOE_TRY(g->join_work.alloc(JOIN_COUNT_AT + JOIN_COUNT_PARTS * 8));
     size_t temp_bytes = 0;
     APOE_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, temp_bytes, g->pick_cnt.p, g->pick_off.p, (int)(n + 1), g->ctx->stream));
     APOE_TRY(g->scan_tmp.alloc(temp_bytes));
-    fill_u64_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->prop.p, (uint64_t)n * JOIN_P, ~0ull);
+    fill_u64_kernel<<<1024, 256, 0, g->ctx->stream>>>(g->prop.p, (uint64_t)n * P, ~0ull);
     APOE_HIP(hipGetLastError());
     return APOE_OK;
 }
@@ -631,34 +726,37 @@ int launch_nnd_join_iterate(apoe_knn* g) {
     apoe_ctx* ctx = g->ctx;
     hipStream_t st = ctx->stream;
     const uint32_t n = g->n;
-    APOE_REQUIRE(g->K == JOIN_K, "the local-join step is built for K = %u lists, this handle has K = %u", JOIN_K, g->K);
+    APOE_REQUIRE(g->K == 64 || g->K == 128, "the local-join step is built for K = 64 and K = 128 lists, this handle has K = %u", g->K);
+    const bool k128 = g->K == 128;
+    const uint32_t halves = g->K / 64;
     if (!g->prop.p) APOE_TRY(join_alloc(g));
     uint32_t index_bits, slot_cap, span;
     join_table_shape(g->corpus, &index_bits, &slot_cap, &span);
-    const JoinLds L(index_bits, slot_cap, g->corpus->narrow);
+    const JoinLds L(index_bits, slot_cap, g->corpus->narrow, g->K);
     APOE_REQUIRE(L.total <= ctx->lds_per_block, "the local-join tile needs %u bytes of LDS, a workgroup may have %zu", L.total, ctx->lds_per_block);
 
     APOE_HIP(hipMemsetAsync(g->counter.p, 0, sizeof(unsigned long long), st)); // [0] inserted; [2], [3] accumulate over the build
     fill_u32_kernel2<<<1024, 256, 0, st>>>(g->pick_cnt.p, (uint64_t)n + 1, 0u);
     fill_u32_kernel2<<<1024, 256, 0, st>>>(g->pick_fill.p, (uint64_t)n + 1, 0u);
     fill_u64_kernel<<<8, 256, 0, st>>>(g->join_work.p, JOIN_COUNT_AT + JOIN_COUNT_PARTS * 8, 0ull);
-    join_pick_kernel<<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->picks.p, g->pick_cnt.p);
+    if (k128) join_pick_kernel<128><<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->picks.p, g->pick_cnt.p);
+    else join_pick_kernel<64><<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->picks.p, g->pick_cnt.p);
     APOE_HIP(hipGetLastError());
-    join_tile_count_kernel<<<(n + 256) / 256, 256, 0, st>>>(n, g->pick_cnt.p, g->tile_cnt.p);
+    join_tile_count_kernel<<<(n + 256) / 256, 256, 0, st>>>(n, halves, g->pick_cnt.p, g->tile_cnt.p);
     APOE_HIP(hipGetLastError());
     size_t temp_bytes = g->scan_tmp.n;
     APOE_HIP(hipcub::DeviceScan::ExclusiveSum(g->scan_tmp.p, temp_bytes, g->pick_cnt.p, g->pick_off.p, (int)(n + 1), st));
     temp_bytes = g->scan_tmp.n;
     APOE_HIP(hipcub::DeviceScan::ExclusiveSum(g->scan_tmp.p, temp_bytes, g->tile_cnt.p, g->tile_off.p, (int)(n + 1), st));
     const uint64_t total = (uint64_t)n * JOIN_PICKS;
-    join_fill_kernel<<<(uint32_t)((total + 255) / 256), 256, 0, st>>>(n, g->picks.p, g->pick_off.p, g->tile_off.p, g->pick_fill.p, g->pick_src.p, g->tile_v.p);
+    join_fill_kernel<<<(uint32_t)((total + 255) / 256), 256, 0, st>>>(n, halves, g->picks.p, g->pick_off.p, g->tile_off.p, g->pick_fill.p, g->pick_src.p, g->tile_v.p);
     APOE_HIP(hipGetLastError());
 
     JoinArgs a{};
     a.C = g->corpus->view();
     a.dense_mul = g->dense_scale * g->dense_scale;
     a.n = n;
-    a.P = JOIN_P;
+    a.P = 2 * g->K;
     a.symmetric = g->join_symmetric ? 1u : 0u;
     a.ids = g->ids.p;
     a.dist = g->dist.p;
@@ -672,14 +770,16 @@ int launch_nnd_join_iterate(apoe_knn* g) {
     a.index_bits = index_bits;
     a.slot_cap = slot_cap;
     a.span = span;
-    auto kernel = g->corpus->narrow ? &join_tile_kernel<true> : &join_tile_kernel<false>;
+    auto kernel = k128 ? (g->corpus->narrow ? &join_tile_kernel<true, 128> : &join_tile_kernel<false, 128>)
+                       : (g->corpus->narrow ? &join_tile_kernel<true, 64> : &join_tile_kernel<false, 64>);
     APOE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total));
     int per_cu = 1;
     APOE_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), JT_THREADS, L.total));
     if (per_cu < 1) per_cu = 1;
     kernel<<<(uint32_t)per_cu * (uint32_t)ctx->num_cus, JT_THREADS, L.total, st>>>(a);
     APOE_HIP(hipGetLastError());
-    join_apply_kernel<<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->dist.p, g->prop.p, g->rev.p, g->rev_cnt.p, g->join_work.p + JOIN_COUNT_AT);
+    if (k128) join_apply_kernel<128><<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->dist.p, g->prop.p, g->rev.p, g->rev_cnt.p, g->join_work.p + JOIN_COUNT_AT);
+    else join_apply_kernel<64><<<(n + 3) / 4, 256, 0, st>>>(n, g->ids.p, g->dist.p, g->prop.p, g->rev.p, g->rev_cnt.p, g->join_work.p + JOIN_COUNT_AT);
     APOE_HIP(hipGetLastError());
     join_account_kernel<<<1, 1, 0, st>>>(g->join_work.p, g->counter.p);
     APOE_HIP(hipGetLastError());

@@ -513,7 +513,6 @@ int apoe_knn_use_half_rows(apoe_knn* g, int on) {
 int apoe_knn_set_join(apoe_knn* g, int mode) {
     APOE_REQUIRE(g, "null argument");
     APOE_REQUIRE(mode >= 0 && mode <= 2, "join mode must be 0 (expansion step), 1 (local join) or 2 (local join, both endpoints), got %d", mode);
-    APOE_REQUIRE(mode == 0 || g->K == 64, "the local-join step is built for K = 64 lists, this handle has K = %u", g->K);
     APOE_REQUIRE(mode == 0 || g->corpus->max_nnz_s + g->corpus->max_nnz_b <= APOE_JOIN_MAX_ROW_TERMS,
                  "the local-join step holds documents of up to %d sparse terms in its table, this corpus has rows of up to %u + %u: use the expansion step (mode 0)",
                  APOE_JOIN_MAX_ROW_TERMS, g->corpus->max_nnz_s, g->corpus->max_nnz_b);

@@ -161,3 +161,63 @@ def test_join_refuses_rows_longer_than_its_table(gpu_ctx):
         knn.set_join(1)
     knn.close()
     gc.close()
+
+
+def test_wide_corpus_with_a_row_of_two_thousand_terms_builds(gpu_ctx, tmp_path, capfd):
+    """Term ids past 65535 (the wide pair format hashes a row's terms into the join tile's table) and one document of about
+    2000 terms: the join chosen by hand either runs or ends with a call-sequence error that names the expansion step, never
+    with lists that lack a sparse part; build_index with its default step builds the index either way."""
+    import apoe
+    import apoe_synth as S
+    import hybrid_search
+    import oracle as O
+    n = 300
+    dense, s_off, s_idx, s_val, b_off, b_idx, b_val = S.to_numpy(S.corpus(n, seed=64, device="cpu"))
+    rng = np.random.default_rng(10)
+    cnt = np.diff(s_off.astype(np.int64))
+    row, terms = 23, 1400
+    keep = np.repeat(np.arange(n) != row, cnt)
+    new_i = np.sort(rng.choice(3_000_000, terms, replace=False)).astype(np.uint32) + np.uint32(70000)
+    new_v = rng.uniform(0.5, 2.0, terms).astype(np.float32)
+    at = int(s_off[row])
+    s_idx = np.concatenate([s_idx[keep][:at], new_i, s_idx[keep][at:]])
+    s_val = np.concatenate([s_val[keep][:at], new_v, s_val[keep][at:]])
+    cnt[row] = terms
+    s_off = np.zeros(n + 1, np.uint32)
+    s_off[1:] = np.cumsum(cnt)
+    bcnt = np.diff(b_off.astype(np.int64))
+    bkeep = np.repeat(np.arange(n) != row, bcnt)
+    nb_i = np.sort(rng.choice(3_000_000, 600, replace=False)).astype(np.uint32) + np.uint32(70000)
+    bat = int(b_off[row])
+    b_idx = np.concatenate([b_idx[bkeep][:bat], nb_i, b_idx[bkeep][bat:]])
+    b_val = np.concatenate([b_val[bkeep][:bat], rng.uniform(0.5, 8.0, 600).astype(np.float32), b_val[bkeep][bat:]])
+    bcnt[row] = 600
+    b_off = np.zeros(n + 1, np.uint32)
+    b_off[1:] = np.cumsum(bcnt)
+    corpus = (dense, s_off, s_idx, s_val, b_off, b_idx, b_val)
+    gc = apoe.Corpus(gpu_ctx, *corpus)
+    assert gc.pair_bytes() == 8 and 1024 < gc.info()[2] + gc.info()[3] <= 2304
+    C = O.HybridSet(*corpus)
+    knn = apoe.Knn(gpu_ctx, gc, 64, 7.0)
+    knn.set_join(1)
+    knn.init(3)
+    try:
+        for it in range(3):
+            knn.iterate(last=(it == 2))
+        ids, dist = knn.download()
+        real = dist < apoe.INF_DIS
+        a = np.repeat(np.arange(n, dtype=np.uint32), 64).reshape(-1, 64)[real]
+        assert_dist_close(dist[real], O.distance_pairs(C, 7.0, a, ids[real]), "stored distance of the join on the wide corpus")
+    except apoe.ApoeError as e:
+        assert "status -3" in str(e) and "expansion step" in str(e)
+    knn.close()
+    gc.close()
+    p = {k: str(tmp_path / k) for k in ("dense.fvecs", "sparse.bin", "bm25.bin", "index.poe")}
+    O.write_fvecs(p["dense.fvecs"], dense)
+    O.write_csr(p["sparse.bin"], s_off, s_idx, s_val)
+    O.write_csr(p["bm25.bin"], b_off, b_idx, b_val)
+    hybrid_search.build_index(dense_data_path=p["dense.fvecs"], sparse_data_path=p["sparse.bin"], bm25_data_path=p["bm25.bin"],
+                              output_graph_path=p["index.poe"], nnd_iters=4)
+    rows, entry = O.read_poe(p["index.poe"])
+    assert rows.shape == (n, 40) and rows[:, :32].max() < n
+    assert "Indexing time" in capfd.readouterr().out
