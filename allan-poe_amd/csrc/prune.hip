@@ -242,14 +242,17 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
 // ---- the prune on a Gram matrix that the tile kernel of join.hip has left in memory (lists of up to 128 entries) ----
 
 constexpr uint32_t PS_MAX = 128;            // longest list
-constexpr uint32_t PS_STRIDE = PS_MAX + 1;  // odd stride: a column read does not collide on the LDS banks
 constexpr int PS_THREADS = 256;
+// The LDS copy of the Gram matrix keeps the upper triangle only, row after row: entry (i, j), i <= j, at tri(i) + j.
+__device__ __forceinline__ uint32_t ps_tri(uint32_t i) { return i * PS_MAX - i * (i + 1) / 2; }
+constexpr uint32_t PS_TRI = PS_MAX * (PS_MAX + 1) / 2;
 
 struct SelectLds {
-    uint32_t G, idmap, umap, R, nb_id, nb_dist, nrm, det, order, o_fwd, o_det, o_kw, ctl, total;
+    uint32_t G, F, idmap, umap, R, nb_id, nb_dist, nrm, det, order, o_fwd, o_det, o_kw, ctl, total;
     __host__ __device__ SelectLds(uint32_t umap_slots, uint32_t map_slots, uint32_t words) {
         uint32_t o = 0;
-        G = o; o += PS_MAX * PS_STRIDE * 4;
+        G = o; o += PS_TRI * 4;
+        F = o; o += PS_MAX * (PS_MAX / 32) * 4; // keyword-flag matrix: bit s of row c = "s holds a term of u that c lacks"
         o = (o + 7) & ~7u;
         idmap = o; o += map_slots * 8;
         umap = o; o += umap_slots * 8;
@@ -279,6 +282,7 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
     extern __shared__ __align__(16) char smem[];
     const SelectLds L(umap_slots, map_slots, words);
     float* G = reinterpret_cast<float*>(smem + L.G);
+    uint32_t* F = reinterpret_cast<uint32_t*>(smem + L.F);
     uint2* idmap = reinterpret_cast<uint2*>(smem + L.idmap);
     uint2* umap = reinterpret_cast<uint2*>(smem + L.umap);
     uint32_t* R = reinterpret_cast<uint32_t*>(smem + L.R);
@@ -302,6 +306,7 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
     for (uint32_t i = tid; i < umap_slots; i += PS_THREADS) umap[i] = make_uint2(EMPTY, 0u);
     for (uint32_t i = tid; i < PS_MAX * words; i += PS_THREADS) R[i] = 0;
     for (uint32_t i = tid; i < PS_MAX; i += PS_THREADS) det[i] = 0;
+    for (uint32_t i = tid; i < PS_MAX * (PS_MAX / 32); i += PS_THREADS) F[i] = 0;
     if (tid < 16) ctl[tid] = 0;
     __syncthreads();
     // valid list entries, in list order (the rows and columns of the Gram matrix)
@@ -342,7 +347,7 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
     // the Gram matrix: rows of the upper triangle, as the tiles wrote them
     for (uint32_t t = tid; t < m * PS_MAX; t += PS_THREADS) {
         const uint32_t i = t / PS_MAX, j = t % PS_MAX;
-        if (j >= i && j < m) G[i * PS_STRIDE + j] = gu[(size_t)i * PS_MAX + j];
+        if (j >= i && j < m) G[ps_tri(i) + j] = gu[(size_t)i * PS_MAX + j];
     }
     // (a) detour counts
     for (uint32_t i = tid; i < m; i += PS_THREADS) {
@@ -372,20 +377,35 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
         }
     }
     __syncthreads();
-    for (uint32_t t = tid; t < m * K; t += PS_THREADS) {
-        const uint32_t r = t / K, j = t % K;
-        const size_t at = (size_t)nb_id[r] * K + j;
-        const uint32_t x = ids[at] & ~FLAG;
-        const float dx = dist[at];
-        uint32_t h = term_hash(x, mmask);
-        while (true) {
-            const uint2 e = idmap[h];
-            if (e.x == x) {
-                if (e.y > r && dx < nb_dist[e.y]) atomicAdd(&det[e.y], 1u);
-                break;
+    // sixteen list entries of this thread are requested before the first of them is looked up
+    for (uint32_t t0 = 0; t0 < m * K; t0 += 16 * PS_THREADS) {
+        uint32_t xs[16];
+        float dxs[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const uint32_t t = t0 + tid + k * PS_THREADS;
+            xs[k] = EMPTY;
+            dxs[k] = 0.f;
+            if (t < m * K) {
+                const size_t at = (size_t)nb_id[t / K] * K + t % K;
+                xs[k] = ids[at] & ~FLAG;
+                dxs[k] = dist[at];
             }
-            if (e.x == EMPTY) break;
-            h = (h + 1) & mmask;
+        }
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const uint32_t r = (t0 + tid + k * PS_THREADS) / K, x = xs[k];
+            if (x == EMPTY) continue;
+            uint32_t h = term_hash(x, mmask);
+            while (true) {
+                const uint2 e = idmap[h];
+                if (e.x == x) {
+                    if (e.y > r && dxs[k] < nb_dist[e.y]) atomicAdd(&det[e.y], 1u);
+                    break;
+                }
+                if (e.x == EMPTY) break;
+                h = (h + 1) & mmask;
+            }
         }
     }
     __syncthreads();
@@ -396,8 +416,16 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
         for (uint32_t j = 0; j < m; j++) r += ((det[j] << 16) | j) < key;
         order[r] = i;
     }
+    // keyword flags of all pairs at once (index.cu:637,651-654): flag(c, s) = (R[s] & ~R[c]) != 0
+    for (uint32_t p = tid; p < m * m; p += PS_THREADS) {
+        const uint32_t c = p / m, sidx = p % m;
+        bool flag = false;
+        for (uint32_t w = 0; w < words; w++) flag |= (R[sidx * words + w] & ~R[c * words + w]) != 0;
+        if (flag) atomicOr(&F[c * (PS_MAX / 32) + (sidx >> 5)], 1u << (sidx & 31));
+    }
     __syncthreads();
-    // (c)+(d) sequential selection, wave 0: member k of the selection order lives in slot k / 64 of lane k % 64
+    // (c)+(d) sequential selection, wave 0: member k of the selection order lives in slot k / 64 of lane k % 64; what a step
+    // needs of its candidate (Gram index, norm, flag row) is read one step ahead
     if (wave == 0) {
         uint32_t gi[2] = {0, 0}, kw[2] = {0, 0}; // Gram index (position in the list) and keyword flag of the member
         bool live[2] = {false, false};
@@ -408,21 +436,29 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
             if (lane == 0) { gi[0] = c0; live[0] = true; mn[0] = nrm[c0]; }
             n_sel = 1;
         }
+        uint32_t c_next = m > 1 ? order[1] : 0u;
+        float norm_next = nrm[c_next];
+        uint4 f_next = *reinterpret_cast<const uint4*>(&F[c_next * (PS_MAX / 32)]);
         for (uint32_t t = 1; t < m; t++) {
-            const uint32_t c = order[t];
-            const float norm_c = nrm[c];
+            const uint32_t c = c_next;
+            const float norm_c = norm_next;
+            const uint4 fc = f_next;
+            if (t + 1 < m) {
+                c_next = order[t + 1];
+                norm_next = nrm[c_next];
+                f_next = *reinterpret_cast<const uint4*>(&F[c_next * (PS_MAX / 32)]);
+            }
             bool rej = false, noflag = false;
 #pragma unroll
             for (int s = 0; s < 2; s++) {
                 const bool act = (uint32_t)lane + 64u * s < n_sel && live[s];
                 if (act) {
                     const uint32_t lo = min(c, gi[s]), hi = max(c, gi[s]);
-                    const float p = G[lo * PS_STRIDE + hi];
-                    bool flag = false;
-                    for (uint32_t w = 0; w < words; w++) flag |= (R[gi[s] * words + w] & ~R[c * words + w]) != 0;
+                    const float p = G[ps_tri(lo) + hi];
+                    const uint32_t q = gi[s] >> 5, fw = q == 0 ? fc.x : q == 1 ? fc.y : q == 2 ? fc.z : fc.w;
                     rej |= norm_c < p;
                     if (mn[s] < p) live[s] = false;
-                    noflag |= !flag;
+                    noflag |= !((fw >> (gi[s] & 31)) & 1u);
                 }
             }
             const bool reject = __ballot(rej) != 0;
