@@ -12,13 +12,6 @@ namespace apoe {
 #ifdef __HIPCC__
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
-#ifdef APOE_PRUNE_TIMING
-__device__ unsigned long long apoe_prune_ticks[16];
-#define GTICK(k) do { if (tid == 0) { const unsigned long long t1_ = wall_clock64(); atomicAdd(&apoe_prune_ticks[k], t1_ - g0_); g0_ = t1_; } } while (0)
-#else
-#define GTICK(k)
-#endif
-
 constexpr int GRAM_ROWS = 64;
 constexpr int GRAM_STRIDE = GRAM_ROWS + 1; // odd stride: column reads do not collide on LDS banks
 
@@ -317,9 +310,6 @@ __device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uin
     const uint32_t bmask = slots / GU_BUCKET - 1;
     const int wave = (int)uniform(tid / WAVE), lane = tid & (WAVE - 1), nwaves = nthreads / WAVE;
     gram_rows_gather(C, ids, m, rowptr, rownnz, tid, nthreads);
-#ifdef APOE_PRUNE_TIMING
-    unsigned long long g0_ = wall_clock64();
-#endif
     __syncthreads();
     uint32_t a0 = 0;
     while (a0 + 1 < m) { // the last row is never a pivot
@@ -369,7 +359,6 @@ __device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uin
             nt = (nt + 1) / 2;
             __syncthreads();
         }
-        GTICK(8);
         const uint32_t novf = uniform(min(ctl2[0], (uint32_t)GU_OVF));
         uint32_t b = a0 + 1 + wave;
         RowPairs cur;
@@ -477,9 +466,7 @@ __device__ __forceinline__ void gram_sparse_union(const CorpusView& C, const uin
             cur = nxt;
             b = bn;
         }
-        GTICK(9);
         __syncthreads();
-        GTICK(10);
         a0 += nt;
     }
     for (uint32_t t = tid; t < m * m; t += nthreads) {

@@ -515,14 +515,7 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
 
 // ---- gather-once form of the prune (K = 64) ----
 
-#ifdef APOE_PRUNE_TIMING
-#define TICK(k) do { if (tid == 0) { const unsigned long long t1_ = wall_clock64(); atomicAdd(&apoe_prune_ticks[k], t1_ - t0_); t0_ = t1_; } } while (0)
-#else
-#define TICK(k)
-#endif
-#ifndef APOE_PRUNE_DENSE_NB
-#define APOE_PRUNE_DENSE_NB 2
-#endif
+constexpr int PRUNE_DENSE_NB = 2; // 8-float blocks of the rows a wave requests ahead of the ones it multiplies
 constexpr int GRAM_THREADS = 512; // 8 waves share one node's tables: more lookups in flight per byte of LDS
 
 struct GramPruneLds {
@@ -574,9 +567,6 @@ __device__ __forceinline__ void gram_sparse_rank(const CorpusView& C, uint32_t m
     uint32_t shape_lanes = 0; // lane k holds own_shape[k]: a wave-uniform pick by index without an indexed array
 #pragma unroll
     for (int k = 0; k < GR_OWN; k++) shape_lanes = lane == k ? own_shape[k] : shape_lanes;
-#ifdef APOE_PRUNE_TIMING
-    unsigned long long g0_ = wall_clock64();
-#endif
     for (uint32_t g = 0; g < ng; g++) {
         // this wave's pivot of the group: own[g], picked with wave-uniform selects so that own[] stays in registers
         RtRow<NARROW> pr = own[0];
@@ -589,7 +579,6 @@ __device__ __forceinline__ void gram_sparse_rank(const CorpusView& C, uint32_t m
         while (lo < 8) {
             const bool mine = (uint32_t)wave >= lo && (uint32_t)wave < lo + cnt && prow < m;
             const uint32_t built = ranktab_build_rows<NARROW>(T, pr, pshape, mine, wave - (int)lo, ptail, scan, tid, nthreads);
-            GTICK(8);
             if (built == EMPTY) {
                 if (cnt == 1) { // one row alone does not fit: the caller falls back
                     if (tid == 0) *fail = 1;
@@ -621,9 +610,7 @@ __device__ __forceinline__ void gram_sparse_rank(const CorpusView& C, uint32_t m
                 __builtin_amdgcn_sched_barrier(0);
             }
             lo += cnt;
-            GTICK(9);
             __syncthreads(); // the table is rebuilt next
-            GTICK(10);
         }
     }
     for (uint32_t t = tid; t < m * m; t += nthreads) {
@@ -680,9 +667,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     for (uint32_t i = tid; i < K; i += NT) det[i] = 0;
     for (uint32_t i = tid; i < K * 2; i += NT) F[i] = 0;
     if (tid < 16) ctl[tid] = 0;
-#ifdef APOE_PRUNE_TIMING
-    unsigned long long t0_ = wall_clock64();
-#endif
     __syncthreads();
 
     if (wave == 0) {
@@ -715,7 +699,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     }
     __syncthreads();
     const uint32_t m = uniform(ctl[PC_M]);
-    TICK(0);
 
     const bool rank = rank_slots != 0; // the sparse part runs on the rank table with the rows held in registers
     if (rank) gram_rows_gather(C, nb_id, m, rowptr, rownnz, tid, NT);
@@ -788,7 +771,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
     }
     __syncthreads();
-    TICK(1);
     // hybrid Gram matrix of the m rows. Only the upper triangle of G is used (the sparse part is added there and the
     // lower triangle is mirrored from it at the end). Every wave takes an eighth of the dimensions and computes the
     // three upper tiles for it from one read of the rows; the partial tiles are added into G in a fixed order
@@ -796,8 +778,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     constexpr int NWAVES = NT / WAVE, BLOCKS = DIM / 8;
     static_assert(NWAVES == 8, "dimensions and rows are dealt out to eight waves");
     floatx16 dacc00, dacc01, dacc11;
-    gram_dense_upper<APOE_PRUNE_DENSE_NB>(C, nb_id, m, lane, wave * (BLOCKS / NWAVES), (wave + 1) * (BLOCKS / NWAVES), dacc00, dacc01, dacc11);
-    TICK(7);
+    gram_dense_upper<PRUNE_DENSE_NB>(C, nb_id, m, lane, wave * (BLOCKS / NWAVES), (wave + 1) * (BLOCKS / NWAVES), dacc00, dacc01, dacc11);
     // this wave's rows w, w + 8, ...: requested as soon as the wave's dense tile is done (its operands need the registers), used from the keyword masks on
     static_assert(NT / WAVE == 8 || NT / WAVE == 4, "rows are dealt out to eight waves");
     RtRow<NARROW> own[GR_OWN];
@@ -905,14 +886,12 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
     }
     __syncthreads();
-    TICK(2);
     if (rank) {
         const RankTab T = ranktab_at(reinterpret_cast<char*>(tabs), rank_bits, rank_slots, rank_span, NARROW);
         gram_sparse_rank<NARROW>(C, m, G, T, ovf_cnt, rowptr, rownnz, own, own_shape, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     } else if (union_slots) gram_sparse_union(C, nb_id, m, G, reinterpret_cast<char*>(tabs), union_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else if (tgroup == 8) gram_sparse_64<8>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else gram_sparse_64<4>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
-    TICK(3);
     // keyword flags of all pairs at once (index.cu:637,651-654): flag(c, s) = (R[s] & ~R[c]) != 0
     for (uint32_t p = tid; p < m * m; p += NT) {
         const uint32_t c = p / m, sidx = p % m;
@@ -921,8 +900,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         if (flag) atomicOr(&F[c * 2 + (sidx >> 5)], 1u << (sidx & 31));
     }
     __syncthreads();
-
-    TICK(4);
     // (c)+(d) sequential selection on the Gram matrix: wave 0, lane i keeps selected member i in registers and the
     // candidate at position i of the order (its Gram row, norm and flag word are handed out with readlane); the Gram
     // entries of step t + 1 are requested before step t is decided (the lane that would hold candidate t as a new
@@ -982,7 +959,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (uint32_t j = cnt + lane; j < d; j += WAVE) { o_fwd[j] = u; o_det[j] = EMPTY; }
         for (uint32_t j = nkw + lane; j < APOE_KW_CAND; j += WAVE) o_kw[1 + j] = 0;
     }
-    TICK(5);
     if (m == 0 && tid == 0) {
         for (uint32_t j = 0; j < d; j++) { o_fwd[j] = u; o_det[j] = EMPTY; }
         for (uint32_t j = 0; j <= APOE_KW_CAND; j++) o_kw[j] = 0;
@@ -997,7 +973,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     if (tid == 0) {
         cnt_out[u] = ctl[PC_CNT];
         if (ctl[PC_FAIL]) atomicOr(gfail, 1ull);
-        TICK(6); // an overflow list was too short: the host redoes the prune with prune_kernel
+        // an overflow list was too short: the host redoes the prune with prune_kernel
     }
 }
 
@@ -1235,14 +1211,6 @@ int launch_final_graph(apoe_knn* g, uint32_t* rows_dev) {
 using namespace apoe;
 
 extern "C" {
-#ifdef APOE_PRUNE_TIMING
-int apoe_debug_prune_ticks(unsigned long long* out16) {
-    hipMemcpyFromSymbol(out16, HIP_SYMBOL(apoe::apoe_prune_ticks), 16 * 8);
-    unsigned long long z[16] = {0};
-    hipMemcpyToSymbol(HIP_SYMBOL(apoe::apoe_prune_ticks), z, 16 * 8);
-    return 0;
-}
-#endif
 
 int apoe_knn_set_prune_form(apoe_knn* g, int form) {
     APOE_REQUIRE(g, "null argument");

@@ -8,18 +8,10 @@
 namespace apoe {
 
 constexpr int MAX_NEW = 64;   // fresh candidates per step: one lane each in wave 0
-// Tuning constants (the defaults are the measured best on MI355X; -D overrides are for measuring others).
-#ifndef APOE_EVAL_BATCH
-#define APOE_EVAL_BATCH 3
-#endif
-#ifndef APOE_DENSE_BATCH
-#define APOE_DENSE_BATCH 1
-#endif
-#ifndef APOE_SEARCH_WAVES_PER_EU
-#define APOE_SEARCH_WAVES_PER_EU 6 // plain search: 12 queries per CU fit its LDS; the other modes need more LDS per query and stay at 5
-#endif
-constexpr int EVAL_BATCH = APOE_EVAL_BATCH;   // candidates whose sparse parts a wave keeps in flight together
-constexpr int DENSE_BATCH = APOE_DENSE_BATCH; // dense rows a wave keeps in flight together
+// Tuning constants: the measured best on MI355X.
+#define APOE_SEARCH_WAVES_PER_EU 6 // plain search: 12 queries per CU fit its LDS; the other modes need more LDS per query and stay at 5 (a macro: it sits in an attribute)
+constexpr int EVAL_BATCH = 3;  // candidates whose sparse parts a wave keeps in flight together
+constexpr int DENSE_BATCH = 1; // dense rows a wave keeps in flight together
 constexpr int MERGE_ROUNDS = 4; // 64-element rounds of the pool that the merge moves per LDS round trip
 constexpr int RING = 32;      // keyword-filter search: evicted keyword hits kept beside the pool (query.cu:18)
 

@@ -263,6 +263,35 @@ def main():
                                             dense_rows_per_evaluation=sc.dense_rows / max(sc.evaluations, 1)))
             log(f"[bench] calibrated weights {tuple(round(float(x), 2) for x in wc)} cands {ec}: {sc.kernel_ms:.2f} ms, recall {calibrated['sweep'][-1]['recall_at_10']:.4f}")
 
+    # ---- the same corpus built with K = 128 lists and degree 64 (the reference's own layout asks for K >= 2 * degree,
+    # index.cu:702): build seconds and the recall sweep as a second row beside the configured one ----
+    k128 = None
+    if not args.no_sweeps and args.nnd_k == 64:
+        knn2 = apoe.Knn(ctx, gc, 128, 7.0)
+        knn2.set_join(args.join)
+        knn2.init(1)
+        for it in range(args.nnd_iters):
+            knn2.iterate(last=(it == args.nnd_iters - 1))
+        nnd2_ms = knn2.elapsed_ms()
+        knn2.merge_reverse()
+        lists2 = knn2.download()[0]
+        knn2.prune(64)
+        graph2 = knn2.finalize()
+        total2_ms = knn2.elapsed_ms()
+        knn2.close()
+        k128 = dict(nnd_k=128, degree=64, nnd_iters=args.nnd_iters, build_seconds_gpu=total2_ms / 1e3, nnd_seconds_gpu=nnd2_ms / 1e3,
+                    knn_list_recall_at_10=float(np.mean([len(set(lists2[samp_np[i], :10].tolist()) & set(exact[i].tolist())) / 10 for i in range(len(samp_np))])),
+                    cands_sweep=[])
+        del lists2
+        for ec in [int(c) for c in args.cands.split(",")]:
+            apoe.search(ctx, gc, gq, graph2, w3, ec, max_iter=iter_cap(ec))
+            ids_2, _, s2 = apoe.search(ctx, gc, gq, graph2, w3, ec, max_iter=iter_cap(ec))
+            k128["cands_sweep"].append(dict(cands=ec, recall=recall_at_k(ids_2[:nq_truth], truth, 10), ms=s2.kernel_ms, qps=args.queries / (s2.kernel_ms / 1e3),
+                                            gbs=s2.algo_bytes / (s2.kernel_ms / 1e3) / 1e9))
+        log(f"[bench] K = 128, degree 64: build {total2_ms / 1e3:.2f}s GPU time (NN-Descent {nnd2_ms / 1e3:.2f}s), list recall@10 {k128['knn_list_recall_at_10']:.4f}; " +
+            ", ".join(f"cands {x['cands']} recall {x['recall']:.3f} {x['ms']:.1f} ms" for x in k128["cands_sweep"]))
+        graph2.close()
+
     # ---- short batches: the launch shape follows the batch (more waves per query while the whole batch is resident at once) ----
     short_batches = None
     if not args.no_sweeps:
@@ -458,6 +487,7 @@ def main():
             **({"weight_sweep_without_rebuild": weight_sweep} if weight_sweep else {}),
             **({"knowledge_graph_search": kg_search} if kg_search else {}),
             **({"reference_semantics_calibrated_weights": calibrated} if calibrated else {}),
+            **({"same_corpus_k128_degree64": k128} if k128 else {}),
             **({"short_batches": short_batches} if short_batches else {}),
             **({"same_generators_smaller_corpora": smaller} if smaller else {}),
             **({"extras": extras} if extras else {}),
