@@ -323,16 +323,17 @@ class Knn:
             pass
 
 
-def build_graph(ctx, corpus, K=64, iters=25, degree=32, dense_scale=7.0, seed=1, half_rows=False, join=0):
-    """NN-Descent + reverse merge + prune + final assembly; returns (Graph, gpu_ms)."""
+def build_graph(ctx, corpus, K=64, iters=25, degree=32, dense_scale=7.0, seed=1, half_rows=False, join=0, expansion_first=0):
+    """NN-Descent + reverse merge + prune + final assembly; returns (Graph, gpu_ms). With a join mode, the first
+    `expansion_first` steps are expansion steps all the same (on very large corpora one such step gets the lists going)."""
     knn = Knn(ctx, corpus, K, dense_scale)
-    if join:
-        knn.set_join(join)
     if half_rows:
         corpus.make_half_rows()
         knn.use_half_rows()
     knn.init(seed)
     for it in range(iters):
+        if join:
+            knn.set_join(0 if it < expansion_first else join)
         knn.iterate(last=(it == iters - 1))
     knn.merge_reverse()
     knn.prune(degree)

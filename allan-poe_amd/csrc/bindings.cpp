@@ -35,7 +35,8 @@ PYBIND11_MODULE(hybrid_search, m) {
         "build_index",
         [](const std::string& dense_data_path, const std::string& sparse_data_path, const std::string& bm25_data_path,
            const std::string& output_graph_path, unsigned degree, unsigned nnd_k, unsigned nnd_iters, float dense_build_scale, uint64_t seed,
-           int device, const std::string& knn_save_path, const std::string& knn_load_path, bool half_rows, int nnd_join) {
+           int device, const std::string& knn_save_path, const std::string& knn_load_path, bool half_rows, int nnd_join,
+           unsigned nnd_expansion_steps) {
             hs::BuildOptions opt;
             opt.degree = degree;
             opt.nnd_k = nnd_k;
@@ -47,13 +48,14 @@ PYBIND11_MODULE(hybrid_search, m) {
             opt.knn_load_path = knn_load_path;
             opt.half_rows = half_rows;
             opt.nnd_join = nnd_join;
+            opt.nnd_expansion_steps = nnd_expansion_steps;
             py::gil_scoped_release release;
             hs::build_index_impl(dense_data_path, sparse_data_path, bm25_data_path, output_graph_path, opt);
         },
         "Build the hybrid index", py::arg("dense_data_path"), py::arg("sparse_data_path"), py::arg("bm25_data_path"),
         py::arg("output_graph_path"), py::arg("degree") = 32, py::arg("nnd_k") = 64, py::arg("nnd_iters") = 25,
         py::arg("dense_build_scale") = 7.0f, py::arg("seed") = 20251125ull, py::arg("device") = 0, py::arg("knn_save_path") = "",
-        py::arg("knn_load_path") = "", py::arg("half_rows") = false, py::arg("nnd_join") = -1);
+        py::arg("knn_load_path") = "", py::arg("half_rows") = false, py::arg("nnd_join") = -1, py::arg("nnd_expansion_steps") = 0);
 
     m.def(
         "search_index",

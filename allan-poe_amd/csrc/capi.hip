@@ -5,6 +5,7 @@
 #include <cstring>
 #include <memory>
 #include <numeric>
+#include <system_error>
 #include <thread>
 
 #include "apoe_internal.h"
@@ -30,6 +31,16 @@ static bool is_device_ptr(const void* p) {
         return false;
     }
     return attr.type == hipMemoryTypeDevice;
+}
+
+// Device memory of one particular GPU.
+static bool is_device_ptr_of(const void* p, int device) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice && attr.device == device;
 }
 
 constexpr size_t STREAM_CHUNK = 32u << 20;     // bytes per pinned staging buffer
@@ -66,7 +77,12 @@ static int stream_in(apoe_ctx* ctx, char* dst_dev, const char* src_host, size_t 
                 const size_t p0 = (size_t)t * part;
                 if (p0 >= len) break;
                 const size_t pl = std::min(part, len - p0);
-                workers[started++] = std::thread([=]() { std::memcpy(stage + p0, src_host + off + p0, pl); });
+                try {
+                    workers[started] = std::thread([=]() { std::memcpy(stage + p0, src_host + off + p0, pl); });
+                    started++;
+                } catch (const std::system_error&) { // no thread to be had: this part is copied here
+                    std::memcpy(stage + p0, src_host + off + p0, pl);
+                }
             }
             for (int t = 0; t < started; t++) workers[t].join();
         }
@@ -521,7 +537,8 @@ int apoe_search_noalloc(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries*
     APOE_HIP(hipSetDevice(ctx->device));
     APOE_REQUIRE(c->n <= APOE_NOALLOC_MAX_DOCS, "apoe_search_noalloc serves corpora of up to %u documents, this one has %u", (unsigned)APOE_NOALLOC_MAX_DOCS,
                  c->n);
-    APOE_REQUIRE(is_device_ptr(out_ids) && is_device_ptr(out_dist), "apoe_search_noalloc writes its results in place: out_ids and out_dist must be device memory");
+    APOE_REQUIRE(is_device_ptr_of(out_ids, ctx->device) && is_device_ptr_of(out_dist, ctx->device),
+                 "apoe_search_noalloc writes its results in place: out_ids and out_dist must be device memory of GPU %d, the context's", ctx->device);
     return launch_search(ctx, c, q, g, kg, p, out_ids, out_dist, stats, ctx->static_ws);
 }
 

@@ -297,10 +297,13 @@ void build_index_impl(const std::string& dense_data_path, const std::string& spa
         const bool rows_fit = longest <= (wide ? 1024u : (unsigned)APOE_JOIN_MAX_ROW_TERMS);
         int join = opt.nnd_join >= 0 ? opt.nnd_join : (!opt.half_rows && rows_fit ? 1 : 0);
         while (true) {
-            check(apoe_knn_set_join(h.knn, join), "apoe_knn_set_join");
+            check(apoe_knn_set_join(h.knn, join), "apoe_knn_set_join"); // refuses what the handle cannot run before any step does
             check(apoe_nnd_init(h.knn, opt.seed), "apoe_nnd_init");
             int status = APOE_OK;
-            for (unsigned it = 0; it < opt.nnd_iters && status == APOE_OK; it++) status = apoe_nnd_iterate(h.knn, it + 1 == opt.nnd_iters, nullptr);
+            for (unsigned it = 0; it < opt.nnd_iters && status == APOE_OK; it++) {
+                check(apoe_knn_set_join(h.knn, it < opt.nnd_expansion_steps ? 0 : join), "apoe_knn_set_join");
+                status = apoe_nnd_iterate(h.knn, it + 1 == opt.nnd_iters, nullptr);
+            }
             if (status == APOE_ERR_STATE && join != 0 && opt.nnd_join < 0) { // a row did not fit the join's table
                 join = 0;
                 continue;

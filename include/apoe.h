@@ -254,8 +254,9 @@ int apoe_search(apoe_ctx* ctx, const apoe_corpus* c, const apoe_queries* q, cons
 
 /*
  * apoe_search without any allocation. No counterpart in the reference: it is for callers that cannot
- * allocate device memory -- code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc. Same kernels, arguments and results as apoe_search, except that
+ * allocate device memory -- tight serving loops, harnesses that forbid hipMalloc. (It still queries the
+ * device and the kernel's attributes on every call, so it is not meant to be recorded into a HIP graph.)
+ * Same kernels, arguments and results as apoe_search, except that
  *  - out_ids / out_dist must be device memory of the context's GPU (results are written in place);
  *  - the counters, the once-per-query arguments and the visited bitmaps live in one static device array of
  *    APOE_NOALLOC_WS_BYTES that each GPU holds from the first apoe_ctx_create on it until the process

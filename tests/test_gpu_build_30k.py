@@ -36,17 +36,17 @@ def _knn_recall(ids, truth, k):
     return float(np.mean([len(set(ids[i, :k].tolist()) & set(truth[i, :k].tolist())) / k for i in range(len(truth))]))
 
 
-@pytest.mark.parametrize("join", [0, 1, 2])
-def test_build_recall_within_half_a_point_of_the_oracle_build(world30k, join):
+@pytest.mark.parametrize("join,first", [(0, 0), (1, 0), (2, 0), (1, 1)])  # first: leading expansion steps of a join build
+def test_build_recall_within_half_a_point_of_the_oracle_build(world30k, join, first):
     import apoe
     w = world30k
     og = apoe.Graph(w["ctx"], w["o_rows"], w["o_entry"])
     lists, graphs = [], []
     for seed in (5, 6, 7):
         knn = apoe.Knn(w["ctx"], w["gc"], 64, 7.0)
-        knn.set_join(join)
         knn.init(seed)
         for it in range(10):
+            knn.set_join(0 if it < first else join)
             knn.iterate(last=(it == 9))
         knn.merge_reverse()
         lists.append(_knn_recall(knn.download()[0][w["samp"]], w["exact"], 10))
@@ -54,7 +54,7 @@ def test_build_recall_within_half_a_point_of_the_oracle_build(world30k, join):
         graphs.append(knn.finalize())
         knn.close()
     l_o = _knn_recall(w["o_knn"][w["samp"]], w["exact"], 10)
-    print(f"join={join}: K-NN list recall@10 gpu {np.round(lists, 4)} oracle {l_o:.4f}")
+    print(f"join={join} first={first}: K-NN list recall@10 gpu {np.round(lists, 4)} oracle {l_o:.4f}")
     assert np.mean(lists) >= l_o - 0.005
     for cands in (128, 512):
         r_g = []
@@ -63,7 +63,7 @@ def test_build_recall_within_half_a_point_of_the_oracle_build(world30k, join):
             r_g.append(recall_at_k(ids, w["truth"], 10))
         ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], og, (1.0, 1.0, 1.0), cands)
         r_o = recall_at_k(ids, w["truth"], 10)
-        print(f"join={join} cands={cands}: search recall@10 gpu-built {np.round(r_g, 4)} mean {np.mean(r_g):.4f}, oracle-built {r_o:.4f}")
+        print(f"join={join} first={first} cands={cands}: search recall@10 gpu-built {np.round(r_g, 4)} mean {np.mean(r_g):.4f}, oracle-built {r_o:.4f}")
         assert np.mean(r_g) >= r_o - 0.005
     for g in graphs:
         g.close()

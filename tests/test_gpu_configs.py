@@ -180,7 +180,7 @@ def test_config4_8m_docs_degree64(gpu_ctx):
     del corpus
     _free()
     gq = apoe.Queries(gpu_ctx, *queries)
-    graph, ms = apoe.build_graph(gpu_ctx, gc, K=64, iters=10, degree=64, seed=1, join=1)
+    graph, ms = apoe.build_graph(gpu_ctx, gc, K=64, iters=10, degree=64, seed=1, join=1, expansion_first=1)
     print(f"8M docs, degree 64: build {ms / 1e3:.1f} s of GPU time")
     w = dict(ctx=gpu_ctx, gc=gc, gq=gq, graph=graph, queries=queries)
     ids, dist, st = _search_dev(apoe, w, (1.0, 1.0, 1.0), cands)
