@@ -235,6 +235,37 @@ def test_gpu_built_index_recall(gpu_world, join):
     gq.close()
 
 
+@pytest.mark.parametrize("join", [0, 1])
+def test_gpu_built_index_recall_k128(gpu_world, join):
+    """K = 128 lists pruned to degree 64 (the reference's layout wants K >= 2 * degree, index.cu:702): the whole GPU build --
+    expansion step or local join, Gram matrices by tiles, selection -- against the oracle's build, recall@10 within half a
+    point on the mean of two seeds."""
+    import apoe
+    import apoe_synth as S
+    import oracle as O
+    w = gpu_world
+    wide = w["gc"].pair_bytes() == 8
+    q_arrays = S.to_numpy(S.queries(2000, seed=412))
+    if wide:
+        q_arrays = q_arrays[:5] + (q_arrays[5] + np.uint32(70000),) + q_arrays[6:]
+    Q = O.HybridSet(*q_arrays)
+    gq = apoe.Queries(w["ctx"], *q_arrays)
+    truth, _ = O.bruteforce_topk(w["C"], Q, (1.0, 1.0, 1.0), 10)
+    seeds = (5,) if wide else (5, 6)  # the wide format: one seed on each side, 1.5 points
+    g_gpu = [apoe.build_graph(w["ctx"], w["gc"], K=128, iters=6, degree=64, dense_scale=7.0, seed=s, join=join)[0] for s in seeds]
+    g_orc = [apoe.Graph(w["ctx"], *O.build_index(w["C"], dense_scale=7.0, K=128, iters=6, d=64, seed=s)) for s in seeds]
+    for cands in (64, 128):
+        r_g, all_g = _mean_recall(g_gpu, w["ctx"], w["gc"], gq, truth, cands)
+        r_c, all_c = _mean_recall(g_orc, w["ctx"], w["gc"], gq, truth, cands)
+        print(f"K=128 join={join} cands={cands}: recall@10 gpu-built {r_g:.4f} {np.round(all_g, 4)}, oracle-built {r_c:.4f} {np.round(all_c, 4)}")
+        assert r_g >= r_c - (0.015 if wide else 0.005)
+    rows, entry = g_gpu[0].download()
+    assert rows.shape == (w["C"].n, 72) and len(entry) == 64
+    for g in g_gpu + g_orc:
+        g.close()
+    gq.close()
+
+
 def test_prune_gives_the_same_rows_on_every_run(gpu_world):
     """The gather-once prune adds its partial Gram tiles in a fixed order and selects with one wave: the same lists
     give the same rows, detour counts and keyword candidates bit for bit, run after run."""
