@@ -50,9 +50,9 @@ def build_index(apoe, ctx, gc, args, join, keep_lists=False):
     """NN-Descent + reverse merge + prune + final rows; returns (graph, timings dict, K-NN ids or None)."""
     t0 = time.time()
     knn = apoe.Knn(ctx, gc, args.nnd_k, 7.0)
-    knn.set_join(join)
     knn.init(1)
     for it in range(args.nnd_iters):
+        knn.set_join(0 if it < args.nnd_expansion_steps else join)
         knn.iterate(last=(it == args.nnd_iters - 1))
     nnd_ms = knn.elapsed_ms()
     evals, rows = knn.counters()
@@ -77,6 +77,8 @@ def main():
     ap.add_argument("--nnd-iters", type=int, default=10)
     ap.add_argument("--join", type=int, default=1, help="NN-Descent step of the index the searches run on: 0 the reference's expansion step, "
                     "1 the local join around the picked neighbour (same pairs), 2 the join that updates both endpoints")
+    ap.add_argument("--nnd-expansion-steps", type=int, default=0, help="with a join: that many leading steps are expansion steps all the same "
+                    "(one such step pays on corpora of several million documents)")
     ap.add_argument("--cands", type=str, default="64,128,256,512,1024,2048",
                     help="pool sizes of the recall sweep; 64,128,256 are the configured ones, the larger ones look for the recall target")
     ap.add_argument("--truth-queries", type=int, default=1000)
@@ -473,6 +475,7 @@ def main():
             "nnd_step": {0: "expansion (the reference's step)", 1: "local join around the picked neighbour", 2: "local join, both endpoints updated"}[args.join],
             "nnd_k": args.nnd_k,
             "nnd_iters": args.nnd_iters,
+            "nnd_leading_expansion_steps": args.nnd_expansion_steps,
             "nnd_seconds_gpu": bt["nnd_ms"] / 1e3,
             "nnd_pair_evaluations": bt["evaluations"],
             "nnd_rows_read": bt["rows_read"],
