@@ -618,14 +618,13 @@ __global__ __launch_bounds__(256) static void fill_u32_kernel2(uint32_t* p, uint
 
 // ---- hybrid Gram matrices of whole neighbour lists, tile by tile (the prune of lists longer than 64 entries) ----
 //
-// For node u = node0 + q / GT_PER_NODE the valid entries of its list (distance below INF_DIS, a document, not u itself),
-// in list order, are the rows and columns of a Gram matrix of at most 128 x 128. Tile t = q % GT_PER_NODE computes rows
+// For node u = node0 + q the valid entries of its list (distance below INF_DIS, a document, not u itself),
+// in list order, are the rows and columns of a Gram matrix of at most 128 x 128. Tile t computes rows
 // [32 t, 32 t + 32) against the columns [32 t, m): the upper triangle, diagonal blocks whole. The products go to
-// gram[(q / GT_PER_NODE) * 128 * 128 + i * 128 + j] for i <= j (entries below the diagonal of a diagonal block are
+// gram[q * 128 * 128 + i * 128 + j] for i <= j (entries below the diagonal of a diagonal block are
 // written too). Same tile body as the local join: every row of a tile is gathered once, dense part on the matrix cores,
 // sparse part through the rank table.
 constexpr uint32_t GT_MAX = 128;                 // longest list
-constexpr uint32_t GT_PER_NODE = GT_MAX / JT_ROWS; // tiles per node
 struct GramTileArgs {
     CorpusView C;
     float dense_mul;
@@ -653,15 +652,14 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
     volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl); // [0] tile, [1] valid entries
     static_assert(JT_SEEN >= (int)GT_MAX, "the id set's words hold a whole list");
     const int tid = threadIdx.x, wave = (int)uniform(tid / WAVE), lane = lane_id();
-    const uint32_t n_tiles = a.n_nodes * GT_PER_NODE;
     const uint64_t lane_lt = (1ull << lane) - 1;
-    while (true) {
+    while (true) { // a workgroup takes a node and runs its tiles one after the other: the columns of a tile are the rows and columns of the next
         __syncthreads();
         if (tid == 0) ctl[0] = (uint32_t)atomicAdd(a.work, 1ull);
         __syncthreads();
-        const uint32_t q = uniform(ctl[0]);
-        if (q >= n_tiles) break;
-        const uint32_t slot = q / GT_PER_NODE, t = q % GT_PER_NODE, u = a.node0 + slot;
+        const uint32_t slot = uniform(ctl[0]);
+        if (slot >= a.n_nodes) break;
+        const uint32_t u = a.node0 + slot;
         if (wave == 0) {
             const size_t base = (size_t)u * a.K;
             uint32_t m = 0;
@@ -676,20 +674,22 @@ __global__ __launch_bounds__(JT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
             if (lane == 0) ctl[1] = m;
         }
         __syncthreads();
-        const uint32_t m = uniform(ctl[1]), r0 = t * JT_ROWS;
-        if (r0 >= m) continue;
-        const uint32_t R = min((uint32_t)JT_ROWS, m - r0), M = m - r0;
-        if ((uint32_t)tid < R) row_id[tid] = valid[r0 + tid];
-        if ((uint32_t)tid < M) col_id[tid] = valid[r0 + tid];
-        __syncthreads();
-        gram_rows_gather(a.C, row_id, R, rowptr, rownnz, tid, JT_THREADS);
-        gram_rows_gather(a.C, col_id, M, rowptr + JT_ROWS, rownnz + JT_ROWS, tid, JT_THREADS);
-        __syncthreads();
-        tile_hybrid_ips<NARROW>(a.C, a.dense_mul, smem + L.tab, T, a.index_bits, a.slot_cap, G, rowptr, rownnz, scan, R, M, a.work + 3, tid, wave, lane);
+        const uint32_t m = uniform(ctl[1]);
         float* out = a.gram + (size_t)slot * GT_MAX * GT_MAX;
-        for (uint32_t p = tid; p < R * M; p += JT_THREADS) {
-            const uint32_t r = p / M, c = p % M;
-            out[(size_t)(r0 + r) * GT_MAX + r0 + c] = G[r * JT_STRIDE + c];
+        for (uint32_t r0 = 0; r0 < m; r0 += JT_ROWS) {
+            const uint32_t R = min((uint32_t)JT_ROWS, m - r0), M = m - r0;
+            if ((uint32_t)tid < R) row_id[tid] = valid[r0 + tid];
+            if ((uint32_t)tid < M) col_id[tid] = valid[r0 + tid];
+            __syncthreads();
+            gram_rows_gather(a.C, row_id, R, rowptr, rownnz, tid, JT_THREADS);
+            gram_rows_gather(a.C, col_id, M, rowptr + JT_ROWS, rownnz + JT_ROWS, tid, JT_THREADS);
+            __syncthreads();
+            tile_hybrid_ips<NARROW>(a.C, a.dense_mul, smem + L.tab, T, a.index_bits, a.slot_cap, G, rowptr, rownnz, scan, R, M, a.work + 3, tid, wave, lane);
+            for (uint32_t p = tid; p < R * M; p += JT_THREADS) {
+                const uint32_t r = p / M, c = p % M;
+                out[(size_t)(r0 + r) * GT_MAX + r0 + c] = G[r * JT_STRIDE + c];
+            }
+            __syncthreads(); // G and the id arrays are rewritten by the next tile
         }
     }
 }
