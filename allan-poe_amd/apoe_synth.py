@@ -38,6 +38,11 @@ _C2 = 0x94D049BB133111EB
 # streams: one per array of a set
 S_DENSE, S_S_COUNT, S_S_TERM, S_S_VAL, S_B_COUNT, S_B_TERM, S_B_VAL = range(1, 8)
 S_KG_DEG, S_KG_E2E, S_KG_DDEG, S_KG_E2D, S_KG_QDEG, S_KG_Q2E = range(16, 22)
+S_L_ROW, S_L_DENSE = range(32, 34)
+
+LATENT_DIM = 16           # latent sets: dimension of the hidden vector behind a dense row
+LATENT_NOISE = 4          # dense row = image of the hidden vector + LATENT_NOISE x own normal vector (in units of the hidden vector's scale)
+LATENT_SCALE = 0.3        # sparse values times this: under 49 x dense + sparse + bm25 the dense part then carries about three quarters
 
 
 def mix64_int(z):
@@ -88,6 +93,9 @@ class _Numpy:
 
     def searchsorted(self, t, u):
         return np.searchsorted(t, u, side="left").astype(np.int64)
+
+    def shr_signed(self, x, s):
+        return x >> s
 
     def repeat_rows(self, counts):
         return np.repeat(np.arange(len(counts), dtype=np.int64), counts)
@@ -179,6 +187,9 @@ class _Torch:
 
     def searchsorted(self, t, u):
         return self.t.searchsorted(t, u, right=False)
+
+    def shr_signed(self, x, s):
+        return x >> s
 
     def repeat_rows(self, counts):
         return self.t.repeat_interleave(self.t.arange(counts.numel(), dtype=self.t.int64, device=self.dev), counts)
@@ -272,11 +283,23 @@ def draws_for_unique(target, vocab=VOCAB):
 
 # ---- samplers ----
 
-def sparse_rows(n, mean_nnz, kind, seed, device="cpu", vocab=VOCAB, chunk=1 << 18, force_backend=None):
+@functools.lru_cache(maxsize=None)
+def rarity_table(mean_nnz, kind, vocab=VOCAB):
+    """Latent sets weight a term by how rare it is, as BM25 and learned sparse encoders do: idf(t) = ln(1 / df(t))
+    with df(t) the share of rows of mean_nnz terms that hold t. BM25-like values are LATENT_SCALE x idf x U[0.3, 1],
+    SPLADE-like values LATENT_SCALE x min(1, idf / 4) x log-normal. The factor in front of the random part, float32."""
+    p, _ = zipf_tables(vocab)
+    df = 1.0 - np.power(1.0 - p, draws_for_unique(mean_nnz, vocab))
+    idf = np.log(1.0 / df)
+    return (LATENT_SCALE * (idf if kind == "bm25" else np.minimum(1.0, idf / 4.0))).astype(np.float32)
+
+
+def sparse_rows(n, mean_nnz, kind, seed, device="cpu", vocab=VOCAB, chunk=1 << 18, force_backend=None, by_rarity=False):
     """CSR with about mean_nnz distinct Zipf terms per row. kind: 'splade' | 'bm25'. Row r draws
     m_r ~ round(N(draws, draws/4)) terms (2 <= m_r < 4096), keeps the distinct ones in ascending order; the value
-    of term t in row r depends on (r, t) only."""
+    of term t in row r depends on (r, t) only. by_rarity: values carry the term's rarity_table() factor."""
     X = backend(device, force_backend)
+    rarity = X.table(rarity_table(mean_nnz, kind, vocab)) if by_rarity else None
     s_count, s_term, s_val = (S_S_COUNT, S_S_TERM, S_S_VAL) if kind == "splade" else (S_B_COUNT, S_B_TERM, S_B_VAL)
     k_count, k_term, k_val = stream_key(seed, s_count), stream_key(seed, s_term), stream_key(seed, s_val)
     _, cdf_h = zipf_tables(vocab)
@@ -301,24 +324,45 @@ def sparse_rows(n, mean_nnz, kind, seed, device="cpu", vocab=VOCAB, chunk=1 << 1
         idx_parts.append(X.i32(kterm))
         hv = X.rnd(k_val, (X.u64(krow) + r0) * 65536 + X.u64(kterm))
         if kind == "splade":
-            val_parts.append(X.take(logn, X.top_bits(hv, LOGN_BITS)))
+            val = X.take(logn, X.top_bits(hv, LOGN_BITS))
+        elif not by_rarity:
+            val = X.f32((X.f64(X.top_bits(hv, 24)) + 0.5) * (7.5 / (1 << 24)) + 0.5)
         else:
-            val_parts.append(X.f32((X.f64(X.top_bits(hv, 24)) + 0.5) * (7.5 / (1 << 24)) + 0.5))
+            val = X.f32((X.f64(X.top_bits(hv, 24)) + 0.5) * (0.7 / (1 << 24)) + 0.3)
+        val_parts.append(val * X.take(rarity, kterm) if by_rarity else val)
     cnt = X.cat(counts, np.int64)
     off = X.i32(X.cumsum0(cnt))
     return X.to_torch(off), X.to_torch(X.cat(idx_parts, np.int32)), X.to_torch(X.cat(val_parts, np.float32))
 
 
-def dense_rows(n, seed, device="cpu", chunk=1 << 14, force_backend=None):
+def hidden_of_rows(X, seed, r0, r1):
+    """The hidden vectors of rows r0..r1-1 of the latent set that `seed` names: [r1 - r0, LATENT_DIM] normal integers
+    with 4 fractional bits (standard deviation 16)."""
+    g = X.take(X.table(gauss_table_fixed()), X.top_bits(X.rnd(stream_key(seed, S_L_ROW), X.arange(r0 * LATENT_DIM, r1 * LATENT_DIM)), GAUSS_BITS))
+    return X.shr_signed(g, 16).reshape(r1 - r0, LATENT_DIM)
+
+
+def dense_rows(n, seed, device="cpu", chunk=1 << 14, force_backend=None, world=None):
     """Rows of 1024 normal values at 2^-20 resolution, L2-normalised: the sum of squares is an exact integer,
-    its square root and the division are float64 operations, the result is rounded to float32 once."""
+    its square root and the division are float64 operations, the result is rounded to float32 once. With `world`
+    (a seed that names a 16 x 1024 normal map shared by every set of that world) a row is the image of its 16 hidden
+    values under the map plus LATENT_NOISE x its own normal vector: two rows have about half the cosine of their
+    hidden vectors."""
     X = backend(device, force_backend)
     key = stream_key(seed, S_DENSE)
     gauss = X.table(gauss_table_fixed())
     out = X.empty_f32(n, DIM)
+    if world is not None:
+        spread = X.take(gauss, X.top_bits(X.rnd(stream_key(world, S_L_DENSE), X.arange(0, LATENT_DIM * DIM)), GAUSS_BITS)).reshape(LATENT_DIM, DIM)
     for r0 in range(0, n, chunk):
         rows = min(chunk, n - r0)
         g = X.take(gauss, X.top_bits(X.rnd(key, X.arange(r0 * DIM, (r0 + rows) * DIM)), GAUSS_BITS)).reshape(rows, DIM)
+        if world is not None:
+            hid = hidden_of_rows(X, seed, r0, r0 + rows)              # 4 fractional bits: LATENT_NOISE counts in sixteenths
+            g = g * (16 * LATENT_NOISE)
+            for k in range(LATENT_DIM):                               # integers: exact, whatever the order
+                g = g + spread[k][None, :] * hid[:, k][:, None]
+            g = X.shr_signed(g, 10)                                   # room for the exact sum of squares
         norm = X.sqrt(X.f64((g * g).sum(1)))
         out[r0:r0 + rows] = X.f32(X.f64(g) / norm[:, None])
     return X.to_torch(out)
@@ -330,6 +374,26 @@ def hybrid_set(n, nnz_splade, nnz_bm25, seed, device="cpu", force_backend=None):
     s = sparse_rows(n, nnz_splade, "splade", seed, device, force_backend=force_backend)
     b = sparse_rows(n, nnz_bm25, "bm25", seed, device, force_backend=force_backend)
     return (dense,) + s + b
+
+
+def latent_set(n, nnz_splade, nnz_bm25, seed, world, device="cpu", force_backend=None):
+    dense = dense_rows(n, seed, device, force_backend=force_backend, world=world)
+    s = sparse_rows(n, nnz_splade, "splade", seed, device, force_backend=force_backend, by_rarity=True)
+    b = sparse_rows(n, nnz_bm25, "bm25", seed, device, force_backend=force_backend, by_rarity=True)
+    return (dense,) + s + b
+
+
+def latent_corpus(n, seed=20251125, world=20251201, device="cpu", force_backend=None):
+    """A hybrid corpus in which a graph has something to find: a hidden 16-dimensional normal vector per row steers
+    its dense vector, so rows have neighbours at every scale, as embedded text has; the terms are drawn as in corpus()
+    (they carry no structure of their own) but valued by rarity and scaled so that the dense part carries about three
+    quarters of a pair's score under 49 x dense + sparse + bm25. Not the distribution of corpus(): it stands next to the
+    structureless one."""
+    return latent_set(n, 120, 60, seed, world, device, force_backend)
+
+
+def latent_queries(n, seed=20251126, world=20251201, device="cpu", force_backend=None):
+    return latent_set(n, 30, 8, seed, world, device, force_backend)
 
 
 def corpus(n, seed=20251125, device="cpu", force_backend=None):

@@ -1,0 +1,58 @@
+"""A corpus whose rows have neighbours (apoe_synth.latent_corpus), 100 000 docs: searched under the metric the graph is
+built for, the path reaches recall@10 >= 0.95 with a pool of 128, the oracle walks the GPU-built graph to the same top-10,
+and the bound on the dense part changes no result although most evaluations now read their dense row."""
+import numpy as np
+import pytest
+
+from parity import assert_topk_match, recall_at_k
+
+pytestmark = pytest.mark.gpu
+
+N_DOCS, N_QUERIES, DEGREE = 100_000, 2_000, 32
+W_BUILD = (49.0, 1.0, 1.0)  # index.cu:836-840: dense x 7 on both sides of a pair
+
+
+@pytest.fixture(scope="module")
+def world(gpu_ctx):
+    import torch
+    import apoe
+    import apoe_synth as S
+    corpus = S.latent_corpus(N_DOCS, seed=501, world=503, device="cuda:0")
+    queries = S.latent_queries(N_QUERIES, seed=502, world=503, device="cuda:0")
+    torch.cuda.synchronize()
+    gc, gq = apoe.Corpus(gpu_ctx, *corpus), apoe.Queries(gpu_ctx, *queries)
+    yield dict(ctx=gpu_ctx, corpus=corpus, queries=queries, gc=gc, gq=gq)
+    gq.close()
+    gc.close()
+
+
+@pytest.mark.parametrize("join", [0, 1])
+def test_recall_target_is_reached_where_rows_have_neighbours(world, join):
+    import apoe
+    import apoe_bruteforce as B
+    import apoe_synth as S
+    import oracle as O
+    w = world
+    graph, _ = apoe.build_graph(w["ctx"], w["gc"], K=64, iters=10, degree=DEGREE, seed=3, join=join)
+    nq = 500
+    truth, _ = B.hybrid_topk(w["corpus"], w["queries"], W_BUILD, 10, nq=nq)
+    rec = {}
+    for cands in (32, 128):
+        ids, dist, st = apoe.search(w["ctx"], w["gc"], w["gq"], graph, W_BUILD, cands, q_count=nq)
+        rec[cands] = recall_at_k(ids, truth, 10)
+    print(f"latent corpus, join={join}: recall@10 {rec}")
+    assert rec[128] >= 0.95 and rec[32] < rec[128]
+    # the bound never changes a result
+    ids2, dist2, st2 = apoe.search(w["ctx"], w["gc"], w["gq"], graph, W_BUILD, 128, q_count=nq, variant=0x100)
+    assert np.array_equal(ids, ids2) and np.array_equal(dist, dist2) and st.dense_rows <= st2.dense_rows == st2.evaluations
+    # the oracle on the same graph
+    rows, entry = graph.download()
+    C = O.HybridSet(*S.to_numpy(w["corpus"]))
+    Q = O.HybridSet(*S.to_numpy(w["queries"])).head(100)
+    oid, odist, _ = O.search(C, Q, rows, entry, W_BUILD, 128)
+    assert assert_topk_match(ids[:100], dist[:100], oid, odist, 10, "latent corpus, GPU-built graph") > 0.97
+    # under the user weights 1/1/1 the terms decide, and they carry no structure: the graph helps little
+    truth1, _ = B.hybrid_topk(w["corpus"], w["queries"], (1.0, 1.0, 1.0), 10, nq=nq)
+    ids1, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], graph, (1.0, 1.0, 1.0), 128, q_count=nq)
+    assert recall_at_k(ids1, truth1, 10) < rec[128]
+    graph.close()

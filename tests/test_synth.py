@@ -68,6 +68,32 @@ def test_distributions():
     assert abs(np.diff(q[1].astype(np.int64)).mean() - 30) < 1 and abs(np.diff(q[4].astype(np.int64)).mean() - 8) < 0.5
 
 
+def test_latent_world_has_the_structure_it_names():
+    n = 3000
+    a = S.latent_corpus(n, seed=41, world=43, force_backend="numpy")
+    _same(a, S.latent_corpus(n, seed=41, world=43, device="cpu", force_backend="torch"))
+    _same(S.latent_queries(300, seed=42, world=43, force_backend="numpy"), S.latent_queries(300, seed=42, world=43, device="cpu", force_backend="torch"))
+    dense, s_off, s_idx, s_val, b_off, b_idx, b_val = S.to_numpy(a)
+    assert np.allclose(np.linalg.norm(dense.astype(np.float64), axis=1), 1.0, atol=1e-6)
+    hid = S.hidden_of_rows(S.backend("cpu", "numpy"), 41, 0, n).astype(np.float64)
+    assert hid.shape == (n, S.LATENT_DIM) and abs(hid.std() - 16.0) < 0.5
+    hn = hid / np.linalg.norm(hid, axis=1)[:, None]
+    iu = np.triu_indices(n, 1)
+    cos_h, cos_d = (hn @ hn.T)[iu], (dense.astype(np.float64) @ dense.astype(np.float64).T)[iu]
+    assert np.corrcoef(cos_h, cos_d)[0, 1] > 0.9                   # the dense row follows the hidden vector ...
+    near = cos_h > 0.8
+    assert near.sum() > 20 and 0.3 < cos_d[near].mean() < 0.6      # ... at about half its cosine: the other half is the row's own noise
+    assert abs(cos_d[np.abs(cos_h) < 0.05].mean()) < 0.01
+    # the terms are those of the structureless corpus of the same seed; their values follow the rarity of the term
+    plain = S.to_numpy(S.corpus(n, seed=41))
+    assert np.array_equal(s_off, plain[1]) and np.array_equal(s_idx, plain[2]) and np.array_equal(b_off, plain[4]) and np.array_equal(b_idx, plain[5])
+    f = S.rarity_table(60, "bm25")
+    assert f[0] < 1e-3 < 0.5 < f[1000] < f[20000] and np.all(b_val <= f[b_idx] * (1 + 1e-6)) and np.all(b_val >= 0.3 * f[b_idx] * (1 - 1e-6))
+    assert np.all(S.rarity_table(120, "splade") <= S.LATENT_SCALE * (1 + 1e-6))
+    # without a world the generator stays the structureless one
+    assert not np.array_equal(S.to_numpy(S.corpus(50, seed=41))[0], dense[:50])
+
+
 def test_knowledge_graph_shape():
     e2e_off, e2e_idx, e2d_off, e2d_idx, q2e_off, q2e_idx = S.to_numpy(S.knowledge_graph(50000, 10000, 2000, seed=8))
     deg = np.diff(e2e_off.astype(np.int64))
@@ -86,3 +112,4 @@ def test_gpu_world_is_the_host_world():
     _same(S.corpus(3000, seed=31), [t.cpu() for t in S.corpus(3000, seed=31, device="cuda:0")])
     _same(S.queries(500, seed=32), [t.cpu() for t in S.queries(500, seed=32, device="cuda:0")])
     _same(S.knowledge_graph(20000, 3000, 500, seed=33), [t.cpu() for t in S.knowledge_graph(20000, 3000, 500, seed=33, device="cuda:0")])
+    _same(S.latent_corpus(2000, seed=34, world=35), [t.cpu() for t in S.latent_corpus(2000, seed=34, world=35, device="cuda:0")])
