@@ -360,13 +360,24 @@ def main():
                                             algo_gbs=sl.algo_bytes / (sl.kernel_ms / 1e3) / 1e9, frac_of_hbm_peak=sl.algo_bytes / (sl.kernel_ms / 1e3) / 1e9 / HBM_PEAK_GBS))
             if rec_l >= 0.95 and structured["cands_at_recall_target"] is None:
                 structured["cands_at_recall_target"], structured["qps_at_recall_target"] = ec, args.queries / (sl.kernel_ms / 1e3)
+        if structured["cands_at_recall_target"]:
+            # the same walk on half-precision copies of the dense rows, the final pool evaluated again in fp32 (variant | 0x200):
+            # here every evaluation reads its dense row, so the narrower row shows
+            gc_l.make_half_rows()
+            hc = structured["cands_at_recall_target"]
+            apoe.search(ctx, gc_l, gq_l, g_l, w_l, hc, max_iter=iter_cap(hc), variant=0x200)
+            ids_h, _, sh = apoe.search(ctx, gc_l, gq_l, g_l, w_l, hc, max_iter=iter_cap(hc), variant=0x200)
+            structured["half_precision_walk"] = dict(cands=hc, recall=recall_at_k(ids_h[:nq_truth], t_l, 10), kernel_ms=sh.kernel_ms,
+                                                     qps=args.queries / (sh.kernel_ms / 1e3), algo_gbs=sh.algo_bytes / (sh.kernel_ms / 1e3) / 1e9)
         for w_o, what in (((1.0, 1.0, 1.0), "1/1/1 as given"), (tuple(float(x) for x in apoe.calibrate_weights(ctx, gc_l, gq_l, (1.0, 1.0, 1.0))), "1/1/1 after the reference's calibration")):
             t_o, _ = B.hybrid_topk(c_l, q_l, w_o, 10, nq=nq_truth)
             ids_o, _, so = apoe.search(ctx, gc_l, gq_l, g_l, w_o, 256)
             structured["other_weights_at_cands_256"].append(dict(weights_dense_sparse_bm25=w_o, what=what, recall=recall_at_k(ids_o[:nq_truth], t_o, 10), kernel_ms=so.kernel_ms))
         log(f"[bench] structured corpus, {args.docs} docs, weights {w_l}: build {ms_l / 1e3:.2f}s, " + ", ".join(f"cands {x['cands']} recall {x['recall']:.3f}" for x in structured["sweep"]) +
             (f" -> {structured['qps_at_recall_target']:.0f} QPS at recall@10 >= 0.95" if structured["qps_at_recall_target"] else " -> target not reached") +
-            "; " + ", ".join(f"{x['what']}: {x['recall']:.3f}" for x in structured["other_weights_at_cands_256"]))
+            "; " + ", ".join(f"{x['what']}: {x['recall']:.3f}" for x in structured["other_weights_at_cands_256"]) +
+            (f"; half-precision walk at cands {structured['half_precision_walk']['cands']}: recall {structured['half_precision_walk']['recall']:.3f}, "
+             f"{structured['half_precision_walk']['qps']:.0f} QPS" if "half_precision_walk" in structured else ""))
         g_l.close()
         gq_l.close()
         gc_l.close()
