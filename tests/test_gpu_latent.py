@@ -56,3 +56,41 @@ def test_recall_target_is_reached_where_rows_have_neighbours(world, join):
     ids1, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], graph, (1.0, 1.0, 1.0), 128, q_count=nq)
     assert recall_at_k(ids1, truth1, 10) < rec[128]
     graph.close()
+
+
+def test_kg_and_keyword_search_match_the_oracle_where_every_evaluation_reads_its_dense_row(world):
+    """Knowledge-graph and keyword-filter search on this corpus (the bound on the dense part rejects nothing here, so
+    every candidate goes through the second stage) against the oracle on the GPU-built graph."""
+    import apoe
+    import apoe_synth as S
+    import oracle as O
+    w = world
+    nq = 100
+    graph, _ = apoe.build_graph(w["ctx"], w["gc"], K=64, iters=10, degree=DEGREE, seed=4, join=1)
+    rows, entry = graph.download()
+    corpus_np, queries_np = S.to_numpy(w["corpus"]), S.to_numpy(w["queries"])
+    C, Q = O.HybridSet(*corpus_np), O.HybridSet(*queries_np).head(nq)
+    kg = S.to_numpy(S.knowledge_graph(20000, N_DOCS, N_QUERIES, seed=22, device="cpu"))
+    gkg = apoe.KnowledgeGraph(w["ctx"], *kg)
+    okg = O.Kg(kg[0], kg[1], kg[2], kg[3], kg[4][:nq + 1], kg[5][:kg[4][nq]])
+    ids, dist, st = apoe.search(w["ctx"], w["gc"], w["gq"], graph, W_BUILD, 128, kg=gkg, kg_weight=40.0, q_count=nq)
+    oid, odist, _ = O.search(C, Q, rows, entry, W_BUILD, 128, kg=okg, kg_weight=40.0)
+    assert assert_topk_match(ids, dist, oid, odist, 10, "latent corpus, knowledge graph") > 0.97
+    assert st.dense_rows > 0.9 * st.evaluations
+    gkg.close()
+    # keyword filter: the rarest BM25 term of each query is required
+    b_off, b_idx = queries_np[4], queries_np[5].copy()
+    df = np.bincount(corpus_np[5], minlength=int(max(corpus_np[5].max(), b_idx.max())) + 1)
+    for q in range(nq):
+        t = b_idx[b_off[q]:b_off[q + 1]]
+        ok = np.where(df[t] > 0)[0] if len(t) else []
+        if len(ok):
+            b_idx[b_off[q] + ok[np.argmin(df[t][ok])]] |= 0x80000000
+    qk = queries_np[:5] + (b_idx,) + queries_np[6:]
+    gqk = apoe.Queries(w["ctx"], *qk)
+    kid, kdist, _ = apoe.search(w["ctx"], w["gc"], gqk, graph, W_BUILD, 128, keyword_filter=True, q_count=nq)
+    okid, okdist, _ = O.search(C, O.HybridSet(*qk).head(nq), rows, entry, W_BUILD, 128, keyword_filter=True)
+    assert (kid == okid).all(axis=1).mean() > 0.97
+    assert (okid != 0x7FFFFFFF).any()
+    gqk.close()
+    graph.close()
