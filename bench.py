@@ -90,6 +90,9 @@ def main():
     ap.add_argument("--extras", action="store_true",
                     help="also time: the keyword-filter search, a four times longer batch, the corpus handed over as host buffers, "
                          "the half-precision walks and build")
+    ap.add_argument("--corpus", choices=("iid", "latent"), default="iid",
+                    help="iid: the configured generators (no document has neighbours); latent: apoe_synth.latent_corpus (dense rows steered by a hidden "
+                         "16-dimensional vector, terms valued by rarity), searched under the build metric 49/1/1")
     ap.add_argument("--calibrate", action="store_true",
                     help="apply the reference's query-time weight calibration to the 1/1/1 weights (off: the metric is literally 1/1/1)")
     ap.add_argument("--copy-calib", action="store_true",
@@ -108,8 +111,11 @@ def main():
         sys.exit("bench.py needs a GPU")
     dev = "cuda:0"
     t0 = time.time()
-    corpus = S.corpus(args.docs, device=dev)
-    queries = S.queries(args.queries, device=dev)
+    latent = args.corpus == "latent"
+    gen_corpus, gen_queries = (S.latent_corpus, S.latent_queries) if latent else (S.corpus, S.queries)
+    user_weights = (49.0, 1.0, 1.0) if latent else (1.0, 1.0, 1.0)
+    corpus = gen_corpus(args.docs, device=dev)
+    queries = gen_queries(args.queries, device=dev)
     torch.cuda.synchronize()
     log(f"[bench] generated {args.docs} docs / {args.queries} queries in {time.time() - t0:.1f}s; "
         f"nnz/doc splade {corpus[2].numel() / args.docs:.1f} bm25 {corpus[5].numel() / args.docs:.1f}")
@@ -157,7 +163,7 @@ def main():
     bt = builds[args.join]
 
     # ---- effective weights and exact ground truth on a query subset ----
-    w3 = apoe.calibrate_weights(ctx, gc, gq, (1.0, 1.0, 1.0)) if args.calibrate else (1.0, 1.0, 1.0)
+    w3 = apoe.calibrate_weights(ctx, gc, gq, (1.0, 1.0, 1.0)) if args.calibrate else user_weights
     nq_truth = min(args.truth_queries, args.queries)
     t0 = time.time()
     truth, _ = B.hybrid_topk(corpus, queries, w3, 10, nq=nq_truth)
@@ -214,7 +220,7 @@ def main():
             full_bytes = stf.algo_bytes
     full_avg = sum(full_ms) / len(full_ms)
     key = (args.docs, args.degree, args.queries, cands, args.variant, args.join)
-    rec_traffic = RECORDED_TRAFFIC.get(key) if not args.calibrate else None
+    rec_traffic = RECORDED_TRAFFIC.get(key) if not args.calibrate and not latent else None
     full_eval = {"kernel_ms": full_avg, "qps": args.queries / (full_avg / 1e3), "achieved": full_bytes / (full_avg / 1e3) / 1e9,
                  "frac": full_bytes / (full_avg / 1e3) / 1e9 / HBM_PEAK_GBS, "algo_bytes_per_launch": full_bytes,
                  "traffic": rec_traffic["every_dense_row_read"] if rec_traffic else None}
@@ -313,16 +319,16 @@ def main():
         for n_small, deg_small in ((4_000, 32), (30_000, 32), (100_000, 32)):
             if n_small >= args.docs:
                 continue
-            c_s = S.corpus(n_small, device=dev)
+            c_s = gen_corpus(n_small, device=dev)
             gc_s = apoe.Corpus(ctx, *c_s)
             g_s, ms_s = apoe.build_graph(ctx, gc_s, K=args.nnd_k, iters=args.nnd_iters, degree=deg_small, seed=1, join=args.join)
-            t_s, _ = B.hybrid_topk(c_s, queries, (1.0, 1.0, 1.0), 10, nq=nq_truth)
+            t_s, _ = B.hybrid_topk(c_s, queries, user_weights, 10, nq=nq_truth)
             row = dict(docs=n_small, degree=deg_small, build_seconds_gpu=ms_s / 1e3, sweep=[], qps_at_recall_target=None, cands_at_recall_target=None)
             for ec in (64, 128, 256, 512, 1024, 2048):
                 if ec >= n_small:
                     break
-                apoe.search(ctx, gc_s, gq, g_s, (1.0, 1.0, 1.0), ec, max_iter=iter_cap(ec))
-                ids_s, _, ss = apoe.search(ctx, gc_s, gq, g_s, (1.0, 1.0, 1.0), ec, max_iter=iter_cap(ec))
+                apoe.search(ctx, gc_s, gq, g_s, user_weights, ec, max_iter=iter_cap(ec))
+                ids_s, _, ss = apoe.search(ctx, gc_s, gq, g_s, user_weights, ec, max_iter=iter_cap(ec))
                 rec_s = recall_at_k(ids_s[:nq_truth], t_s, 10)
                 row["sweep"].append(dict(cands=ec, recall=rec_s, kernel_ms=ss.kernel_ms, qps=args.queries / (ss.kernel_ms / 1e3)))
                 if rec_s >= 0.95 and row["cands_at_recall_target"] is None:
@@ -340,7 +346,7 @@ def main():
     # pair's score), searched under the metric its graph is built for (49 x dense + sparse + bm25, index.cu:836-840); the user
     # weights 1/1/1, raw and through the reference's calibration, beside it ----
     structured = None
-    if not args.no_sweeps:
+    if not args.no_sweeps and not latent:
         c_l = S.latent_corpus(args.docs, device=dev)
         q_l = S.latent_queries(args.queries, device=dev)
         gc_l, gq_l = apoe.Corpus(ctx, *c_l), apoe.Queries(ctx, *q_l)
@@ -514,7 +520,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": f"{args.docs} hybrid docs (dense 1024-d f32 + SPLADE ~120 nnz + BM25 ~60 nnz), degree {args.degree}, "
+            "workload": f"{args.docs} hybrid docs (dense 1024-d f32 + SPLADE ~120 nnz + BM25 ~60 nnz{'; apoe_synth.latent_corpus: dense rows with neighbours, terms valued by rarity' if latent else ''}), degree {args.degree}, "
                         f"{args.queries} queries, weights dense/sparse/bm25 = {tuple(round(x, 3) for x in w3)}"
                         f"{' (1/1/1 after calibration)' if args.calibrate else ''}, top_k 10",
             "cands": cands,
