@@ -27,11 +27,13 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per search launch, RECORDED from FETCH_SIZE + WRITE_SIZE counter runs (rocprofv3 --pmc, scaled by what the
 # counters read for a 1 GiB copy) and not measured by this script: keyed by the workload they were taken on
-# (docs, degree, queries, cands, variant, NN-Descent step) with the profiles/ file that holds the run. Any other
+# (corpus, docs, degree, queries, cands, variant, NN-Descent step) with the profiles/ file that holds the run. Any other
 # workload reports null.
 RECORDED_TRAFFIC = {
-    (1_000_000, 48, 10_000, 256, 0, 1): {"default": 1.876e11, "every_dense_row_read": 5.315e11,
-                                          "source": "profiles/bench_1Mdocs_degree48_cands256.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy)"},
+    ("iid", 1_000_000, 48, 10_000, 256, 0, 1): {"default": 1.876e11, "every_dense_row_read": 5.315e11,
+                                                 "source": "profiles/bench_1Mdocs_degree48_cands256.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy)"},
+    ("latent", 1_000_000, 48, 10_000, 80, 0, 1): {"default": 1.872e11, "every_dense_row_read": 1.872e11,
+                                                  "source": "profiles/bench_1Mdocs_latent_degree48_cands80.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy)"},
 }
 
 
@@ -219,8 +221,8 @@ def main():
             full_ms.append(stf.kernel_ms)
             full_bytes = stf.algo_bytes
     full_avg = sum(full_ms) / len(full_ms)
-    key = (args.docs, args.degree, args.queries, cands, args.variant, args.join)
-    rec_traffic = RECORDED_TRAFFIC.get(key) if not args.calibrate and not latent else None
+    key = (args.corpus, args.docs, args.degree, args.queries, cands, args.variant, args.join)
+    rec_traffic = RECORDED_TRAFFIC.get(key) if not args.calibrate else None
     full_eval = {"kernel_ms": full_avg, "qps": args.queries / (full_avg / 1e3), "achieved": full_bytes / (full_avg / 1e3) / 1e9,
                  "frac": full_bytes / (full_avg / 1e3) / 1e9 / HBM_PEAK_GBS, "algo_bytes_per_launch": full_bytes,
                  "traffic": rec_traffic["every_dense_row_read"] if rec_traffic else None}
