@@ -1,7 +1,8 @@
 """Build parity where list quality starts to drop: 30 000 docs (kNN-list recall of a 10-step build is well below 1
 here). Recall@10 of the search on the GPU-built index (expansion step and local join, mean over three seeds) against
 the index the oracle builds with the reference's algorithm, on 2 000 queries and exact brute force; and the K-NN lists
-of both against exact lists of a node sample."""
+of both against exact lists of a node sample. Twice: on the structureless corpus under the weights 1/1/1, and on the
+corpus whose dense rows have neighbours under the build metric, where recall is high and small pools tell builds apart."""
 import numpy as np
 import pytest
 
@@ -12,22 +13,27 @@ pytestmark = pytest.mark.gpu
 N, NQ = 30_000, 2_000
 
 
-@pytest.fixture(scope="module")
-def world30k(gpu_ctx):
+@pytest.fixture(scope="module", params=["iid", "latent"])
+def world30k(gpu_ctx, request):
     import torch
     import apoe
     import apoe_synth as S
     import apoe_bruteforce as B
     import oracle as O
-    corpus = S.corpus(N, seed=201, device="cuda:0")
-    queries = S.queries(NQ, seed=202, device="cuda:0")
+    if request.param == "iid":
+        corpus, queries = S.corpus(N, seed=201, device="cuda:0"), S.queries(NQ, seed=202, device="cuda:0")
+        w3, pools = (1.0, 1.0, 1.0), (128, 512)
+    else:
+        corpus, queries = S.latent_corpus(N, seed=201, world=203, device="cuda:0"), S.latent_queries(NQ, seed=202, world=203, device="cuda:0")
+        w3, pools = (49.0, 1.0, 1.0), (16, 64)
     gc, gq = apoe.Corpus(gpu_ctx, *corpus), apoe.Queries(gpu_ctx, *queries)
-    truth, _ = B.hybrid_topk(corpus, queries, (1.0, 1.0, 1.0), 10)
+    truth, _ = B.hybrid_topk(corpus, queries, w3, 10)
     samp = torch.arange(0, N, 15, device="cuda:0")
     exact, _ = B.hybrid_topk(corpus, B.rows_as_queries(corpus, samp), (49.0, 1.0, 1.0), 64, self_ids=samp.cpu().numpy())
     C = O.HybridSet(*S.to_numpy(corpus))
     rows, entry, knn_ids, _ = O.build_index(C, dense_scale=7.0, K=64, iters=10, d=32, seed=5, return_knn=True)
-    yield dict(ctx=gpu_ctx, gc=gc, gq=gq, truth=truth, samp=samp.cpu().numpy(), exact=exact, o_rows=rows, o_entry=entry, o_knn=knn_ids)
+    yield dict(ctx=gpu_ctx, gc=gc, gq=gq, truth=truth, samp=samp.cpu().numpy(), exact=exact, o_rows=rows, o_entry=entry, o_knn=knn_ids, w3=w3, pools=pools,
+               kind=request.param)
     gq.close()
     gc.close()
 
@@ -54,16 +60,16 @@ def test_build_recall_within_half_a_point_of_the_oracle_build(world30k, join, fi
         graphs.append(knn.finalize())
         knn.close()
     l_o = _knn_recall(w["o_knn"][w["samp"]], w["exact"], 10)
-    print(f"join={join} first={first}: K-NN list recall@10 gpu {np.round(lists, 4)} oracle {l_o:.4f}")
+    print(f"{w['kind']} join={join} first={first}: K-NN list recall@10 gpu {np.round(lists, 4)} oracle {l_o:.4f}")
     assert np.mean(lists) >= l_o - 0.005
-    for cands in (128, 512):
+    for cands in w["pools"]:
         r_g = []
         for g in graphs:
-            ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], g, (1.0, 1.0, 1.0), cands)
+            ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], g, w["w3"], cands)
             r_g.append(recall_at_k(ids, w["truth"], 10))
-        ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], og, (1.0, 1.0, 1.0), cands)
+        ids, _, _ = apoe.search(w["ctx"], w["gc"], w["gq"], og, w["w3"], cands)
         r_o = recall_at_k(ids, w["truth"], 10)
-        print(f"join={join} first={first} cands={cands}: search recall@10 gpu-built {np.round(r_g, 4)} mean {np.mean(r_g):.4f}, oracle-built {r_o:.4f}")
+        print(f"{w['kind']} join={join} first={first} cands={cands}: search recall@10 gpu-built {np.round(r_g, 4)} mean {np.mean(r_g):.4f}, oracle-built {r_o:.4f}")
         assert np.mean(r_g) >= r_o - 0.005
     for g in graphs:
         g.close()
