@@ -94,3 +94,38 @@ def test_kg_and_keyword_search_match_the_oracle_where_every_evaluation_reads_its
     assert (okid != 0x7FFFFFFF).any()
     gqk.close()
     graph.close()
+
+
+def test_k128_degree64_and_the_wide_pair_format_on_this_corpus(world):
+    """Lists of 128 pruned to degree 64 (the gather-once prune by tiles, the join with two tiles per row block) and the
+    8-byte pair format, where every evaluation reads its dense row: recall, the oracle on the same graph, and the same
+    rows from narrow and wide records."""
+    import torch
+    import apoe
+    import apoe_bruteforce as B
+    import apoe_synth as S
+    import oracle as O
+    w = world
+    nq = 300
+    graph, _ = apoe.build_graph(w["ctx"], w["gc"], K=128, iters=10, degree=64, seed=5, join=1)
+    truth, _ = B.hybrid_topk(w["corpus"], w["queries"], W_BUILD, 10, nq=nq)
+    ids, dist, _ = apoe.search(w["ctx"], w["gc"], w["gq"], graph, W_BUILD, 64, q_count=nq)
+    assert recall_at_k(ids, truth, 10) >= 0.97
+    rows, entry = graph.download()
+    assert rows.shape == (N_DOCS, 64 + 8)
+    C = O.HybridSet(*S.to_numpy(w["corpus"]))
+    Q = O.HybridSet(*S.to_numpy(w["queries"])).head(100)
+    oid, odist, _ = O.search(C, Q, rows, entry, W_BUILD, 64)
+    assert assert_topk_match(ids[:100], dist[:100], oid, odist, 10, "latent corpus, K = 128 / degree 64") > 0.97
+    shift = 70000
+    corpus_w = tuple(w["corpus"][:5]) + (w["corpus"][5] + shift,) + tuple(w["corpus"][6:])
+    queries_w = tuple(w["queries"][:5]) + (w["queries"][5] + shift,) + tuple(w["queries"][6:])
+    torch.cuda.synchronize()
+    gc2, gq2 = apoe.Corpus(w["ctx"], *corpus_w), apoe.Queries(w["ctx"], *queries_w)
+    assert w["gc"].pair_bytes() == 6 and gc2.pair_bytes() == 8
+    ids2, dist2, _ = apoe.search(w["ctx"], gc2, gq2, graph, W_BUILD, 64, q_count=nq)
+    assert np.array_equal(ids, ids2)
+    assert np.allclose(dist, dist2, rtol=1e-5, atol=1e-5)
+    gq2.close()
+    gc2.close()
+    graph.close()
