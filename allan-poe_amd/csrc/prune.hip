@@ -243,17 +243,14 @@ __global__ __launch_bounds__(PR_THREADS) void prune_kernel(CorpusView C, float d
 
 constexpr uint32_t PS_MAX = 128;            // longest list
 constexpr int PS_THREADS = 256;
-// The LDS copy of the Gram matrix keeps the upper triangle only, row after row: entry (i, j), i <= j, at tri(i) + j.
-__device__ __forceinline__ uint32_t ps_tri(uint32_t i) { return i * PS_MAX - i * (i + 1) / 2; }
-constexpr uint32_t PS_TRI = PS_MAX * (PS_MAX + 1) / 2;
 
 struct SelectLds {
-    uint32_t G, F, idmap, umap, R, nb_id, nb_dist, nrm, det, order, o_fwd, o_det, o_kw, ctl, total;
+    uint32_t F, rdesc, idmap, umap, R, nb_id, nb_dist, nrm, det, order, o_fwd, o_det, o_kw, ctl, total;
     __host__ __device__ SelectLds(uint32_t umap_slots, uint32_t map_slots, uint32_t words) {
         uint32_t o = 0;
-        G = o; o += PS_TRI * 4;
         F = o; o += PS_MAX * (PS_MAX / 32) * 4; // keyword-flag matrix: bit s of row c = "s holds a term of u that c lacks"
         o = (o + 7) & ~7u;
+        rdesc = o; o += PS_MAX * 8;             // descriptors of the rows
         idmap = o; o += map_slots * 8;
         umap = o; o += umap_slots * 8;
         R = o; o += PS_MAX * words * 4;
@@ -273,16 +270,18 @@ struct SelectLds {
 // allan_poe (index.cu:539-714) for node u = node0 + blockIdx.x, as prune_kernel, with every inner product <c, s> read from the
 // node's Gram matrix gram[blockIdx.x][i][j] (i <= j: positions in the list of valid entries) instead of being evaluated:
 // detour counts and the (detour, rank) order as there; the keyword flag of a pair from bit masks R[i] = the BM25 terms of u
-// that row i holds (flag(c, s) = R[s] has a bit that R[c] lacks); the sequential selection by wave 0 alone on the LDS copy of
-// the matrix, two selected members per lane (slots `lane` and `lane + 64` of the selection order).
+// that row i holds (flag(c, s) = R[s] has a bit that R[c] lacks); the sequential selection by wave 0 alone, two selected
+// members per lane (slots `lane` and `lane + 64` of the selection order), every member's product with the NEXT candidate
+// requested from the matrix in memory while the current candidate is decided. The workgroup keeps no copy of the matrix:
+// several nodes share a CU, and the others cover the selection's waits.
 __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, const float* __restrict__ norms, uint32_t K, const uint32_t* __restrict__ ids,
                                                                   const float* __restrict__ dist, uint32_t d, uint32_t node0, const float* __restrict__ gram,
                                                                   uint32_t* fwd, uint32_t* det_out, uint32_t* cnt_out, uint32_t* kw_out, uint32_t umap_slots,
                                                                   uint32_t map_slots, uint32_t words) {
     extern __shared__ __align__(16) char smem[];
     const SelectLds L(umap_slots, map_slots, words);
-    float* G = reinterpret_cast<float*>(smem + L.G);
     uint32_t* F = reinterpret_cast<uint32_t*>(smem + L.F);
+    uint64_t* rdesc = reinterpret_cast<uint64_t*>(smem + L.rdesc);
     uint2* idmap = reinterpret_cast<uint2*>(smem + L.idmap);
     uint2* umap = reinterpret_cast<uint2*>(smem + L.umap);
     uint32_t* R = reinterpret_cast<uint32_t*>(smem + L.R);
@@ -297,6 +296,7 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
     volatile uint32_t* ctl = reinterpret_cast<volatile uint32_t*>(smem + L.ctl);
 
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    constexpr uint32_t NWV = PS_THREADS / WAVE;
     const uint32_t u = node0 + blockIdx.x, umask = umap_slots - 1, mmask = map_slots - 1;
     const size_t base = (size_t)u * K;
     const uint64_t lane_lt = (1ull << lane) - 1;
@@ -306,7 +306,6 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
     for (uint32_t i = tid; i < umap_slots; i += PS_THREADS) umap[i] = make_uint2(EMPTY, 0u);
     for (uint32_t i = tid; i < PS_MAX * words; i += PS_THREADS) R[i] = 0;
     for (uint32_t i = tid; i < PS_MAX; i += PS_THREADS) det[i] = 0;
-    for (uint32_t i = tid; i < PS_MAX * (PS_MAX / 32); i += PS_THREADS) F[i] = 0;
     if (tid < 16) ctl[tid] = 0;
     __syncthreads();
     // valid list entries, in list order (the rows and columns of the Gram matrix)
@@ -322,6 +321,7 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
                 nb_id[pos] = v;
                 nb_dist[pos] = dv;
                 nrm[pos] = norms[v];
+                rdesc[pos] = C.desc[v];
             }
             m += __popcll(b);
         }
@@ -344,11 +344,6 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
     }
     __syncthreads();
     const uint32_t m = ctl[PC_M];
-    // the Gram matrix: rows of the upper triangle, as the tiles wrote them
-    for (uint32_t t = tid; t < m * PS_MAX; t += PS_THREADS) {
-        const uint32_t i = t / PS_MAX, j = t % PS_MAX;
-        if (j >= i && j < m) G[ps_tri(i) + j] = gu[(size_t)i * PS_MAX + j];
-    }
     // (a) detour counts
     for (uint32_t i = tid; i < m; i += PS_THREADS) {
         const uint32_t key = nb_id[i];
@@ -360,19 +355,43 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
             h = (h + 1) & mmask;
         }
     }
-    // R[r] = bits of u's BM25 terms that row r holds too: one wave per row, lanes over its BM25 pairs
-    for (uint32_t r = wave; r < m; r += PS_THREADS / WAVE) {
-        const uint64_t dr = C.desc[nb_id[r]];
-        const Pairs sp = record_pairs(C, dr);
-        const uint32_t ns = desc_nnz_s(dr), nb = desc_nnz_b(dr);
-        for (uint32_t j = lane; j < nb; j += WAVE) {
-            const uint32_t key = sp.key(ns + j);
-            uint32_t h = term_hash(key, umask);
-            while (true) {
-                const uint2 e = umap[h];
-                if (e.x == key) { atomicOr(&R[r * words + (e.y >> 5)], 1u << (e.y & 31)); break; }
-                if (e.x == EMPTY) break;
-                h = (h + 1) & umask;
+    // R[r] = bits of u's BM25 terms that row r holds too: one wave per row, lanes over its BM25 pairs; the first 128 BM25 terms
+    // of four rows are requested before the first of them is looked up
+    auto mark = [&](uint32_t r, uint32_t key) {
+        uint32_t h = term_hash(key, umask);
+        while (true) {
+            const uint2 e = umap[h];
+            if (e.x == key) { atomicOr(&R[r * words + (e.y >> 5)], 1u << (e.y & 31)); break; }
+            if (e.x == EMPTY) break;
+            h = (h + 1) & umask;
+        }
+    };
+    for (uint32_t r0 = wave; r0 < m; r0 += 4 * NWV) {
+        uint32_t key[4][2], nbs[4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const uint32_t r = r0 + b * NWV;
+            nbs[b] = 0;
+            key[b][0] = key[b][1] = EMPTY;
+            if (r < m) {
+                const uint64_t dr = rdesc[r];
+                const Pairs sp = record_pairs(C, dr);
+                const uint32_t ns = desc_nnz_s(dr);
+                nbs[b] = desc_nnz_b(dr);
+                if ((uint32_t)lane < nbs[b]) key[b][0] = sp.key(ns + lane);
+                if ((uint32_t)lane + WAVE < nbs[b]) key[b][1] = sp.key(ns + lane + WAVE);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const uint32_t r = r0 + b * NWV;
+            if ((uint32_t)lane < nbs[b]) mark(r, key[b][0]);
+            if ((uint32_t)lane + WAVE < nbs[b]) mark(r, key[b][1]);
+            if (nbs[b] > 2 * WAVE) { // a longer row: the rest as it comes
+                const uint64_t dr = rdesc[r];
+                const Pairs sp = record_pairs(C, dr);
+                const uint32_t ns = desc_nnz_s(dr);
+                for (uint32_t j = 2 * WAVE + lane; j < nbs[b]; j += WAVE) mark(r, sp.key(ns + j));
             }
         }
     }
@@ -416,12 +435,29 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
         for (uint32_t j = 0; j < m; j++) r += ((det[j] << 16) | j) < key;
         order[r] = i;
     }
-    // keyword flags of all pairs at once (index.cu:637,651-654): flag(c, s) = (R[s] & ~R[c]) != 0
-    for (uint32_t p = tid; p < m * m; p += PS_THREADS) {
-        const uint32_t c = p / m, sidx = p % m;
-        bool flag = false;
-        for (uint32_t w = 0; w < words; w++) flag |= (R[sidx * words + w] & ~R[c * words + w]) != 0;
-        if (flag) atomicOr(&F[c * (PS_MAX / 32) + (sidx >> 5)], 1u << (sidx & 31));
+    // keyword flags of all pairs at once (index.cu:637,651-654): flag(c, s) = (R[s] & ~R[c]) != 0. A thread takes one row c and
+    // half of the columns: its own mask stays in registers (the first four words), the lanes of a wave read the same R[s]
+    {
+        static_assert(PS_THREADS == 2 * PS_MAX && PS_MAX == 128, "one row and two flag words per thread");
+        const uint32_t c = tid % PS_MAX, half = tid / PS_MAX;
+        uint32_t rc[4];
+#pragma unroll
+        for (int w = 0; w < 4; w++) rc[w] = (uint32_t)w < words && c < m ? R[c * words + w] : 0u;
+#pragma unroll
+        for (int q2 = 0; q2 < 2; q2++) {
+            const uint32_t q = half * 2 + q2;
+            uint32_t word = 0;
+            for (uint32_t b = 0; b < 32 && q * 32 + b < m; b++) {
+                const uint32_t sidx = q * 32 + b;
+                uint32_t any = 0;
+#pragma unroll
+                for (int w = 0; w < 4; w++)
+                    if ((uint32_t)w < words) any |= R[sidx * words + w] & ~rc[w];
+                for (uint32_t w = 4; w < words; w++) any |= R[sidx * words + w] & ~(c < m ? R[c * words + w] : 0u);
+                word |= (any != 0 ? 1u : 0u) << b;
+            }
+            F[c * (PS_MAX / 32) + q] = c < m ? word : 0u;
+        }
     }
     __syncthreads();
     // (c)+(d) sequential selection, wave 0: member k of the selection order lives in slot k / 64 of lane k % 64; what a step
@@ -439,22 +475,31 @@ __global__ __launch_bounds__(PS_THREADS) void prune_select_kernel(CorpusView C, 
         uint32_t c_next = m > 1 ? order[1] : 0u;
         float norm_next = nrm[c_next];
         uint4 f_next = *reinterpret_cast<const uint4*>(&F[c_next * (PS_MAX / 32)]);
+        auto product = [&](uint32_t a, uint32_t b) { return gu[(size_t)min(a, b) * PS_MAX + max(a, b)]; };
+        float p_next[2] = {0.f, 0.f}; // <member, next candidate>
+        if (m > 1 && lane == 0) p_next[0] = product(gi[0], c_next);
         for (uint32_t t = 1; t < m; t++) {
             const uint32_t c = c_next;
             const float norm_c = norm_next;
             const uint4 fc = f_next;
+            const float p_cur[2] = {p_next[0], p_next[1]};
             if (t + 1 < m) {
                 c_next = order[t + 1];
                 norm_next = nrm[c_next];
                 f_next = *reinterpret_cast<const uint4*>(&F[c_next * (PS_MAX / 32)]);
+#pragma unroll
+                for (int s = 0; s < 2; s++) { // also for the slot that c takes if it is accepted
+                    const uint32_t slot = (uint32_t)lane + 64u * s;
+                    if (slot < n_sel && live[s]) p_next[s] = product(gi[s], c_next);
+                    else if (slot == n_sel) p_next[s] = product(c, c_next);
+                }
             }
             bool rej = false, noflag = false;
 #pragma unroll
             for (int s = 0; s < 2; s++) {
                 const bool act = (uint32_t)lane + 64u * s < n_sel && live[s];
                 if (act) {
-                    const uint32_t lo = min(c, gi[s]), hi = max(c, gi[s]);
-                    const float p = G[ps_tri(lo) + hi];
+                    const float p = p_cur[s];
                     const uint32_t q = gi[s] >> 5, fw = q == 0 ? fc.x : q == 1 ? fc.y : q == 2 ? fc.z : fc.w;
                     rej |= norm_c < p;
                     if (mn[s] < p) live[s] = false;
