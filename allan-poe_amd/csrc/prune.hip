@@ -937,12 +937,23 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     } else if (union_slots) gram_sparse_union(C, nb_id, m, G, reinterpret_cast<char*>(tabs), union_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else if (tgroup == 8) gram_sparse_64<8>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
     else gram_sparse_64<4>(C, nb_id, m, G, tabs, term_slots, ovf_cnt, rowptr, rownnz, (uint32_t*)&ctl[PC_FAIL], tid, NT);
-    // keyword flags of all pairs at once (index.cu:637,651-654): flag(c, s) = (R[s] & ~R[c]) != 0
-    for (uint32_t p = tid; p < m * m; p += NT) {
-        const uint32_t c = p / m, sidx = p % m;
-        bool flag = false;
-        for (uint32_t w = 0; w < words; w++) flag |= (R[sidx * words + w] & ~R[c * words + w]) != 0;
-        if (flag) atomicOr(&F[c * 2 + (sidx >> 5)], 1u << (sidx & 31));
+    // keyword flags of all pairs at once (index.cu:637,651-654): flag(c, s) = (R[s] & ~R[c]) != 0. A thread takes one row c and
+    // one of its two flag words: its own mask stays in registers (the first four words), the lanes of a wave read the same R[s]
+    if (tid < 2 * (int)K) {
+        const uint32_t c = (uint32_t)tid % K, q = (uint32_t)tid / K;
+        uint32_t rc[4], word = 0;
+#pragma unroll
+        for (int w = 0; w < 4; w++) rc[w] = (uint32_t)w < words && c < m ? R[c * words + w] : 0u;
+        for (uint32_t b = 0; b < 32 && q * 32 + b < m; b++) {
+            const uint32_t sidx = q * 32 + b;
+            uint32_t any = 0;
+#pragma unroll
+            for (int w = 0; w < 4; w++)
+                if ((uint32_t)w < words) any |= R[sidx * words + w] & ~rc[w];
+            for (uint32_t w = 4; w < words; w++) any |= R[sidx * words + w] & ~(c < m ? R[c * words + w] : 0u);
+            word |= (any != 0 ? 1u : 0u) << b;
+        }
+        F[c * 2 + q] = c < m ? word : 0u;
     }
     __syncthreads();
     // (c)+(d) sequential selection on the Gram matrix: wave 0, lane i keeps selected member i in registers and the
