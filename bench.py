@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # (corpus, docs, degree, queries, cands, variant, NN-Descent step) with the profiles/ file that holds the run. Any other
 # workload reports null.
 RECORDED_TRAFFIC = {
-    ("iid", 1_000_000, 48, 10_000, 256, 0, 1): {"default": 1.876e11, "every_dense_row_read": 5.313e11,
+    ("iid", 1_000_000, 48, 10_000, 256, 0, 1): {"default": 1.876e11, "every_dense_row_read": 5.312e11,
                                                  "source": "profiles/bench_1Mdocs_degree48_cands256.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy)"},
     ("latent", 1_000_000, 48, 10_000, 80, 0, 1): {"default": 1.872e11, "every_dense_row_read": 1.872e11,
                                                   "source": "profiles/bench_1Mdocs_latent_degree48_cands80.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy)"},
